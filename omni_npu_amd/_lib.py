@@ -1,0 +1,56 @@
+"""ctypes binding of libmla_hip.so.
+
+There is no fallback: if the library is missing or a symbol is absent this module raises, and so
+does every op built on it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmla_hip.so")
+
+P, I32, I64, F32, SZ = c_void_p, c_int32, c_int64, c_float, c_size_t
+
+# name -> (restype, argtypes); mirrors include/mla_hip.h one to one
+SIGNATURES = {
+    "mlahip_version": (c_int32, []),
+    "mlahip_last_error_string": (c_char_p, []),
+    "mla_cache_write_bf16": (c_int32, [P, I64, P, I64, P, I32, P, I64, I64, P, I64, I64, I32, I64, P]),
+    "mla_scatter_rows": (c_int32, [P, I64, I32, P, I32, P, I64, I64, I32, I64, P]),
+    "mla_decode_workspace_bytes": (SZ, [I32, I32, I32, I32]),
+    "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
+                                  I32, I32, F32, P, I64, I64, P, P, SZ, I32, P]),
+}
+
+
+class MlaHipError(RuntimeError):
+    """A C-ABI entry point returned a negative code."""
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(or `make -C omni_npu_amd/csrc`). There is no non-HIP fallback.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError if the symbol is missing
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().mlahip_last_error_string()
+        raise MlaHipError(f"{what} failed with code {rc}: {msg.decode() if msg else ''}")

@@ -1,0 +1,399 @@
+// Absorbed-MLA paged decode for gfx950 (bf16 cache), split-KV, plus the split reduction.
+//
+// Replaces the reference's decode call of npu_fused_infer_attention_score
+// (src/omni_npu/attention/backends/mla.py:781-804): for sequence b, head n, query token t
+//   s_j = scale * (ql[t,n] . Kc[j] + qr[t,n] . Kr[j]),  j < L_b - (q_len-1-t)   (right-down causal)
+//   o   = sum_j softmax(s)_j * Kc[j]
+// with ONE latent KV row (512 + 64) shared by all heads.
+//
+// Work decomposition.  One workgroup = 4 wavefronts = (sequence b, KV split s, group of 128 query
+// rows), a query row being a (query token, head) pair.  Each wavefront owns 32 rows and keeps, in
+// registers, their whole 576-wide query (as the B operand of S^T = K . Q^T, 36 k-steps) and their
+// 512 x 32 fp32 output accumulator O^T (16 MFMA 32x32 blocks).  K tiles of 64 tokens are copied
+// global -> LDS without touching registers, double buffered, the nope part (64 x 1024 B) and the rope
+// part (64 x 128 B) as two swizzled regions.  Per 32 tokens a wavefront issues 36 MFMA 32x32x16 for
+// S^T = K Q^T (A operand = K rows, 16-byte LDS reads), an online-softmax update, and 32 MFMA for
+// O^T += V^T P^T, whose A operand V^T (V = first 512 columns of the same K rows) comes from
+// transposed LDS reads.  Computing the transposed products makes the accumulator layout of S^T the
+// B-operand layout of P^T, so P never leaves registers.
+//
+// Each workgroup writes a normalised fp32 partial and its log-sum-exp; mla_splitkv_reduce_kernel folds the
+// splits with the N-way merge of src/omni_npu/attention/ops.py:109-141 and writes bf16.
+#include "mla_common.hpp"
+
+namespace mlahip {
+
+constexpr int kTile = 64;                          // tokens per LDS tile
+constexpr int kNopeRowB = kDNope * 2;              // 1024
+constexpr int kRopeRowB = kDRope * 2;              // 128
+constexpr int kNopeTileB = kTile * kNopeRowB;      // 65536
+constexpr int kRopeTileB = kTile * kRopeRowB;      // 8192
+constexpr int kBufB = kNopeTileB + kRopeTileB;     // 73728
+constexpr int kDecodeLdsB = 2 * kBufB;             // 147456
+constexpr int kRowsPerWg = 128;
+
+// 16-byte granule swizzles (functions of row % 16).  A nope row has 64 granules, a rope row 8.
+// They spread (i) 16 consecutive rows at one column over 16 distinct 16-byte bank groups for the
+// row-wise reads and (ii) 4 consecutive rows x 64 bytes over distinct bank groups for the transposed
+// reads.
+__device__ __forceinline__ int swz_nope(int r) {
+  int r0 = r & 1, r1 = (r >> 1) & 1, r2 = (r >> 2) & 1, r3 = (r >> 3) & 1;
+  return ((r1 ^ r3) << 3) | (r0 << 2) | (r1 << 1) | r2;
+}
+__device__ __forceinline__ int swz_rope(int r) {
+  int r0 = r & 1, r1 = (r >> 1) & 1, r2 = (r >> 2) & 1, r3 = (r >> 3) & 1;
+  return ((r0 ^ r3) << 2) | (r1 << 1) | r2;
+}
+
+struct DecodeParams {
+  const __bf16* q_nope; int64_t qn_st, qn_sh;
+  const __bf16* q_rope; int64_t qr_st, qr_sh;
+  const __bf16* nope; int64_t nope_sp, nope_sr;
+  const __bf16* rope; int64_t rope_sp, rope_sr;
+  const int32_t* block_table; int64_t bt_stride; int32_t max_blocks;
+  const int32_t* seq_lens;
+  const int32_t* qsl;            // [B+1] or null
+  int32_t batch, max_q_len, num_heads;
+  int64_t num_pages;
+  float scale_log2;              // scale * log2(e)
+  float* o_part;                 // [B*S, R_max, 512]
+  float* lse_part;               // [B*S, R_max]   (natural log)
+  int32_t num_splits;
+};
+
+// Issue the global -> LDS copies of one 64-token tile (18 x 16 B per lane).
+__device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int tile, int L, char* buf, int wave, int lane) {
+  const int tok0 = tile * kTile;
+  int page = tok0 / kPage;
+  page = page < p.max_blocks ? page : p.max_blocks - 1;
+  int64_t blk = p.block_table[(int64_t)b * p.bt_stride + page];
+  blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
+  const int row_in_page0 = tok0 % kPage;
+  const int last = L - 1 - tok0;                   // last valid row of this tile (>= 0)
+  const char* nope_pg = (const char*)(p.nope + blk * p.nope_sp);
+  const char* rope_pg = (const char*)(p.rope + blk * p.rope_sp);
+#pragma unroll
+  for (int i = 0; i < 16; i++) {
+    const int r = wave * 16 + i;
+    const int re = r < last ? r : last;            // rows past the end re-read the last valid row
+    const int c = lane ^ swz_nope(r & 15);
+    const char* g = nope_pg + (int64_t)(row_in_page0 + re) * p.nope_sr * 2 + c * 16;
+    dma16(g, buf + r * kNopeRowB);
+  }
+#pragma unroll
+  for (int j = 0; j < 2; j++) {
+    const int gi = wave * 128 + j * 64 + lane;
+    const int r = gi >> 3;
+    const int re = r < last ? r : last;
+    const int c = (gi & 7) ^ swz_rope(r & 15);
+    const char* g = rope_pg + (int64_t)(row_in_page0 + re) * p.rope_sr * 2 + c * 16;
+    dma16(g, buf + kNopeTileB + (wave * 128 + j * 64) * 16);
+  }
+}
+
+__global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodeParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int h32 = lane & 31;
+  const int half = lane >> 5;
+  const int split = blockIdx.x;
+  const int b = blockIdx.y;
+  const int grp = blockIdx.z;
+
+  const int L = p.seq_lens[b];
+  int q0, qlen;
+  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
+  qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
+  const int rows = qlen * p.num_heads;
+  const int r_max = p.max_q_len * p.num_heads;
+  if (grp * kRowsPerWg >= r_max) return;
+
+  const int row = grp * kRowsPerWg + wave * 32 + h32;        // this lane's query row
+  const bool row_ok = row < rows && L > 0;
+  const int t_local = row / p.num_heads;
+  const int head = row - t_local * p.num_heads;
+  int limit = row_ok ? (L - qlen + t_local + 1) : 0;         // number of visible keys
+  limit = limit < 0 ? 0 : limit;
+
+  const int64_t part_row = ((int64_t)b * p.num_splits + split) * r_max + row;
+
+  // ---- token range of this split (whole tiles) ----
+  const int tiles_total = (L + kTile - 1) / kTile;
+  const int tps = (tiles_total + p.num_splits - 1) / p.num_splits;
+  const int tile_begin = split * tps;
+  int tile_end = tile_begin + tps;
+  tile_end = tile_end < tiles_total ? tile_end : tiles_total;
+
+  if (tile_begin >= tile_end || grp * kRowsPerWg >= rows) {   // empty split / no rows: uniform per workgroup
+    if (row < r_max && half == 0) p.lse_part[part_row] = -INFINITY;
+    return;
+  }
+
+  // ---- prologue: first tile in flight, then the query into registers ----
+  issue_tile(p, b, tile_begin, L, lds, wave, lane);
+
+  bf16x8 qf[36];
+  {
+    const __bf16* qn = p.q_nope + (int64_t)(q0 + t_local) * p.qn_st + (int64_t)head * p.qn_sh + half * 8;
+    const __bf16* qr = p.q_rope + (int64_t)(q0 + t_local) * p.qr_st + (int64_t)head * p.qr_sh + half * 8;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int kk = 0; kk < 32; kk++) qf[kk] = row_ok ? *(const bf16x8*)(qn + kk * 16) : zero;
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) qf[32 + kk] = row_ok ? *(const bf16x8*)(qr + kk * 16) : zero;
+  }
+
+  f32x16 acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+  float m_run = -INFINITY;    // running max (log2 domain), identical in both half-waves
+  float l_run = 0.f;          // running sum of this lane's 16-token slices
+
+  // per-lane LDS offsets
+  const int fk = swz_nope(h32 & 15);
+  const int fr = swz_rope(h32 & 15);
+  const int k_row_off = h32 * kNopeRowB;                      // + tb*32*1024
+  const int r_row_off = kNopeTileB + h32 * kRopeRowB;         // + tb*32*128
+  // transposed V reads: lane (g16 = lane/16, j = lane%16) points at token 4*(g16/2) + j/4 (+8*rd),
+  // columns 16*(g16%2) + 4*(j%4) .. +3 of the 32-wide d block
+  const int g16 = lane >> 4, j16 = lane & 15;
+  const int v_row = 4 * (g16 >> 1) + (j16 >> 2);              // + 8*rd + 16*kb + 32*tb
+  const int v_cl = 2 * (g16 & 1) + ((j16 & 3) >> 1);          // low 2 bits of the granule index
+  const int v_in = (j16 & 1) * 8;
+  const int v_off0 = v_row * kNopeRowB + v_in;                // rd = 0
+  const int v_off1 = (v_row + 8) * kNopeRowB + v_in;          // rd = 1
+  const int v_x0 = v_cl ^ swz_nope(v_row & 15);               // granule xor term, rd = 0
+  const int v_x1 = v_cl ^ swz_nope((v_row + 8) & 15);
+
+  for (int tile = tile_begin; tile < tile_end; tile++) {
+    char* buf = lds + ((tile - tile_begin) & 1) * kBufB;
+    if (tile + 1 < tile_end) {
+      issue_tile(p, b, tile + 1, L, lds + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane);
+      MLA_WAIT_VMCNT(18);
+    } else {
+      MLA_WAIT_VMCNT(0);
+    }
+    __syncthreads();
+
+    const int tok_base = tile * kTile;
+#pragma unroll 1
+    for (int tb = 0; tb < 2; tb++) {
+      if (tok_base + tb * 32 >= L) break;                     // uniform: nothing visible in this block
+      // ---- S^T = K Q^T : 32 tokens x 32 rows ----
+      f32x16 s;
+#pragma unroll
+      for (int r = 0; r < 16; r++) s[r] = 0.f;
+      const char* kb_ptr = buf + tb * 32 * kNopeRowB + k_row_off;
+#pragma unroll
+      for (int kk = 0; kk < 32; kk++) {
+        const int c = (kk * 2 + half) ^ fk;
+        bf16x8 a = *(const bf16x8*)(kb_ptr + c * 16);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
+      }
+      const char* rb_ptr = buf + tb * 32 * kRopeRowB + r_row_off;
+#pragma unroll
+      for (int kk = 0; kk < 4; kk++) {
+        const int c = (kk * 2 + half) ^ fr;
+        bf16x8 a = *(const bf16x8*)(rb_ptr + c * 16);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[32 + kk], s, 0, 0, 0);
+      }
+      // ---- online softmax (log2 domain) ----
+      const int tok_lane0 = tok_base + tb * 32 + 4 * half;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int tok = tok_lane0 + 8 * (r >> 2) + (r & 3);
+        s[r] = tok < limit ? s[r] * p.scale_log2 : -INFINITY;
+        mx = fmaxf(mx, s[r]);
+      }
+      mx = fmaxf(mx, xor32(mx));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        s[r] = fast_exp2(s[r] - m_safe);
+        psum += s[r];
+      }
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][r] *= alpha;
+      }
+      bf16x8 pb[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) pb[kb][e] = (__bf16)s[kb * 8 + e];
+      // ---- O^T += V^T P^T ----
+      const char* vb = buf + tb * 32 * kNopeRowB;
+#pragma unroll
+      for (int db = 0; db < 16; db++) {
+        const int c0 = ((db * 4) ^ v_x0) * 16;
+        const int c1 = ((db * 4) ^ v_x1) * 16;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+          bf16x4 lo = lds_read_tr16(vb + kb * 16 * kNopeRowB + v_off0 + c0);
+          bf16x4 hi = lds_read_tr16(vb + kb * 16 * kNopeRowB + v_off1 + c1);
+          bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[kb], acc[db], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: normalised partial + lse ----
+  const float l_tot = l_run + xor32(l_run);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (row < r_max) {
+    if (half == 0) p.lse_part[part_row] = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
+    float* op = p.o_part + part_row * kDNope + 4 * half;
+#pragma unroll
+    for (int db = 0; db < 16; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        f32x4 v = {acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv, acc[db][rg * 4 + 2] * inv,
+                   acc[db][rg * 4 + 3] * inv};
+        *(f32x4*)(op + db * 32 + rg * 8) = v;
+      }
+  }
+}
+
+// N-way merge over the splits (src/omni_npu/attention/ops.py:109-141): one wavefront per query row.
+struct ReduceParams {
+  const float* o_part; const float* lse_part;
+  const int32_t* qsl;
+  int32_t batch, max_q_len, num_heads, num_splits;
+  __bf16* out; int64_t out_st, out_sh;
+  float* lse_out; int64_t lse_st;      // optional [T, N]
+};
+
+__global__ __launch_bounds__(256) void mla_splitkv_reduce_kernel(const ReduceParams p) {
+  const int lane = threadIdx.x & 63;
+  const int r_max = p.max_q_len * p.num_heads;
+  const int64_t gr = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gr >= (int64_t)p.batch * r_max) return;
+  const int b = gr / r_max;
+  const int row = gr - (int64_t)b * r_max;
+  int q0, qlen;
+  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
+  qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
+  if (row >= qlen * p.num_heads) return;
+  const int t_local = row / p.num_heads;
+  const int head = row - t_local * p.num_heads;
+
+  const int64_t base = ((int64_t)b * p.num_splits) * r_max + row;
+  float m = -INFINITY;
+  for (int s = 0; s < p.num_splits; s++) {
+    float l = p.lse_part[base + (int64_t)s * r_max];
+    l = l == INFINITY ? -INFINITY : l;
+    m = fmaxf(m, l);
+  }
+  float tot = 0.f;
+  f32x4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
+  if (m != -INFINITY) {
+    for (int s = 0; s < p.num_splits; s++) {
+      float l = p.lse_part[base + (int64_t)s * r_max];
+      if (l == INFINITY || l == -INFINITY) continue;         // empty split: its partial is never read
+      const float w = __expf(l - m);
+      tot += w;
+      const float* o = p.o_part + (base + (int64_t)s * r_max) * kDNope;
+      f32x4 v0 = *(const f32x4*)(o + lane * 4);
+      f32x4 v1 = *(const f32x4*)(o + 256 + lane * 4);
+      a0 += v0 * w;
+      a1 += v1 * w;
+    }
+  }
+  const float inv = tot > 0.f ? 1.f / tot : 0.f;
+  __bf16* out = p.out + (int64_t)(q0 + t_local) * p.out_st + (int64_t)head * p.out_sh;
+  bf16x4 o0, o1;
+#pragma unroll
+  for (int e = 0; e < 4; e++) { o0[e] = (__bf16)(a0[e] * inv); o1[e] = (__bf16)(a1[e] * inv); }
+  *(bf16x4*)(out + lane * 4) = o0;
+  *(bf16x4*)(out + 256 + lane * 4) = o1;
+  if (p.lse_out && lane == 0)
+    p.lse_out[(int64_t)(q0 + t_local) * p.lse_st + head] = tot > 0.f ? __logf(tot) + m : -INFINITY;
+}
+
+}  // namespace mlahip
+
+using namespace mlahip;
+
+extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits) {
+  if (batch <= 0 || max_q_len <= 0 || num_heads <= 0 || num_splits <= 0) return 0;
+  const size_t rows = (size_t)batch * num_splits * max_q_len * num_heads;
+  return rows * kDNope * sizeof(float) + rows * sizeof(float);
+}
+
+extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                               int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                               int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                               int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                               const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                               const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                               int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                               int64_t out_stride_h, float* lse_out, void* workspace, size_t workspace_bytes,
+                               int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && block_table && seq_lens && out, MLA_ERR_NULL,
+              "mla_decode_bf16: null pointer argument");
+  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && max_blocks >= 1 && num_pages >= 1,
+              MLA_ERR_SHAPE, "mla_decode_bf16: batch=%d max_q_len=%d num_heads=%d num_splits=%d max_blocks=%d num_pages=%lld",
+              batch, max_q_len, num_heads, num_splits, max_blocks, (long long)num_pages);
+  MLA_REQUIRE(num_splits <= 65535 && batch <= 65535, MLA_ERR_SHAPE, "mla_decode_bf16: grid limits exceeded");
+  MLA_REQUIRE((qn_stride_t % 8 == 0) && (qn_stride_h % 8 == 0) && (qr_stride_t % 8 == 0) && (qr_stride_h % 8 == 0) &&
+                  (nope_row_stride % 8 == 0) && (rope_row_stride % 8 == 0) && (nope_page_stride % 8 == 0) &&
+                  (rope_page_stride % 8 == 0) && (out_stride_t % 4 == 0) && (out_stride_h % 4 == 0),
+              MLA_ERR_SHAPE, "mla_decode_bf16: strides must keep 16-byte alignment of 8-element groups");
+  MLA_REQUIRE(((uintptr_t)q_nope % 16 == 0) && ((uintptr_t)q_rope % 16 == 0) && ((uintptr_t)nope_cache % 16 == 0) &&
+                  ((uintptr_t)rope_cache % 16 == 0) && ((uintptr_t)out % 8 == 0),
+              MLA_ERR_SHAPE, "mla_decode_bf16: pointers must be 16-byte aligned");
+  if (batch == 0) return MLA_OK;
+  const size_t need = mla_decode_workspace_bytes(batch, max_q_len, num_heads, num_splits);
+  MLA_REQUIRE(workspace && workspace_bytes >= need, MLA_ERR_WORKSPACE,
+              "mla_decode_bf16: workspace %zu bytes < required %zu", workspace_bytes, need);
+  MLA_REQUIRE((uintptr_t)workspace % 16 == 0, MLA_ERR_SHAPE, "mla_decode_bf16: workspace must be 16-byte aligned");
+
+  const int r_max = max_q_len * num_heads;
+  const size_t rows = (size_t)batch * num_splits * r_max;
+  DecodeParams p;
+  p.q_nope = (const __bf16*)q_nope; p.qn_st = qn_stride_t; p.qn_sh = qn_stride_h;
+  p.q_rope = (const __bf16*)q_rope; p.qr_st = qr_stride_t; p.qr_sh = qr_stride_h;
+  p.nope = (const __bf16*)nope_cache; p.nope_sp = nope_page_stride; p.nope_sr = nope_row_stride;
+  p.rope = (const __bf16*)rope_cache; p.rope_sp = rope_page_stride; p.rope_sr = rope_row_stride;
+  p.block_table = block_table; p.bt_stride = bt_stride; p.max_blocks = max_blocks;
+  p.seq_lens = seq_lens; p.qsl = query_start_loc;
+  p.batch = batch; p.max_q_len = max_q_len; p.num_heads = num_heads; p.num_pages = num_pages;
+  p.scale_log2 = scale * kLog2e;
+  p.o_part = (float*)workspace;
+  p.lse_part = (float*)workspace + rows * kDNope;
+  p.num_splits = num_splits;
+
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kDecodeLdsB);
+    if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_decode_bf16: cannot reserve %d bytes of LDS: %s", kDecodeLdsB,
+                                     hipGetErrorString(e));
+    attr_set = true;
+  }
+  dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
+  hipLaunchKernelGGL(mla_decode_bf16_kernel, grid, dim3(256), kDecodeLdsB, stream, p);
+  if (int rc = check_launch("mla_decode_bf16_kernel")) return rc;
+
+  ReduceParams rp;
+  rp.o_part = p.o_part; rp.lse_part = p.lse_part; rp.qsl = query_start_loc;
+  rp.batch = batch; rp.max_q_len = max_q_len; rp.num_heads = num_heads; rp.num_splits = num_splits;
+  rp.out = (__bf16*)out; rp.out_st = out_stride_t; rp.out_sh = out_stride_h;
+  rp.lse_out = lse_out; rp.lse_st = num_heads;
+  const int64_t nrows = (int64_t)batch * r_max;
+  hipLaunchKernelGGL(mla_splitkv_reduce_kernel, dim3((unsigned)((nrows + 3) / 4)), dim3(256), 0, stream, rp);
+  return check_launch("mla_splitkv_reduce_kernel");
+}

@@ -1,0 +1,73 @@
+// Shared declarations for the gfx950 MLA / DSA kernels: vector types, error reporting, small
+// device helpers.  Everything here is internal to the library; the exported C-ABI is declared in
+// include/mla_hip.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mlahip {
+
+// ---- error reporting -------------------------------------------------------------------------
+// Entry points never throw: they return 0 or a negative code and leave a message that
+// mlahip_last_error_string() hands back (thread-local).
+enum : int {
+  MLA_OK = 0,
+  MLA_ERR_NULL = -1,      // a required pointer is null
+  MLA_ERR_SHAPE = -2,     // a size / stride is out of the range the kernel supports
+  MLA_ERR_UNSUPPORTED = -3,
+  MLA_ERR_WORKSPACE = -4, // workspace too small
+  MLA_ERR_LAUNCH = -100,  // the HIP runtime refused the launch
+};
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* what);
+
+#define MLA_REQUIRE(cond, code, ...)                 \
+  do {                                               \
+    if (!(cond)) return ::mlahip::fail((code), __VA_ARGS__); \
+  } while (0)
+
+// ---- types -----------------------------------------------------------------------------------
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define LDS_PTR(T) __attribute__((address_space(3))) T*
+#define GLB_PTR(T) __attribute__((address_space(1))) T*
+
+constexpr int kPage = 128;    // tokens per cache page
+constexpr int kDNope = 512;   // latent width (kv_lora_rank)
+constexpr int kDRope = 64;    // rope width
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// ---- device helpers --------------------------------------------------------------------------
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// value held by lane (l ^ 32)
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// 16-byte global -> LDS copy without passing through registers.  The LDS address is wave-uniform:
+// lane i's 16 bytes land at lds_base + 16 * i.
+__device__ __forceinline__ void dma16(const void* gsrc, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const GLB_PTR(void))gsrc, (LDS_PTR(void))lds_wave_base, 16, 0, 0);
+}
+
+// Transposed LDS read: within each group of 16 lanes the 16 addresses name a 4 x 16 block of
+// 16-bit elements (lane 4e+c points at row e, columns 4c..4c+3); lane j receives column j,
+// i.e. the four rows' elements at that column.
+__device__ __forceinline__ bf16x4 lds_read_tr16(const void* lds_addr) {
+  typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 v4;
+  v4 v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((LDS_PTR(v4))lds_addr);
+  return __builtin_bit_cast(bf16x4, v);
+}
+
+__device__ __forceinline__ void wait_vm(int) = delete;
+#define MLA_WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+
+}  // namespace mlahip

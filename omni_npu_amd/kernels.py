@@ -1,0 +1,154 @@
+"""torch-tensor front end of the C-ABI: validates shapes on the host, passes raw device pointers,
+strides and the current HIP stream, and never allocates behind the caller's back except for the
+split-KV workspace, which is cached per (device, size)."""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+PAGE = 128
+D_NOPE = 512
+D_ROPE = 64
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("this op runs HIP kernels only: every tensor must live on a GPU (there is no CPU path)")
+
+
+def _cache3(c: torch.Tensor, width: int) -> torch.Tensor:
+    """[nblk, page, (1,) width] -> [nblk, page, width] view."""
+    if c.dim() == 4 and c.shape[2] == 1:
+        c = c.squeeze(2)
+    if c.dim() != 3 or c.shape[-1] != width or c.stride(-1) != 1:
+        raise ValueError(f"cache must be [num_blocks, page, {width}] with a contiguous last dim, got {tuple(c.shape)}")
+    return c
+
+
+# ------------------------------------------------------------------------------------------------
+def cache_write(kv_c: torch.Tensor, k_pe: torch.Tensor, slot_mapping: torch.Tensor,
+                nope_cache: torch.Tensor, rope_cache: torch.Tensor) -> None:
+    """nope.flatten(0,1)[slot[t]] = kv_c[t]; rope.flatten(0,1)[slot[t]] = k_pe[t]; negative slots skipped
+    (reference: store_kv, src/omni_npu/attention/backends/mla.py:868-881)."""
+    _need_cuda(kv_c, k_pe, slot_mapping, nope_cache, rope_cache)
+    lib = _lib.load()
+    nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
+    k_pe = k_pe.reshape(k_pe.shape[0], -1) if k_pe.dim() == 3 else k_pe
+    t = min(slot_mapping.numel(), kv_c.shape[0])
+    if kv_c.shape[-1] != D_NOPE or k_pe.shape[-1] != D_ROPE or kv_c.stride(-1) != 1 or k_pe.stride(-1) != 1:
+        raise ValueError(f"kv_c must be [T,512] and k_pe [T,64], got {tuple(kv_c.shape)} {tuple(k_pe.shape)}")
+    if kv_c.dtype != torch.bfloat16 or k_pe.dtype != torch.bfloat16 or nope.dtype != torch.bfloat16 or rope.dtype != torch.bfloat16:
+        raise TypeError("cache_write: bf16 only")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.to(torch.int64).contiguous()
+    if nope.shape[0] != rope.shape[0] or nope.shape[1] != rope.shape[1]:
+        raise ValueError("nope and rope caches disagree on [num_blocks, page]")
+    rc = lib.mla_cache_write_bf16(kv_c.data_ptr(), kv_c.stride(0), k_pe.data_ptr(), k_pe.stride(0),
+                                  slot_mapping.data_ptr(), t, nope.data_ptr(), nope.stride(0), nope.stride(1),
+                                  rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[1], nope.shape[0],
+                                  _stream(kv_c))
+    _lib.check(rc, "mla_cache_write_bf16")
+
+
+def scatter_rows(src: torch.Tensor, slot_mapping: torch.Tensor, cache: torch.Tensor) -> None:
+    """cache.flatten(0,1)[slot[t]] = src[t] for one cache of any 16-byte-multiple row width
+    (indexer K: vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:116-121)."""
+    _need_cuda(src, slot_mapping, cache)
+    lib = _lib.load()
+    if cache.dim() == 4 and cache.shape[2] == 1:
+        cache = cache.squeeze(2)
+    src = src.reshape(src.shape[0], -1)
+    es = cache.element_size()
+    if cache.dim() != 3 or cache.stride(-1) != 1 or src.stride(-1) != 1 or src.shape[-1] != cache.shape[-1] or src.dtype != cache.dtype:
+        raise ValueError("scatter_rows: src [T,W] and cache [num_blocks,page,W] must agree in width and dtype")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.to(torch.int64).contiguous()
+    t = min(slot_mapping.numel(), src.shape[0])
+    rc = lib.mla_scatter_rows(src.data_ptr(), src.stride(0) * es, src.shape[-1] * es, slot_mapping.data_ptr(), t,
+                              cache.data_ptr(), cache.stride(0) * es, cache.stride(1) * es, cache.shape[1],
+                              cache.shape[0], _stream(src))
+    _lib.check(rc, "mla_scatter_rows")
+
+
+# ------------------------------------------------------------------------------------------------
+_workspaces: dict = {}
+
+
+def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    key = (dev.index, )
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
+def default_num_splits(batch: int, max_q_len: int, num_heads: int, max_seq_len: int, num_cus: int = 256) -> int:
+    """Static split count (a function of shapes only, so a captured graph stays valid)."""
+    groups = batch * math.ceil(max_q_len * num_heads / 128)
+    tiles = max(1, math.ceil(max_seq_len / 64))
+    want = max(1, math.ceil(4 * num_cus / max(groups, 1)))
+    return int(max(1, min(want, tiles, 64)))
+
+
+def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
+           block_table: torch.Tensor, seq_lens: torch.Tensor, scale: float, out: torch.Tensor,
+           q_len: int = 1, query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
+           num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
+           workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Absorbed-MLA paged decode (reference: FIA decode call, src/omni_npu/attention/backends/mla.py:781-804).
+
+    q_nope [T,N,512], q_rope [T,N,64] (any token/head strides), caches [nblk,128,512] / [nblk,128,64],
+    block_table int32 [B,maxblk], seq_lens int32 [B] on the device, ``out`` a bf16 tensor viewed as
+    [T,N,512] through its strides: pass ``o.transpose(0,1)`` of an [N,T,512] buffer for the reference's
+    head-major result.  Sequence b owns query tokens [b*q_len, (b+1)*q_len) unless query_start_loc
+    (int32 [B+1], device) says otherwise; token i of a request sees keys [0, L - s + i].
+    """
+    _need_cuda(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, out)
+    lib = _lib.load()
+    nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
+    t, n, _ = q_nope.shape
+    b = seq_lens.numel()
+    if q_nope.shape != (t, n, D_NOPE) or q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, D_NOPE):
+        raise ValueError(f"decode: q_nope {tuple(q_nope.shape)} q_rope {tuple(q_rope.shape)} out {tuple(out.shape)}")
+    for x in (q_nope, q_rope, out, nope, rope):
+        if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+            raise TypeError("decode: bf16 tensors with a contiguous last dim only")
+    if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32 or block_table.stride(-1) != 1:
+        raise TypeError("decode: block_table and seq_lens must be int32")
+    if not seq_lens.is_contiguous():
+        seq_lens = seq_lens.contiguous()
+    if block_table.shape[0] < b:
+        raise ValueError("decode: block_table has fewer rows than seq_lens")
+    if query_start_loc is None and t != b * q_len:
+        raise ValueError(f"decode: {t} query tokens != batch {b} x q_len {q_len}")
+    if query_start_loc is not None and (query_start_loc.dtype != torch.int32 or query_start_loc.numel() != b + 1):
+        raise TypeError("decode: query_start_loc must be int32 [B+1]")
+    if lse_out is not None and (lse_out.dtype != torch.float32 or lse_out.shape != (t, n) or not lse_out.is_contiguous()):
+        raise TypeError("decode: lse_out must be contiguous fp32 [T,N]")
+    if max_seq_len is None:
+        max_seq_len = block_table.shape[1] * nope.shape[1]
+    if nope.shape[1] != PAGE:
+        raise ValueError("decode: page size must be 128")
+    if num_splits is None:
+        num_splits = default_num_splits(b, q_len, n, max_seq_len)
+    need = lib.mla_decode_workspace_bytes(b, q_len, n, num_splits)
+    ws = workspace if workspace is not None else _workspace(q_nope.device, need)
+    rc = lib.mla_decode_bf16(
+        q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
+        nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[0],
+        block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
+        query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, n, float(scale),
+        out.data_ptr(), out.stride(0), out.stride(1), lse_out.data_ptr() if lse_out is not None else None,
+        ws.data_ptr(), ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
+    _lib.check(rc, "mla_decode_bf16")
+    return out

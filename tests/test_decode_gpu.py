@@ -1,0 +1,125 @@
+"""Parity of the HIP absorbed-MLA paged decode (through the C-ABI) against the CPU oracle.
+
+Tolerance (bf16 cache): max-abs 2e-2, mean-rel 2e-3 against the fp32 oracle.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import mla_oracle as O
+from tests.conftest import attn_close
+
+pytestmark = pytest.mark.gpu
+MAX_ABS, MEAN_REL = 2e-2, 2e-3
+
+
+def _run(case, dev, num_splits=None, head_major=False, with_lse=False):
+    from omni_npu_amd import kernels as K
+    q_nope, q_rope = case["q_nope"].to(dev), case["q_rope"].to(dev)
+    nope, rope = case["nope"].to(dev), case["rope"].to(dev)
+    bt, sl = case["block_table"].to(dev), case["seq_lens"].to(dev)
+    t, n, _ = q_nope.shape
+    if head_major:
+        buf = torch.full((n, t, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+        out = buf.transpose(0, 1)
+    else:
+        buf = out = torch.full((t, n, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(t, n, dtype=torch.float32, device=dev) if with_lse else None
+    K.decode(q_nope, q_rope, nope, rope, bt, sl, case["scale"], out, q_len=case["q_len"], lse_out=lse,
+             num_splits=num_splits)
+    torch.cuda.synchronize()
+    return buf, lse
+
+
+@pytest.mark.parametrize("num_splits", [1, 3, None])
+def test_decode_config1_plumbing(dev, num_splits):
+    """16 heads, batch 4, lens in [128,1024], shuffled block tables."""
+    case = O.make_decode_case(4, 16, 128, 1024, seed=0)
+    ref, ref_lse = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                                     case["seq_lens"], case["scale"], return_lse=True)
+    got, lse = _run(case, dev, num_splits, with_lse=True)
+    attn_close(got, ref, MAX_ABS, MEAN_REL)
+    assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
+
+
+@pytest.mark.parametrize("lens", [(1, 1), (1, 70), (63, 65), (127, 129), (200, 300)])
+def test_decode_ragged_edges(dev, lens):
+    """Sequence lengths around tile (64) and page (128) boundaries, 128 heads, head-major output."""
+    case = O.make_decode_case(5, 128, lens[0], lens[1], seed=3)
+    ref = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"])
+    got, _ = _run(case, dev, num_splits=2, head_major=True)
+    attn_close(got.transpose(0, 1), ref, MAX_ABS, MEAN_REL)
+
+
+def test_decode_single_key_returns_the_row(dev):
+    """L = 1: softmax over one key is 1, the output is that latent row exactly (in bf16)."""
+    case = O.make_decode_case(3, 128, 1, 1, seed=5)
+    got, _ = _run(case, dev, num_splits=1)
+    for b in range(3):
+        row = case["nope"][case["block_table"][b, 0].long(), 0]
+        assert torch.equal(got[b].cpu(), row.view(1, -1).expand(128, -1))
+
+
+@pytest.mark.parametrize("q_len,heads", [(2, 128), (3, 16), (2, 40)])
+def test_decode_mtp_right_down_causal(dev, q_len, heads):
+    """q_len > 1: token i of a request sees keys [0, L - q_len + i]."""
+    case = O.make_decode_case(4, heads, 130, 600, seed=7, q_len=q_len)
+    ref = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"])
+    got, _ = _run(case, dev, num_splits=3)
+    attn_close(got, ref, MAX_ABS, MEAN_REL)
+
+
+def test_decode_varlen_query_start_loc(dev):
+    from omni_npu_amd import kernels as K
+    case = O.make_decode_case(3, 16, 100, 400, seed=9, q_len=3)
+    qsl = [0, 3, 4, 6]                                  # request lengths 3, 1, 2 (tokens 0..5 used)
+    ref = O.absorbed_decode(case["q_nope"][:6], case["q_rope"][:6], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"], query_start_loc=qsl)
+    out = torch.zeros(6, 16, 512, dtype=torch.bfloat16, device=dev)
+    K.decode(case["q_nope"][:6].to(dev), case["q_rope"][:6].to(dev), case["nope"].to(dev), case["rope"].to(dev),
+             case["block_table"].to(dev), case["seq_lens"].to(dev), case["scale"], out, q_len=3,
+             query_start_loc=torch.tensor(qsl, dtype=torch.int32, device=dev), num_splits=2)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+
+
+def test_decode_strided_q_views(dev):
+    """q_rope as a slice of a wider q tensor, as the reference passes it (mla.py:902-904)."""
+    from omni_npu_amd import kernels as K
+    case = O.make_decode_case(4, 32, 64, 512, seed=11)
+    ref = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"])
+    q = torch.zeros(4, 32, 192, dtype=torch.bfloat16, device=dev)
+    q[..., 128:] = case["q_rope"].to(dev)
+    ql = case["q_nope"].to(dev).transpose(0, 1).contiguous().transpose(0, 1)     # [T,N,512] view of [N,T,512]
+    out = torch.zeros(4, 32, 512, dtype=torch.bfloat16, device=dev)
+    K.decode(ql, q[..., 128:], case["nope"].to(dev), case["rope"].to(dev), case["block_table"].to(dev),
+             case["seq_lens"].to(dev), case["scale"], out)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+
+
+def test_decode_headline_shape_properties(dev):
+    """128 heads, batch 64, lens in [4096,8192]: a sample of sequences against the oracle, and invariance of
+    the whole output under the split count and under a re-shuffle of the physical pages."""
+    from omni_npu_amd import kernels as K
+    case = O.make_decode_case(64, 128, 4096, 8192, seed=0)
+    got8, _ = _run(case, dev, num_splits=8)
+    got5, _ = _run(case, dev, num_splits=5)
+    assert (got8.float() - got5.float()).abs().max().item() <= 8e-3
+    for b in (0, 17, 63):
+        sub = dict(case)
+        ref = O.absorbed_decode(case["q_nope"][b:b + 1], case["q_rope"][b:b + 1], case["nope"], case["rope"],
+                                case["block_table"][b:b + 1], case["seq_lens"][b:b + 1], case["scale"])
+        attn_close(got8[b:b + 1], ref, MAX_ABS, MEAN_REL)
+    # physical page permutation: move every page, rewrite the tables, same answer bit for bit
+    nblk = case["nope"].shape[0]
+    perm = torch.randperm(nblk, generator=torch.Generator().manual_seed(1))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(nblk)
+    c2 = dict(case)
+    c2["nope"], c2["rope"] = case["nope"][perm], case["rope"][perm]
+    c2["block_table"] = inv[case["block_table"].long()].to(torch.int32)
+    got_perm, _ = _run(c2, dev, num_splits=8)
+    assert torch.equal(got_perm, got8)
