@@ -1,0 +1,165 @@
+#!/usr/bin/env python3
+"""Headline benchmark: DeepSeek-V3-shape absorbed-MLA paged decode, bf16, one MI355X.
+
+A step = one layer's decode attention for the whole batch: the latent-KV cache write of the new
+tokens, the split-KV decode kernel and the split reduction, inputs resident in HBM.  Prints ONE JSON
+line with the metric (us/layer, lower is better), the roofline of the dominant kernel (the split-KV
+decode kernel, timed on its own with HIP events on the launch stream) and a CPU baseline (the oracle
+on a bounded sample of the same workload, on the host cores of this box).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
+
+
+def build_workload(seed: int, batch: int, heads: int, lo: int, hi: int, q_len: int):
+    from oracle import mla_oracle as O       # input generator only (bits identical for oracle and GPU)
+    return O.make_decode_case(batch, heads, lo, hi, seed=seed, q_len=q_len)
+
+
+def algorithmic_bytes(case, heads):
+    lens = case["seq_lens"].long()
+    b = lens.numel()
+    t = b * case["q_len"]
+    kv = int(lens.sum()) * 576 * 2
+    q = t * heads * 576 * 2
+    o = t * heads * 512 * 2
+    wr = t * 576 * 2
+    tables = 4 * (int(((lens + 127) // 128).sum()) + 2 * b)
+    return dict(kv=kv, q=q, out=o, cache_write=wr, tables=tables, total=kv + q + o + wr + tables)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--heads", type=int, default=128)
+    ap.add_argument("--len-lo", type=int, default=4096)
+    ap.add_argument("--len-hi", type=int, default=8192)
+    ap.add_argument("--q-len", type=int, default=1)
+    ap.add_argument("--splits", type=int, default=0, help="KV splits per sequence (0 = library default)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no sharding, no collectives); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+
+    from omni_npu_amd import kernels as K
+    dev = torch.device("cuda:0")
+    case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
+    heads, b, q_len = args.heads, args.batch, args.q_len
+    t = b * q_len
+    g = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in case.items()}
+    out = torch.empty(heads, t, 512, dtype=torch.bfloat16, device=dev)     # head-major, as the reference returns it
+    out_v = out.transpose(0, 1)
+    max_len = int(case["seq_lens"].max())
+    splits = args.splits or K.default_num_splits(b, q_len, heads, max_len)
+    ws = torch.empty(K._lib.load().mla_decode_workspace_bytes(b, q_len, heads, splits), dtype=torch.uint8, device=dev)
+
+    def step():
+        K.cache_write(g["new_c"], g["new_r"], g["slot_mapping"], g["nope"], g["rope"])
+        K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], g["block_table"], g["seq_lens"], case["scale"], out_v,
+                 q_len=q_len, num_splits=splits, workspace=ws)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    us_per_step = wall / args.steps * 1e6
+
+    # device-side time of the whole step and of the dominant kernel alone (events on the launch stream)
+    def event_time(fn, n):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for a, e in ev:
+            a.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(e) * 1e3 for a, e in ev)
+        return sum(ts) / len(ts), ts[len(ts) // 2]
+
+    dev_step_avg, dev_step_med = event_time(step, args.steps)
+    split_only = lambda: K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], g["block_table"], g["seq_lens"],
+                                  case["scale"], out_v, q_len=q_len, num_splits=splits, workspace=ws, phase="split")
+    k_avg, k_med = event_time(split_only, args.steps)
+
+    ab = algorithmic_bytes(case, heads)
+    sum_l = int(case["seq_lens"].sum())
+    flops = sum_l * heads * q_len * 2 * (576 + 512)
+    kern_bytes = ab["kv"] + ab["q"] + ab["tables"]          # what the split kernel must read (partials excluded)
+    achieved = kern_bytes / (k_avg * 1e-6) / 1e9
+    res = {
+        "metric": "MLA decode us/layer (B=64, ctx 4k-8k, 128 heads, bf16, cache write + split-KV decode + reduce)",
+        "value": round(dev_step_avg, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(us_per_step / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: absorbed-MLA paged decode, DeepSeek-V3 shape", "batch": b, "heads": heads,
+                   "q_len": q_len, "seq_lens": f"uniform[{args.len_lo},{args.len_hi}]", "sum_seq_len": sum_l,
+                   "page": 128, "kv_splits": splits, "seed": args.seed},
+        "step_us": {"host_wall": round(us_per_step, 2), "device_avg": round(dev_step_avg, 2),
+                    "device_median": round(dev_step_med, 2)},
+        "step_tflops": round(flops / (dev_step_avg * 1e-6) / 1e12, 1),
+        "step_hbm_gbs": round(ab["total"] / (dev_step_avg * 1e-6) / 1e9, 1),
+        "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
+                                    / (dev_step_avg * 1e-6), 4),
+        "roofline": {"kernel": "mla_decode_bf16_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel_us_avg": round(k_avg, 2), "kernel_us_median": round(k_med, 2),
+                     "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),
+                     "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import mla_oracle as O
+        ncpu = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(ncpu)
+        ns = min(args.cpu_seqs, b)
+        sl = slice(0, ns * q_len)
+        cn, cr = case["nope"].clone(), case["rope"].clone()      # the oracle sees the same new rows in its cache
+        O.cache_write(cn, case["slot_mapping"], case["new_c"])
+        O.cache_write(cr, case["slot_mapping"], case["new_r"])
+
+        def cpu_once():
+            return O.absorbed_decode(case["q_nope"][sl], case["q_rope"][sl], cn, cr,
+                                     case["block_table"][:ns], case["seq_lens"][:ns], case["scale"])
+        cpu_once()
+        ts = []
+        for _ in range(3):
+            c0 = time.perf_counter()
+            ref = cpu_once()
+            ts.append(time.perf_counter() - c0)
+        sample_l = int(case["seq_lens"][:ns].sum())
+        cpu_us_full = sorted(ts)[1] * 1e6 * sum_l / sample_l
+        err = (out_v[sl].float().cpu() - ref).abs().max().item()
+        res["cpu_baseline"] = {"value": round(cpu_us_full, 1), "unit": "us/layer", "cores": ncpu, "kind": "port",
+                               "sample": f"oracle (torch fp32) on the first {ns} of {b} sequences ({sample_l} of {sum_l} "
+                                         f"cached tokens), median of 3, scaled by token count",
+                               "sample_seconds": round(sorted(ts)[1], 3), "gpu_vs_oracle_max_abs": round(err, 5)}
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

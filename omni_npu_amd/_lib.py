@@ -10,7 +10,8 @@ import os
 from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmla_hip.so")
+# OMNI_NPU_AMD_LIB points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("OMNI_NPU_AMD_LIB") or os.path.join(_HERE, "libmla_hip.so")
 
 P, I32, I64, F32, SZ = c_void_p, c_int32, c_int64, c_float, c_size_t
 
@@ -21,6 +22,9 @@ SIGNATURES = {
     "mla_cache_write_bf16": (c_int32, [P, I64, P, I64, P, I32, P, I64, I64, P, I64, I64, I32, I64, P]),
     "mla_scatter_rows": (c_int32, [P, I64, I32, P, I32, P, I64, I64, I32, I64, P]),
     "mla_decode_workspace_bytes": (SZ, [I32, I32, I32, I32]),
+    "mla_decode_bf16_split": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
+                                        I32, I32, F32, P, SZ, I32, P]),
+    "mla_splitkv_reduce": (c_int32, [P, SZ, P, I32, I32, I32, I32, P, I64, I64, P, P]),
     "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                   I32, I32, F32, P, I64, I64, P, P, SZ, I32, P]),
 }

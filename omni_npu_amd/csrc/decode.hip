@@ -31,6 +31,14 @@ constexpr int kRopeTileB = kTile * kRopeRowB;      // 8192
 constexpr int kBufB = kNopeTileB + kRopeTileB;     // 73728
 constexpr int kDecodeLdsB = 2 * kBufB;             // 147456
 constexpr int kRowsPerWg = 128;
+#ifndef MLA_QK_AHEAD
+#define MLA_QK_AHEAD 2
+#endif
+#ifndef MLA_PV_AHEAD
+#define MLA_PV_AHEAD 2
+#endif
+constexpr int kQkAhead = MLA_QK_AHEAD;               // LDS read-ahead depth, in MFMA steps
+constexpr int kPvAhead = MLA_PV_AHEAD;
 
 // 16-byte granule swizzles (functions of row % 16).  A nope row has 64 granules, a rope row 8.
 // They spread (i) 16 consecutive rows at one column over 16 distinct 16-byte bank groups for the
@@ -61,33 +69,37 @@ struct DecodeParams {
   int32_t num_splits;
 };
 
-// Issue the global -> LDS copies of one 64-token tile (18 x 16 B per lane).
-__device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int tile, int L, char* buf, int wave, int lane) {
+// Issue the global -> LDS copies of one 64-token tile (18 x 16 B per lane).  Row bases are
+// wave-uniform (scalar registers).  Wave w copies the nope rows r with r % 16 in [4w, 4w+4), so that
+// only four distinct per-lane granule permutations (dma_off, bytes) are needed.
+__device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int tile, int L, uint32_t buf, int wave, int lane,
+                                           const uint32_t (&dma_off)[4], const uint32_t (&rope_off)[2]) {
   const int tok0 = tile * kTile;
   int page = tok0 / kPage;
   page = page < p.max_blocks ? page : p.max_blocks - 1;
-  int64_t blk = p.block_table[(int64_t)b * p.bt_stride + page];
+  int64_t blk = __builtin_amdgcn_readfirstlane(p.block_table[(int64_t)b * p.bt_stride + page]);
   blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
   const int row_in_page0 = tok0 % kPage;
   const int last = L - 1 - tok0;                   // last valid row of this tile (>= 0)
-  const char* nope_pg = (const char*)(p.nope + blk * p.nope_sp);
-  const char* rope_pg = (const char*)(p.rope + blk * p.rope_sp);
+  const char* nope_pg = (const char*)(p.nope + blk * p.nope_sp) + (int64_t)row_in_page0 * p.nope_sr * 2;
+  const char* rope_pg = (const char*)(p.rope + blk * p.rope_sp) + (int64_t)row_in_page0 * p.rope_sr * 2;
 #pragma unroll
-  for (int i = 0; i < 16; i++) {
-    const int r = wave * 16 + i;
-    const int re = r < last ? r : last;            // rows past the end re-read the last valid row
-    const int c = lane ^ swz_nope(r & 15);
-    const char* g = nope_pg + (int64_t)(row_in_page0 + re) * p.nope_sr * 2 + c * 16;
-    dma16(g, buf + r * kNopeRowB);
-  }
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const int r = q * 16 + wave * 4 + j;
+      const int re = r < last ? r : last;          // rows past the end re-read the last valid row
+      const char* rowp = nope_pg + (int64_t)re * p.nope_sr * 2;
+      dma16_sv(rowp, dma_off[j], buf + r * kNopeRowB);
+    }
+  // rope: 8 lanes per row, wave w copies rows 16w .. 16w+15 in two steps of 8 rows
 #pragma unroll
   for (int j = 0; j < 2; j++) {
-    const int gi = wave * 128 + j * 64 + lane;
-    const int r = gi >> 3;
+    const int r0 = wave * 16 + j * 8;              // first row of this step (uniform)
+    const int r = r0 + (lane >> 3);
     const int re = r < last ? r : last;
-    const int c = (gi & 7) ^ swz_rope(r & 15);
-    const char* g = rope_pg + (int64_t)(row_in_page0 + re) * p.rope_sr * 2 + c * 16;
-    dma16(g, buf + kNopeTileB + (wave * 128 + j * 64) * 16);
+    const char* g = rope_pg + (int64_t)re * p.rope_sr * 2 + rope_off[j];
+    dma16_v(g, buf + kNopeTileB + r0 * kRopeRowB);
   }
 }
 
@@ -131,17 +143,28 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
   }
 
   // ---- prologue: first tile in flight, then the query into registers ----
-  issue_tile(p, b, tile_begin, L, lds, wave, lane);
+  // per-lane source permutations of the copies (the LDS side is linear in the lane index)
+  uint32_t dma_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) dma_off[j] = (uint32_t)((lane ^ swz_nope((wave * 4 + j) & 15)) << 4);
+  uint32_t rope_off[2];          // rope step j copies rows 16*wave + 8j + lane/8, granule slot lane%8
+#pragma unroll
+  for (int j = 0; j < 2; j++) rope_off[j] = (uint32_t)(((lane & 7) ^ swz_rope(j * 8 + (lane >> 3))) << 4);
+  const uint32_t lds0 = lds_addr_of(lds);
+  issue_tile(p, b, tile_begin, L, lds0, wave, lane, dma_off, rope_off);
 
   bf16x8 qf[36];
   {
-    const __bf16* qn = p.q_nope + (int64_t)(q0 + t_local) * p.qn_st + (int64_t)head * p.qn_sh + half * 8;
-    const __bf16* qr = p.q_rope + (int64_t)(q0 + t_local) * p.qr_st + (int64_t)head * p.qr_sh + half * 8;
+    // rows past the end read row 0 of the first token (valid memory) and are zeroed afterwards
+    const int64_t tq = row_ok ? (q0 + t_local) : q0;
+    const int64_t hq = row_ok ? head : 0;
+    const __bf16* qn = p.q_nope + tq * p.qn_st + hq * p.qn_sh + half * 8;
+    const __bf16* qr = p.q_rope + tq * p.qr_st + hq * p.qr_sh + half * 8;
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int kk = 0; kk < 32; kk++) qf[kk] = row_ok ? *(const bf16x8*)(qn + kk * 16) : zero;
+    for (int kk = 0; kk < 32; kk++) { bf16x8 v = *(const bf16x8*)(qn + kk * 16); qf[kk] = row_ok ? v : zero; }
 #pragma unroll
-    for (int kk = 0; kk < 4; kk++) qf[32 + kk] = row_ok ? *(const bf16x8*)(qr + kk * 16) : zero;
+    for (int kk = 0; kk < 4; kk++) { bf16x8 v = *(const bf16x8*)(qr + kk * 16); qf[32 + kk] = row_ok ? v : zero; }
   }
 
   f32x16 acc[16];
@@ -152,31 +175,40 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
   float m_run = -INFINITY;    // running max (log2 domain), identical in both half-waves
   float l_run = 0.f;          // running sum of this lane's 16-token slices
 
-  // per-lane LDS offsets
+  // ---- per-lane LDS offsets (the swizzle touches only the low 4 bits of a granule index, so a
+  // handful of offsets plus compile-time immediates cover every read) ----
   const int fk = swz_nope(h32 & 15);
   const int fr = swz_rope(h32 & 15);
-  const int k_row_off = h32 * kNopeRowB;                      // + tb*32*1024
-  const int r_row_off = kNopeTileB + h32 * kRopeRowB;         // + tb*32*128
+  int koff[8], roff[4];
+#pragma unroll
+  for (int j = 0; j < 8; j++) koff[j] = h32 * kNopeRowB + (((j * 2 + half) ^ fk) << 4);     // + (kk/8)*256 + tb*32768
+#pragma unroll
+  for (int j = 0; j < 4; j++) roff[j] = kNopeTileB + h32 * kRopeRowB + (((j * 2 + half) ^ fr) << 4);
   // transposed V reads: lane (g16 = lane/16, j = lane%16) points at token 4*(g16/2) + j/4 (+8*rd),
-  // columns 16*(g16%2) + 4*(j%4) .. +3 of the 32-wide d block
+  // columns 16*(g16%2) + 4*(j%4) .. +3 of the 32-wide d block db; granule = db*4 + cl
   const int g16 = lane >> 4, j16 = lane & 15;
   const int v_row = 4 * (g16 >> 1) + (j16 >> 2);              // + 8*rd + 16*kb + 32*tb
-  const int v_cl = 2 * (g16 & 1) + ((j16 & 3) >> 1);          // low 2 bits of the granule index
+  const int v_cl = 2 * (g16 & 1) + ((j16 & 3) >> 1);
   const int v_in = (j16 & 1) * 8;
-  const int v_off0 = v_row * kNopeRowB + v_in;                // rd = 0
-  const int v_off1 = (v_row + 8) * kNopeRowB + v_in;          // rd = 1
-  const int v_x0 = v_cl ^ swz_nope(v_row & 15);               // granule xor term, rd = 0
-  const int v_x1 = v_cl ^ swz_nope((v_row + 8) & 15);
+  int voff[2][4];
+#pragma unroll
+  for (int rd = 0; rd < 2; rd++) {
+    const int rr = v_row + 8 * rd;
+    const int f = swz_nope(rr & 15);
+#pragma unroll
+    for (int dl = 0; dl < 4; dl++)                            // db = 4*dq + dl; + dq*256 + kb*16384 + tb*32768
+      voff[rd][dl] = rr * kNopeRowB + v_in + ((((dl * 4 + v_cl) ^ f)) << 4);
+  }
 
   for (int tile = tile_begin; tile < tile_end; tile++) {
     char* buf = lds + ((tile - tile_begin) & 1) * kBufB;
     if (tile + 1 < tile_end) {
-      issue_tile(p, b, tile + 1, L, lds + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane);
+      issue_tile(p, b, tile + 1, L, lds0 + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane, dma_off, rope_off);
       MLA_WAIT_VMCNT(18);
     } else {
       MLA_WAIT_VMCNT(0);
     }
-    __syncthreads();
+    lds_barrier();                                            // tile visible to all four waves
 
     const int tok_base = tile * kTile;
 #pragma unroll 1
@@ -186,19 +218,21 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
       f32x16 s;
 #pragma unroll
       for (int r = 0; r < 16; r++) s[r] = 0.f;
-      const char* kb_ptr = buf + tb * 32 * kNopeRowB + k_row_off;
+      // LDS reads run kQkAhead k-steps ahead of the MFMAs that consume them
+      const char* kb_ptr = buf + tb * 32 * kNopeRowB;
+      const char* rb_ptr = buf + tb * 32 * kRopeRowB;
+      auto k_frag = [&](int kk) -> bf16x8 {
+        return kk < 32 ? *(const bf16x8*)(kb_ptr + koff[kk & 7] + (kk >> 3) * 256)
+                       : *(const bf16x8*)(rb_ptr + roff[kk & 3]);
+      };
+      bf16x8 ka[kQkAhead];
 #pragma unroll
-      for (int kk = 0; kk < 32; kk++) {
-        const int c = (kk * 2 + half) ^ fk;
-        bf16x8 a = *(const bf16x8*)(kb_ptr + c * 16);
+      for (int i = 0; i < kQkAhead; i++) ka[i] = k_frag(i);
+#pragma unroll
+      for (int kk = 0; kk < 36; kk++) {
+        const bf16x8 a = ka[kk % kQkAhead];
+        if (kk + kQkAhead < 36) ka[kk % kQkAhead] = k_frag(kk + kQkAhead);
         s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
-      }
-      const char* rb_ptr = buf + tb * 32 * kRopeRowB + r_row_off;
-#pragma unroll
-      for (int kk = 0; kk < 4; kk++) {
-        const int c = (kk * 2 + half) ^ fr;
-        bf16x8 a = *(const bf16x8*)(rb_ptr + c * 16);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[32 + kk], s, 0, 0, 0);
       }
       // ---- online softmax (log2 domain) ----
       const int tok_lane0 = tok_base + tb * 32 + 4 * half;
@@ -234,20 +268,23 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
         for (int e = 0; e < 8; e++) pb[kb][e] = (__bf16)s[kb * 8 + e];
       // ---- O^T += V^T P^T ----
       const char* vb = buf + tb * 32 * kNopeRowB;
+      auto v_frag = [&](int st) -> bf16x8 {                    // step st = 2*db + kb
+        const int db = st >> 1, kb = st & 1;
+        bf16x4 lo = lds_read_tr16(vb + kb * 16 * kNopeRowB + voff[0][db & 3] + (db >> 2) * 256);
+        bf16x4 hi = lds_read_tr16(vb + kb * 16 * kNopeRowB + voff[1][db & 3] + (db >> 2) * 256);
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      };
+      bf16x8 va[kPvAhead];
 #pragma unroll
-      for (int db = 0; db < 16; db++) {
-        const int c0 = ((db * 4) ^ v_x0) * 16;
-        const int c1 = ((db * 4) ^ v_x1) * 16;
+      for (int i = 0; i < kPvAhead; i++) va[i] = v_frag(i);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-          bf16x4 lo = lds_read_tr16(vb + kb * 16 * kNopeRowB + v_off0 + c0);
-          bf16x4 hi = lds_read_tr16(vb + kb * 16 * kNopeRowB + v_off1 + c1);
-          bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[kb], acc[db], 0, 0, 0);
-        }
+      for (int st = 0; st < 32; st++) {
+        const bf16x8 a = va[st % kPvAhead];
+        if (st + kPvAhead < 32) va[st % kPvAhead] = v_frag(st + kPvAhead);
+        acc[st >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[st & 1], acc[st >> 1], 0, 0, 0);
       }
     }
-    __syncthreads();
+    lds_barrier();                                            // everyone is done reading this buffer
   }
 
   // ---- epilogue: normalised partial + lse ----
@@ -333,16 +370,16 @@ extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, i
   return rows * kDNope * sizeof(float) + rows * sizeof(float);
 }
 
-extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
-                               int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
-                               int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
-                               int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
-                               const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
-                               const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
-                               int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
-                               int64_t out_stride_h, float* lse_out, void* workspace, size_t workspace_bytes,
-                               int32_t num_splits, hipStream_t stream) {
-  MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && block_table && seq_lens && out, MLA_ERR_NULL,
+// Phase 1: one normalised fp32 partial + log-sum-exp per (sequence, split, query row) into the workspace.
+extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                     int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                                     int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                                     int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                                     const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                     const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                                     int32_t max_q_len, int32_t num_heads, float scale, void* workspace,
+                                     size_t workspace_bytes, int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && block_table && seq_lens, MLA_ERR_NULL,
               "mla_decode_bf16: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && max_blocks >= 1 && num_pages >= 1,
               MLA_ERR_SHAPE, "mla_decode_bf16: batch=%d max_q_len=%d num_heads=%d num_splits=%d max_blocks=%d num_pages=%lld",
@@ -350,10 +387,10 @@ extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t 
   MLA_REQUIRE(num_splits <= 65535 && batch <= 65535, MLA_ERR_SHAPE, "mla_decode_bf16: grid limits exceeded");
   MLA_REQUIRE((qn_stride_t % 8 == 0) && (qn_stride_h % 8 == 0) && (qr_stride_t % 8 == 0) && (qr_stride_h % 8 == 0) &&
                   (nope_row_stride % 8 == 0) && (rope_row_stride % 8 == 0) && (nope_page_stride % 8 == 0) &&
-                  (rope_page_stride % 8 == 0) && (out_stride_t % 4 == 0) && (out_stride_h % 4 == 0),
+                  (rope_page_stride % 8 == 0),
               MLA_ERR_SHAPE, "mla_decode_bf16: strides must keep 16-byte alignment of 8-element groups");
   MLA_REQUIRE(((uintptr_t)q_nope % 16 == 0) && ((uintptr_t)q_rope % 16 == 0) && ((uintptr_t)nope_cache % 16 == 0) &&
-                  ((uintptr_t)rope_cache % 16 == 0) && ((uintptr_t)out % 8 == 0),
+                  ((uintptr_t)rope_cache % 16 == 0),
               MLA_ERR_SHAPE, "mla_decode_bf16: pointers must be 16-byte aligned");
   if (batch == 0) return MLA_OK;
   const size_t need = mla_decode_workspace_bytes(batch, max_q_len, num_heads, num_splits);
@@ -386,14 +423,51 @@ extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t 
   }
   dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
   hipLaunchKernelGGL(mla_decode_bf16_kernel, grid, dim3(256), kDecodeLdsB, stream, p);
-  if (int rc = check_launch("mla_decode_bf16_kernel")) return rc;
+  return check_launch("mla_decode_bf16_kernel");
+}
 
+// Phase 2: N-way log-sum-exp merge of the workspace partials into the bf16 output (and optional lse).
+extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* query_start_loc,
+                                  int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits, void* out,
+                                  int64_t out_stride_t, int64_t out_stride_h, float* lse_out, hipStream_t stream) {
+  MLA_REQUIRE(workspace && out, MLA_ERR_NULL, "mla_splitkv_reduce: null pointer argument");
+  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1, MLA_ERR_SHAPE,
+              "mla_splitkv_reduce: batch=%d max_q_len=%d num_heads=%d num_splits=%d", batch, max_q_len, num_heads, num_splits);
+  MLA_REQUIRE((out_stride_t % 4 == 0) && (out_stride_h % 4 == 0) && ((uintptr_t)out % 8 == 0) &&
+                  ((uintptr_t)workspace % 16 == 0),
+              MLA_ERR_SHAPE, "mla_splitkv_reduce: output rows must be 8-byte aligned");
+  if (batch == 0) return MLA_OK;
+  const size_t need = mla_decode_workspace_bytes(batch, max_q_len, num_heads, num_splits);
+  MLA_REQUIRE(workspace_bytes >= need, MLA_ERR_WORKSPACE, "mla_splitkv_reduce: workspace %zu bytes < required %zu",
+              workspace_bytes, need);
+  const int r_max = max_q_len * num_heads;
+  const size_t rows = (size_t)batch * num_splits * r_max;
   ReduceParams rp;
-  rp.o_part = p.o_part; rp.lse_part = p.lse_part; rp.qsl = query_start_loc;
+  rp.o_part = (const float*)workspace; rp.lse_part = (const float*)workspace + rows * kDNope; rp.qsl = query_start_loc;
   rp.batch = batch; rp.max_q_len = max_q_len; rp.num_heads = num_heads; rp.num_splits = num_splits;
   rp.out = (__bf16*)out; rp.out_st = out_stride_t; rp.out_sh = out_stride_h;
   rp.lse_out = lse_out; rp.lse_st = num_heads;
   const int64_t nrows = (int64_t)batch * r_max;
   hipLaunchKernelGGL(mla_splitkv_reduce_kernel, dim3((unsigned)((nrows + 3) / 4)), dim3(256), 0, stream, rp);
   return check_launch("mla_splitkv_reduce_kernel");
+}
+
+// Both phases on one stream.
+extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                               int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                               int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                               int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                               const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                               const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                               int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                               int64_t out_stride_h, float* lse_out, void* workspace, size_t workspace_bytes,
+                               int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(out, MLA_ERR_NULL, "mla_decode_bf16: null output pointer");
+  int rc = mla_decode_bf16_split(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
+                                 nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride,
+                                 num_pages, block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch,
+                                 max_q_len, num_heads, scale, workspace, workspace_bytes, num_splits, stream);
+  if (rc != MLA_OK) return rc;
+  return mla_splitkv_reduce(workspace, workspace_bytes, query_start_loc, batch, max_q_len, num_heads, num_splits, out,
+                            out_stride_t, out_stride_h, lse_out, stream);
 }

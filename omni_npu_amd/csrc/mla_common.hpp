@@ -52,10 +52,27 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // value held by lane (l ^ 32)
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
-// 16-byte global -> LDS copy without passing through registers.  The LDS address is wave-uniform:
-// lane i's 16 bytes land at lds_base + 16 * i.
-__device__ __forceinline__ void dma16(const void* gsrc, void* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((const GLB_PTR(void))gsrc, (LDS_PTR(void))lds_wave_base, 16, 0, 0);
+// 16-byte global -> LDS copies that bypass the register file.  The LDS address is wave-uniform
+// (it travels in M0): lane i's 16 bytes land at lds_addr + 16 * i.  They are written as inline
+// assembly on purpose: the compiler then does not track them, so the only waits on them are the
+// explicit MLA_WAIT_VMCNT() calls, which lets the copy of the next tile stay in flight while the
+// current one is consumed.
+__device__ __forceinline__ uint32_t lds_addr_of(const void* p) {
+  return (uint32_t)(uintptr_t)(LDS_PTR(const char))(const char*)p;
+}
+// source = uniform 64-bit base + per-lane 32-bit byte offset
+__device__ __forceinline__ void dma16_sv(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+// source = per-lane 64-bit address
+__device__ __forceinline__ void dma16_v(const void* gaddr, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+               :
+               : "s"(lds_addr_uniform), "v"(gaddr)
+               : "memory", "m0");
 }
 
 // Transposed LDS read: within each group of 16 lanes the 16 addresses name a 4 x 16 block of
@@ -67,7 +84,12 @@ __device__ __forceinline__ bf16x4 lds_read_tr16(const void* lds_addr) {
   return __builtin_bit_cast(bf16x4, v);
 }
 
-__device__ __forceinline__ void wait_vm(int) = delete;
+// Wait until at most n of this wave's global loads (LDS copies included) are outstanding.
 #define MLA_WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+
+// Workgroup barrier without the global-memory release fence of __syncthreads(): that fence waits for
+// every outstanding global load, which would serialise the prefetch of the next K tile.  All data
+// exchanged across the barrier lives in LDS; the caller waits for its own LDS copies (vmcnt) first.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 }  // namespace mlahip

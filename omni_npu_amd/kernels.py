@@ -96,7 +96,7 @@ def default_num_splits(batch: int, max_q_len: int, num_heads: int, max_seq_len: 
     """Static split count (a function of shapes only, so a captured graph stays valid)."""
     groups = batch * math.ceil(max_q_len * num_heads / 128)
     tiles = max(1, math.ceil(max_seq_len / 64))
-    want = max(1, math.ceil(4 * num_cus / max(groups, 1)))
+    want = max(1, math.ceil(num_cus / max(groups, 1)))
     return int(max(1, min(want, tiles, 64)))
 
 
@@ -104,7 +104,7 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
            block_table: torch.Tensor, seq_lens: torch.Tensor, scale: float, out: torch.Tensor,
            q_len: int = 1, query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
            num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
-           workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+           workspace: Optional[torch.Tensor] = None, phase: str = "both") -> torch.Tensor:
     """Absorbed-MLA paged decode (reference: FIA decode call, src/omni_npu/attention/backends/mla.py:781-804).
 
     q_nope [T,N,512], q_rope [T,N,64] (any token/head strides), caches [nblk,128,512] / [nblk,128,64],
@@ -112,6 +112,7 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
     [T,N,512] through its strides: pass ``o.transpose(0,1)`` of an [N,T,512] buffer for the reference's
     head-major result.  Sequence b owns query tokens [b*q_len, (b+1)*q_len) unless query_start_loc
     (int32 [B+1], device) says otherwise; token i of a request sees keys [0, L - s + i].
+    ``phase`` = "both" | "split" | "reduce" runs the split-KV kernel, the reduction, or both (one C call).
     """
     _need_cuda(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, out)
     lib = _lib.load()
@@ -143,12 +144,23 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
         num_splits = default_num_splits(b, q_len, n, max_seq_len)
     need = lib.mla_decode_workspace_bytes(b, q_len, n, num_splits)
     ws = workspace if workspace is not None else _workspace(q_nope.device, need)
-    rc = lib.mla_decode_bf16(
-        q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
-        nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[0],
-        block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
-        query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, n, float(scale),
-        out.data_ptr(), out.stride(0), out.stride(1), lse_out.data_ptr() if lse_out is not None else None,
-        ws.data_ptr(), ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
-    _lib.check(rc, "mla_decode_bf16")
+    qsl = query_start_loc.data_ptr() if query_start_loc is not None else None
+    front = (q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
+             nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1),
+             nope.shape[0], block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
+             qsl, b, q_len, n, float(scale))
+    ws_args = (ws.data_ptr(), ws.numel() * ws.element_size())
+    lse_p = lse_out.data_ptr() if lse_out is not None else None
+    st = _stream(q_nope)
+    if phase == "both":
+        rc = lib.mla_decode_bf16(*front, out.data_ptr(), out.stride(0), out.stride(1), lse_p, *ws_args, num_splits, st)
+        _lib.check(rc, "mla_decode_bf16")
+    elif phase == "split":
+        _lib.check(lib.mla_decode_bf16_split(*front, *ws_args, num_splits, st), "mla_decode_bf16_split")
+    elif phase == "reduce":
+        rc = lib.mla_splitkv_reduce(*ws_args, qsl, b, q_len, n, num_splits, out.data_ptr(), out.stride(0), out.stride(1),
+                                    lse_p, st)
+        _lib.check(rc, "mla_splitkv_reduce")
+    else:
+        raise ValueError(f"decode: unknown phase {phase!r}")
     return out
