@@ -74,3 +74,70 @@ extern "C" int mla_scatter_rows(const void* src, int64_t src_stride_bytes, int32
                      slot_mapping, num_tokens, page_size, num_pages);
   return check_launch("mla_scatter_rows");
 }
+
+// ------------------------------------------------------------------------------------------------
+// fp8-e4m3 block-scaled latent cache.  One cache row (656 bytes) per token:
+//   [0,512)    512 x float8_e4m3fn   latent, quantised per 128-element block
+//   [512,528)  4 x fp32              block scales (scale = amax / 448, 1.0 for an all-zero block)
+//   [528,656)  64 x bf16             rope part, stored unquantised
+// The reference has no fp8 KV format (attention/ops.py:11-12 ignores its scale argument), so this
+// layout is this library's own; the arithmetic is the closed form x_q = rne_e4m3(x / scale).
+// One wavefront per token: lane l owns latent elements [8l, 8l+8); 16 lanes share a block.
+namespace mlahip {
+constexpr int kFp8RowB = 656;
+constexpr int kFp8ScaleOff = 512;
+constexpr int kFp8RopeOff = 528;
+
+__global__ __launch_bounds__(256) void cache_write_fp8_kernel(const __bf16* kv_c, int64_t kv_c_stride, const __bf16* k_pe,
+                                                              int64_t k_pe_stride, const int64_t* slots,
+                                                              int32_t num_tokens, char* cache, int64_t page_stride_b,
+                                                              int64_t row_stride_b, int32_t page_size,
+                                                              int64_t num_pages) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= num_tokens) return;
+  const int64_t slot = slots[t];
+  if (slot < 0 || slot >= num_pages * page_size) return;
+  const int64_t pg = slot / page_size;
+  char* row = cache + pg * page_stride_b + (slot - pg * page_size) * row_stride_b;
+
+  const bf16x8 v = *(const bf16x8*)(kv_c + t * kv_c_stride + lane * 8);
+  float x[8];
+  float amax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) { x[e] = (float)v[e]; amax = fmaxf(amax, fabsf(x[e])); }
+#pragma unroll
+  for (int off = 1; off < 16; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));   // 16 lanes = one 128-block
+  const float scale = amax > 0.f ? amax / 448.f : 1.f;
+  float y[8];
+#pragma unroll
+  for (int e = 0; e < 8; e++) y[e] = fminf(fmaxf(x[e] / scale, -448.f), 448.f);
+  int w0 = 0, w1 = 0;
+  w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[0], y[1], w0, false);
+  w0 = __builtin_amdgcn_cvt_pk_fp8_f32(y[2], y[3], w0, true);
+  w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[4], y[5], w1, false);
+  w1 = __builtin_amdgcn_cvt_pk_fp8_f32(y[6], y[7], w1, true);
+  u32x2 packed = {(uint32_t)w0, (uint32_t)w1};
+  *(u32x2*)(row + lane * 8) = packed;
+  if ((lane & 15) == 0) *(float*)(row + kFp8ScaleOff + (lane >> 4) * 4) = scale;
+  if (lane < 8) *(u32x4*)(row + kFp8RopeOff + lane * 16) = *(const u32x4*)((const char*)(k_pe + t * k_pe_stride) + lane * 16);
+}
+}  // namespace mlahip
+
+extern "C" int mla_cache_write_fp8(const void* kv_c, int64_t kv_c_stride, const void* k_pe, int64_t k_pe_stride,
+                                   const int64_t* slot_mapping, int32_t num_tokens, void* cache,
+                                   int64_t page_stride_bytes, int64_t row_stride_bytes, int32_t page_size,
+                                   int64_t num_pages, hipStream_t stream) {
+  MLA_REQUIRE(kv_c && k_pe && slot_mapping && cache, MLA_ERR_NULL, "mla_cache_write_fp8: null pointer argument");
+  MLA_REQUIRE(num_tokens >= 0 && page_size >= 1 && num_pages >= 1, MLA_ERR_SHAPE,
+              "mla_cache_write_fp8: num_tokens=%d page_size=%d num_pages=%lld", num_tokens, page_size, (long long)num_pages);
+  MLA_REQUIRE(row_stride_bytes >= kFp8RowB && row_stride_bytes % 16 == 0 && page_stride_bytes % 16 == 0 &&
+                  kv_c_stride % 8 == 0 && k_pe_stride % 8 == 0 && (uintptr_t)kv_c % 16 == 0 && (uintptr_t)k_pe % 16 == 0 &&
+                  (uintptr_t)cache % 16 == 0,
+              MLA_ERR_SHAPE, "mla_cache_write_fp8: rows are 656 bytes, 16-byte aligned");
+  if (num_tokens == 0) return MLA_OK;
+  hipLaunchKernelGGL(cache_write_fp8_kernel, dim3((unsigned)((num_tokens + 3) / 4)), dim3(256), 0, stream,
+                     (const __bf16*)kv_c, kv_c_stride, (const __bf16*)k_pe, k_pe_stride, slot_mapping, num_tokens,
+                     (char*)cache, page_stride_bytes, row_stride_bytes, page_size, num_pages);
+  return check_launch("mla_cache_write_fp8");
+}

@@ -1,0 +1,123 @@
+// Paged gather of latent rows into a contiguous workspace, and the two-way log-sum-exp merge of
+// attention states: the two torch helpers of the reference's chunked-context prefill,
+// src/omni_npu/attention/ops.py:5-41 (gather_and_maybe_dequant_cache, which never dequantises) and
+// ops.py:44-106 (merge_attn_states).
+#include "mla_common.hpp"
+
+namespace mlahip {
+
+// One wavefront per destination row: dst[cu[i] + j] = cat(nope[row], rope[row]) for position seq_starts[i] + j.
+__global__ __launch_bounds__(256) void gather_paged_kernel(const char* nope, int64_t nope_sp, int64_t nope_sr,
+                                                           const char* rope, int64_t rope_sp, int64_t rope_sr,
+                                                           char* dst, int64_t dst_stride_b, const int32_t* block_table,
+                                                           int64_t bt_stride, int32_t max_blocks, const int32_t* cu_seq_lens,
+                                                           const int32_t* seq_starts, int32_t batch, int32_t page_size,
+                                                           int64_t num_pages, int64_t dst_rows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t total = cu_seq_lens[batch];
+  if (row >= total || row >= dst_rows) return;
+  int lo = 0, hi = batch;                          // largest i with cu[i] <= row
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_seq_lens[mid] <= row) lo = mid; else hi = mid;
+  }
+  const int64_t pos = (seq_starts ? seq_starts[lo] : 0) + (row - cu_seq_lens[lo]);
+  int64_t pg = pos / page_size;
+  const int64_t off = pos - pg * page_size;
+  pg = pg < max_blocks ? pg : max_blocks - 1;
+  int64_t blk = block_table[(int64_t)lo * bt_stride + pg];
+  blk = blk < 0 ? 0 : (blk >= num_pages ? num_pages - 1 : blk);
+  char* d = dst + row * dst_stride_b;
+  *(u32x4*)(d + lane * 16) = *(const u32x4*)(nope + blk * nope_sp + off * nope_sr + lane * 16);
+  if (lane < 8) *(u32x4*)(d + kDNope * 2 + lane * 16) = *(const u32x4*)(rope + blk * rope_sp + off * rope_sr + lane * 16);
+}
+
+template <typename T> __device__ __forceinline__ float ld(const T* p) { return (float)*p; }
+template <typename T> __device__ __forceinline__ void st(T* p, float v) { *p = (T)v; }
+
+// One wavefront per (token, head) row of width D.
+template <typename TIn, typename TOut>
+__global__ __launch_bounds__(256) void merge_states_kernel(const TIn* po, int64_t po_st, int64_t po_sh, const float* pl,
+                                                           const TIn* so, int64_t so_st, int64_t so_sh, const float* sl,
+                                                           TOut* out, int64_t out_st, int64_t out_sh, float* out_lse,
+                                                           int32_t tokens, int32_t heads, int32_t dim) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= (int64_t)tokens * heads) return;
+  const int64_t t = r / heads, h = r - t * heads;
+  float a = pl[r], b = sl[r];
+  a = a == INFINITY ? -INFINITY : a;               // +inf is what some kernels report for empty rows
+  b = b == INFINITY ? -INFINITY : b;
+  const float m = fmaxf(a, b);
+  float wa = 0.f, wb = 0.f, lse = -INFINITY;
+  if (m != -INFINITY) {
+    const float ea = __expf(a - m), eb = __expf(b - m);
+    const float tot = ea + eb;
+    wa = ea / tot;
+    wb = eb / tot;
+    lse = __logf(tot) + m;
+  }
+  const TIn* p = po + t * po_st + h * po_sh;
+  const TIn* s = so + t * so_st + h * so_sh;
+  TOut* o = out + t * out_st + h * out_sh;
+  for (int i = lane; i < dim; i += 64) {
+    // a side with zero weight contributes nothing even if it holds NaN / inf garbage
+    const float pv = wa > 0.f ? ld(p + i) * wa : 0.f;
+    const float sv = wb > 0.f ? ld(s + i) * wb : 0.f;
+    st(o + i, pv + sv);
+  }
+  if (out_lse && lane == 0) out_lse[r] = lse;
+}
+
+}  // namespace mlahip
+using namespace mlahip;
+
+extern "C" int mla_gather_paged(const void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride,
+                                const void* rope_cache, int64_t rope_page_stride, int64_t rope_row_stride,
+                                int64_t num_pages, int32_t page_size, void* dst, int64_t dst_row_stride, int64_t dst_rows,
+                                const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                const int32_t* cu_seq_lens, const int32_t* seq_starts, int32_t batch,
+                                int64_t total_rows_hint, hipStream_t stream) {
+  MLA_REQUIRE(nope_cache && rope_cache && dst && block_table && cu_seq_lens, MLA_ERR_NULL,
+              "mla_gather_paged: null pointer argument");
+  MLA_REQUIRE(batch >= 0 && page_size >= 1 && num_pages >= 1 && max_blocks >= 1 && dst_rows >= 0 && total_rows_hint >= 0,
+              MLA_ERR_SHAPE, "mla_gather_paged: batch=%d page_size=%d num_pages=%lld max_blocks=%d", batch, page_size,
+              (long long)num_pages, max_blocks);
+  MLA_REQUIRE(nope_row_stride % 8 == 0 && rope_row_stride % 8 == 0 && nope_page_stride % 8 == 0 &&
+                  rope_page_stride % 8 == 0 && dst_row_stride % 8 == 0 && dst_row_stride >= kDNope + kDRope &&
+                  (uintptr_t)nope_cache % 16 == 0 && (uintptr_t)rope_cache % 16 == 0 && (uintptr_t)dst % 16 == 0,
+              MLA_ERR_SHAPE, "mla_gather_paged: rows must be 16-byte aligned and dst rows at least 576 wide");
+  const int64_t rows = total_rows_hint < dst_rows ? total_rows_hint : dst_rows;
+  if (batch == 0 || rows == 0) return MLA_OK;
+  hipLaunchKernelGGL(gather_paged_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, (const char*)nope_cache,
+                     nope_page_stride * 2, nope_row_stride * 2, (const char*)rope_cache, rope_page_stride * 2,
+                     rope_row_stride * 2, (char*)dst, dst_row_stride * 2, block_table, bt_stride, max_blocks, cu_seq_lens,
+                     seq_starts, batch, page_size, num_pages, dst_rows);
+  return check_launch("mla_gather_paged");
+}
+
+// dtype codes: 0 = bf16, 1 = fp32
+extern "C" int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_stride_h, const float* prefix_lse,
+                                const void* suffix_out, int64_t so_stride_t, int64_t so_stride_h, const float* suffix_lse,
+                                int32_t in_dtype, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
+                                float* out_lse, int32_t tokens, int32_t heads, int32_t dim, hipStream_t stream) {
+  MLA_REQUIRE(prefix_out && prefix_lse && suffix_out && suffix_lse && out, MLA_ERR_NULL,
+              "mla_merge_states: null pointer argument");
+  MLA_REQUIRE(tokens >= 0 && heads >= 1 && dim >= 1, MLA_ERR_SHAPE, "mla_merge_states: tokens=%d heads=%d dim=%d", tokens,
+              heads, dim);
+  MLA_REQUIRE((in_dtype == 0 || in_dtype == 1) && (out_dtype == 0 || out_dtype == 1), MLA_ERR_UNSUPPORTED,
+              "mla_merge_states: dtype codes are 0 (bf16) and 1 (fp32)");
+  if (tokens == 0) return MLA_OK;
+  const dim3 grid((unsigned)(((int64_t)tokens * heads + 3) / 4)), block(256);
+#define MLA_MERGE(TI, TO)                                                                                              \
+  hipLaunchKernelGGL((merge_states_kernel<TI, TO>), grid, block, 0, stream, (const TI*)prefix_out, po_stride_t,        \
+                     po_stride_h, prefix_lse, (const TI*)suffix_out, so_stride_t, so_stride_h, suffix_lse, (TO*)out,   \
+                     out_stride_t, out_stride_h, out_lse, tokens, heads, dim)
+  if (in_dtype == 0 && out_dtype == 0) MLA_MERGE(__bf16, __bf16);
+  else if (in_dtype == 0 && out_dtype == 1) MLA_MERGE(__bf16, float);
+  else if (in_dtype == 1 && out_dtype == 0) MLA_MERGE(float, __bf16);
+  else MLA_MERGE(float, float);
+#undef MLA_MERGE
+  return check_launch("mla_merge_states");
+}

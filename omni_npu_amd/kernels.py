@@ -79,6 +79,81 @@ def scatter_rows(src: torch.Tensor, slot_mapping: torch.Tensor, cache: torch.Ten
     _lib.check(rc, "mla_scatter_rows")
 
 
+FP8_ROW_BYTES = 656      # 512 e4m3 + 4 fp32 block scales + 64 bf16 rope
+
+
+def cache_write_fp8(kv_c: torch.Tensor, k_pe: torch.Tensor, slot_mapping: torch.Tensor, cache: torch.Tensor) -> None:
+    """Quantise the new tokens' latent to e4m3 with one fp32 scale per 128 elements and write 656-byte rows
+    (512 fp8 | 4 fp32 scales | 64 bf16 rope) into ``cache`` = uint8 [num_blocks, page, 656]."""
+    _need_cuda(kv_c, k_pe, slot_mapping, cache)
+    lib = _lib.load()
+    k_pe = k_pe.reshape(k_pe.shape[0], -1) if k_pe.dim() == 3 else k_pe
+    if cache.dtype != torch.uint8 or cache.dim() != 3 or cache.shape[-1] != FP8_ROW_BYTES or cache.stride(-1) != 1:
+        raise ValueError(f"fp8 cache must be uint8 [num_blocks, page, {FP8_ROW_BYTES}], got {cache.dtype} {tuple(cache.shape)}")
+    if kv_c.shape[-1] != D_NOPE or k_pe.shape[-1] != D_ROPE or kv_c.dtype != torch.bfloat16 or k_pe.dtype != torch.bfloat16 \
+            or kv_c.stride(-1) != 1 or k_pe.stride(-1) != 1:
+        raise ValueError("cache_write_fp8: kv_c must be bf16 [T,512] and k_pe bf16 [T,64]")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.to(torch.int64).contiguous()
+    t = min(slot_mapping.numel(), kv_c.shape[0])
+    rc = lib.mla_cache_write_fp8(kv_c.data_ptr(), kv_c.stride(0), k_pe.data_ptr(), k_pe.stride(0), slot_mapping.data_ptr(),
+                                 t, cache.data_ptr(), cache.stride(0), cache.stride(1), cache.shape[1], cache.shape[0],
+                                 _stream(kv_c))
+    _lib.check(rc, "mla_cache_write_fp8")
+
+
+def gather_paged(nope_cache: torch.Tensor, rope_cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor,
+                 cu_seq_lens: torch.Tensor, batch_size: int, seq_starts: Optional[torch.Tensor] = None,
+                 total_rows: Optional[int] = None) -> None:
+    """dst[cu[i]:cu[i+1]] = cat(nope[blk, slot], rope[blk, slot]) for positions seq_starts[i] .. +len_i
+    (reference: gather_and_maybe_dequant_cache, src/omni_npu/attention/ops.py:5-41).  cu_seq_lens / seq_starts are
+    int32 device tensors; ``total_rows`` bounds the launch (defaults to dst.shape[0]) so no host sync is needed."""
+    _need_cuda(nope_cache, rope_cache, dst, block_table, cu_seq_lens, seq_starts)
+    lib = _lib.load()
+    nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
+    if dst.dim() != 2 or dst.shape[1] < D_NOPE + D_ROPE or dst.stride(1) != 1 or dst.dtype != nope.dtype or nope.dtype != torch.bfloat16:
+        raise ValueError("gather_paged: dst must be bf16 [rows, >=576] like the caches")
+    if block_table.dtype != torch.int32 or cu_seq_lens.dtype != torch.int32 or not cu_seq_lens.is_contiguous():
+        raise TypeError("gather_paged: block_table and cu_seq_lens must be int32 (cu_seq_lens contiguous)")
+    if seq_starts is not None and (seq_starts.dtype != torch.int32 or not seq_starts.is_contiguous()):
+        raise TypeError("gather_paged: seq_starts must be contiguous int32")
+    if cu_seq_lens.numel() < batch_size + 1:
+        raise ValueError("gather_paged: cu_seq_lens needs batch_size + 1 entries")
+    rows = dst.shape[0] if total_rows is None else min(int(total_rows), dst.shape[0])
+    rc = lib.mla_gather_paged(nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1),
+                              nope.shape[0], nope.shape[1], dst.data_ptr(), dst.stride(0), dst.shape[0],
+                              block_table.data_ptr(), block_table.stride(0), block_table.shape[1], cu_seq_lens.data_ptr(),
+                              seq_starts.data_ptr() if seq_starts is not None else None, batch_size, rows, _stream(dst))
+    _lib.check(rc, "mla_gather_paged")
+
+
+_DT = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def merge_states(prefix_out: torch.Tensor, prefix_lse: torch.Tensor, suffix_out: torch.Tensor, suffix_lse: torch.Tensor,
+                 out: torch.Tensor, out_lse: Optional[torch.Tensor] = None) -> None:
+    """Two-way log-sum-exp merge (reference: merge_attn_states, src/omni_npu/attention/ops.py:44-106).
+    outputs [T,N,D] (bf16 or fp32, any token/head strides), lse fp32 [T,N] or [T,N,1] contiguous."""
+    _need_cuda(prefix_out, prefix_lse, suffix_out, suffix_lse, out, out_lse)
+    lib = _lib.load()
+    t, n, d = out.shape
+    if prefix_out.shape != out.shape or suffix_out.shape != out.shape or prefix_out.dtype != suffix_out.dtype:
+        raise ValueError("merge_states: prefix, suffix and out must share [T,N,D]; prefix and suffix share a dtype")
+    if prefix_out.dtype not in _DT or out.dtype not in _DT:
+        raise TypeError("merge_states: bf16 / fp32 only")
+    for x in (prefix_out, suffix_out, out):
+        if x.stride(-1) != 1:
+            raise ValueError("merge_states: last dim must be contiguous")
+    for l in (prefix_lse, suffix_lse, out_lse):
+        if l is not None and (l.dtype != torch.float32 or l.numel() != t * n or not l.is_contiguous()):
+            raise TypeError("merge_states: lse tensors must be contiguous fp32 with T*N elements")
+    rc = lib.mla_merge_states(prefix_out.data_ptr(), prefix_out.stride(0), prefix_out.stride(1), prefix_lse.data_ptr(),
+                              suffix_out.data_ptr(), suffix_out.stride(0), suffix_out.stride(1), suffix_lse.data_ptr(),
+                              _DT[prefix_out.dtype], out.data_ptr(), out.stride(0), out.stride(1), _DT[out.dtype],
+                              out_lse.data_ptr() if out_lse is not None else None, t, n, d, _stream(out))
+    _lib.check(rc, "mla_merge_states")
+
+
 # ------------------------------------------------------------------------------------------------
 _workspaces: dict = {}
 
