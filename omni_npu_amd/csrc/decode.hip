@@ -67,20 +67,51 @@ struct DecodeParams {
   float* o_part;                 // [B*S, R_max, 512]
   float* lse_part;               // [B*S, R_max]   (natural log)
   int32_t num_splits;
+  // sparse variant: the keys of "sequence" b are the flat cache rows sparse_rows[b, 0 .. seq_lens[b])
+  const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
 };
 
 // Issue the global -> LDS copies of one 64-token tile (18 x 16 B per lane).  Row bases are
 // wave-uniform (scalar registers).  Wave w copies the nope rows r with r % 16 in [4w, 4w+4), so that
 // only four distinct per-lane granule permutations (dma_off, bytes) are needed.
+template <bool kSparse>
 __device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int tile, int L, uint32_t buf, int wave, int lane,
                                            const uint32_t (&dma_off)[4], const uint32_t (&rope_off)[2]) {
   const int tok0 = tile * kTile;
+  const int last = L - 1 - tok0;                   // last valid row of this tile (>= 0)
+  if constexpr (kSparse) {
+    // every row has its own flat cache row id, read through the scalar cache
+    const __attribute__((address_space(4))) int32_t* rows =
+        (const __attribute__((address_space(4))) int32_t*)(p.sparse_rows + (int64_t)b * p.sparse_stride + tok0);
+    const int64_t max_row = p.num_pages * p.page_size - 1;
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int r = q * 16 + wave * 4 + j;
+        const int re = r < last ? r : last;
+        int64_t slot = rows[re];
+        slot = slot < 0 ? 0 : (slot > max_row ? max_row : slot);
+        const char* rowp = (const char*)(p.nope + slot * p.nope_sr);     // pages are contiguous (checked on the host)
+        dma16_sv(rowp, dma_off[j], buf + r * kNopeRowB);
+      }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int r0 = wave * 16 + j * 8;
+      const int r = r0 + (lane >> 3);
+      const int re = r < last ? r : last;
+      int64_t slot = p.sparse_rows[(int64_t)b * p.sparse_stride + tok0 + re];
+      slot = slot < 0 ? 0 : (slot > max_row ? max_row : slot);
+      const char* g = (const char*)(p.rope + slot * p.rope_sr) + rope_off[j];
+      dma16_v(g, buf + kNopeTileB + r0 * kRopeRowB);
+    }
+    return;
+  }
   int page = tok0 / kPage;
   page = page < p.max_blocks ? page : p.max_blocks - 1;
   int64_t blk = __builtin_amdgcn_readfirstlane(p.block_table[(int64_t)b * p.bt_stride + page]);
   blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
   const int row_in_page0 = tok0 % kPage;
-  const int last = L - 1 - tok0;                   // last valid row of this tile (>= 0)
   const char* nope_pg = (const char*)(p.nope + blk * p.nope_sp) + (int64_t)row_in_page0 * p.nope_sr * 2;
   const char* rope_pg = (const char*)(p.rope + blk * p.rope_sp) + (int64_t)row_in_page0 * p.rope_sr * 2;
 #pragma unroll
@@ -103,6 +134,7 @@ __device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int til
   }
 }
 
+template <bool kSparse>
 __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodeParams p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
@@ -151,7 +183,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
 #pragma unroll
   for (int j = 0; j < 2; j++) rope_off[j] = (uint32_t)(((lane & 7) ^ swz_rope(j * 8 + (lane >> 3))) << 4);
   const uint32_t lds0 = lds_addr_of(lds);
-  issue_tile(p, b, tile_begin, L, lds0, wave, lane, dma_off, rope_off);
+  issue_tile<kSparse>(p, b, tile_begin, L, lds0, wave, lane, dma_off, rope_off);
 
   bf16x8 qf[36];
   {
@@ -203,7 +235,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
   for (int tile = tile_begin; tile < tile_end; tile++) {
     char* buf = lds + ((tile - tile_begin) & 1) * kBufB;
     if (tile + 1 < tile_end) {
-      issue_tile(p, b, tile + 1, L, lds0 + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane, dma_off, rope_off);
+      issue_tile<kSparse>(p, b, tile + 1, L, lds0 + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane, dma_off, rope_off);
       MLA_WAIT_VMCNT(18);
     } else {
       MLA_WAIT_VMCNT(0);
@@ -370,18 +402,19 @@ extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, i
   return rows * kDNope * sizeof(float) + rows * sizeof(float);
 }
 
-// Phase 1: one normalised fp32 partial + log-sum-exp per (sequence, split, query row) into the workspace.
-extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
                                      int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
                                      int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
                                      int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
                                      const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
                                      const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
                                      int32_t max_q_len, int32_t num_heads, float scale, void* workspace,
-                                     size_t workspace_bytes, int32_t num_splits, hipStream_t stream) {
-  MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && block_table && seq_lens, MLA_ERR_NULL,
+                                     size_t workspace_bytes, int32_t num_splits, const int32_t* sparse_rows,
+                                     int64_t sparse_stride, int32_t page_size, hipStream_t stream) {
+  MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && (block_table || sparse_rows) && seq_lens, MLA_ERR_NULL,
               "mla_decode_bf16: null pointer argument");
-  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && max_blocks >= 1 && num_pages >= 1,
+  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && (sparse_rows || max_blocks >= 1) &&
+                  num_pages >= 1 && page_size >= 1,
               MLA_ERR_SHAPE, "mla_decode_bf16: batch=%d max_q_len=%d num_heads=%d num_splits=%d max_blocks=%d num_pages=%lld",
               batch, max_q_len, num_heads, num_splits, max_blocks, (long long)num_pages);
   MLA_REQUIRE(num_splits <= 65535 && batch <= 65535, MLA_ERR_SHAPE, "mla_decode_bf16: grid limits exceeded");
@@ -412,18 +445,39 @@ extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, in
   p.o_part = (float*)workspace;
   p.lse_part = (float*)workspace + rows * kDNope;
   p.num_splits = num_splits;
+  p.sparse_rows = sparse_rows; p.sparse_stride = sparse_stride; p.page_size = page_size;
 
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kDecodeLdsB);
+    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<false>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLdsB);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kDecodeLdsB);
     if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_decode_bf16: cannot reserve %d bytes of LDS: %s", kDecodeLdsB,
                                      hipGetErrorString(e));
     attr_set = true;
   }
   dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
-  hipLaunchKernelGGL(mla_decode_bf16_kernel, grid, dim3(256), kDecodeLdsB, stream, p);
+  if (sparse_rows) hipLaunchKernelGGL(mla_decode_bf16_kernel<true>, grid, dim3(256), kDecodeLdsB, stream, p);
+  else hipLaunchKernelGGL(mla_decode_bf16_kernel<false>, grid, dim3(256), kDecodeLdsB, stream, p);
   return check_launch("mla_decode_bf16_kernel");
+}
+
+// Phase 1: one normalised fp32 partial + log-sum-exp per (sequence, split, query row) into the workspace.
+extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                     int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                                     int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                                     int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                                     const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                     const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                                     int32_t max_q_len, int32_t num_heads, float scale, void* workspace,
+                                     size_t workspace_bytes, int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(block_table, MLA_ERR_NULL, "mla_decode_bf16: null block table");
+  return decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
+                           nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
+                           block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
+                           scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, stream);
 }
 
 // Phase 2: N-way log-sum-exp merge of the workspace partials into the bf16 output (and optional lse).
@@ -470,4 +524,29 @@ extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t 
   if (rc != MLA_OK) return rc;
   return mla_splitkv_reduce(workspace, workspace_bytes, query_start_loc, batch, max_q_len, num_heads, num_splits, out,
                             out_stride_t, out_stride_h, lse_out, stream);
+}
+
+// Sparse absorbed MLA over a per-token list of cache rows (reference: npu_sparse_flash_attention as called in
+// src/omni_npu/attention/backends/dsa.py:259-291).  Token t attends to the rows sparse_rows[t, 0 .. counts[t]) that
+// dsa_build_rows produced from the indexer's top-k positions.  Same split-KV kernel and reduction as the dense decode.
+extern "C" int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                      int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                                      int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                                      int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                                      int32_t page_size, const int32_t* sparse_rows, int64_t sparse_stride,
+                                      const int32_t* counts, int32_t num_tokens, int32_t num_heads, float scale, void* out,
+                                      int64_t out_stride_t, int64_t out_stride_h, float* lse_out, void* workspace,
+                                      size_t workspace_bytes, int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(sparse_rows && counts && out, MLA_ERR_NULL, "dsa_sparse_decode_bf16: null pointer argument");
+  MLA_REQUIRE(sparse_stride >= 1 && page_size >= 1, MLA_ERR_SHAPE, "dsa_sparse_decode_bf16: sparse_stride=%lld page_size=%d",
+              (long long)sparse_stride, page_size);
+  MLA_REQUIRE(nope_page_stride == (int64_t)page_size * nope_row_stride && rope_page_stride == (int64_t)page_size * rope_row_stride,
+              MLA_ERR_UNSUPPORTED, "dsa_sparse_decode_bf16: cache pages must be contiguous (page stride == page_size * row stride)");
+  int rc = decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
+                             nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
+                             nullptr, 0, 0, counts, nullptr, num_tokens, 1, num_heads, scale, workspace, workspace_bytes,
+                             num_splits, sparse_rows, sparse_stride, page_size, stream);
+  if (rc != MLA_OK) return rc;
+  return mla_splitkv_reduce(workspace, workspace_bytes, nullptr, num_tokens, 1, num_heads, num_splits, out, out_stride_t,
+                            out_stride_h, lse_out, stream);
 }

@@ -1,0 +1,161 @@
+// DSA lightning indexer: fp8 score GEMM + weighted ReLU reduction over index heads.
+//
+// Replaces the score half of torch.ops.custom.npu_lightning_indexer as the reference calls it
+// (src/omni_npu/v1/layers/attention/npu_dsa.py:92-103,
+//  src/omni_npu/vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:133-144):
+//   logit[t, s] = k_scale[s] * sum_h w[t,h] * relu(q8[t,h,:] . k8[s,:]),   s < visible(t)
+// q8 / k8 are float8_e4m3fn (OCP), 128 wide; w already carries the per-(token, head) q scale unless a
+// separate q_scale is passed.  The selection half is dsa_topk (topk.hip).
+//
+// Pure streaming kernel, no LDS: a wavefront walks blocks of 32 keys.  Lane (key = l % 32, half = l / 32)
+// loads bytes [64*half, 64*half + 64) of its key row straight from the paged cache and uses them as the B
+// operand of 8 MFMA 32x32x16 fp8 steps per head block (the k order inside a step is free as long as A
+// uses the same one).  A = the query's 64 heads x 128, held in 32 registers.  In the accumulator layout
+// a lane owns one key and 16 of the 32 heads of a block, so the weighted ReLU sum is 32 in-lane FMAs plus
+// one exchange between the two half-waves.
+#include "mla_common.hpp"
+
+namespace mlahip {
+
+constexpr int kIdxDim = 128;
+constexpr int kIdxKeysPerWave = 512;                  // 16 blocks of 32 keys
+constexpr int kIdxKeysPerWg = 4 * kIdxKeysPerWave;    // 2048
+
+struct IndexerParams {
+  const uint8_t* q8; int64_t q_st, q_sh;              // bytes
+  const float* weights; int64_t w_st;                 // [T, H]
+  const float* q_scale; int64_t qs_st;                // optional [T, H]
+  const uint8_t* k8; int64_t k_sp, k_sr;              // bytes: page stride, row stride
+  const float* k_scale; int64_t ks_sp;                // elements: page stride (row stride 1)
+  const int32_t* block_table; int64_t bt_stride; int32_t max_blocks;
+  const int32_t* seq_lens; const int32_t* qsl;
+  int32_t batch, max_q_len, num_heads, page_size;
+  int64_t num_pages;
+  float* logits; int64_t l_st;                        // [T, l_st]
+};
+
+__global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerParams p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int key_l = lane & 31, half = lane >> 5;
+  const int b = blockIdx.y / p.max_q_len;
+  const int ti = blockIdx.y - b * p.max_q_len;        // query token inside the request
+  int q0, qlen;
+  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
+  if (ti >= qlen) return;
+  const int t = q0 + ti;
+  const int L = p.seq_lens[b];
+  int limit = L - qlen + ti + 1;                       // visible keys (right-down causal)
+  limit = limit < 0 ? 0 : limit;
+  const int key_begin = blockIdx.x * kIdxKeysPerWg + wave * kIdxKeysPerWave;
+  if (key_begin >= limit) return;
+  int key_end = key_begin + kIdxKeysPerWave;
+  key_end = key_end < limit ? key_end : limit;
+
+  // A operand: head = hb*32 + key_l (as row index), bytes [64*half, +64) of that head's query row
+  long qa[2][8];
+  float wr[2][16];
+#pragma unroll
+  for (int hb = 0; hb < 2; hb++) {
+    const uint8_t* qrow = p.q8 + (int64_t)t * p.q_st + (int64_t)(hb * 32 + key_l) * p.q_sh + half * 64;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      u32x4 v = *(const u32x4*)(qrow + j * 16);
+      qa[hb][2 * j] = (long)(((uint64_t)v[1] << 32) | v[0]);
+      qa[hb][2 * j + 1] = (long)(((uint64_t)v[3] << 32) | v[2]);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int h = hb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+      float w = p.weights[(int64_t)t * p.w_st + h];
+      if (p.q_scale) w *= p.q_scale[(int64_t)t * p.qs_st + h];
+      wr[hb][r] = w;
+    }
+  }
+
+  auto load_block = [&](int key0, u32x4 (&kb)[4], float& ks) {
+    int key = key0 + key_l;
+    key = key < limit ? key : limit - 1;               // tail lanes re-read the last visible key
+    int pg = key / p.page_size;
+    const int off = key - pg * p.page_size;
+    pg = pg < p.max_blocks ? pg : p.max_blocks - 1;
+    int64_t blk = p.block_table[(int64_t)b * p.bt_stride + pg];
+    blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
+    const uint8_t* row = p.k8 + blk * p.k_sp + (int64_t)off * p.k_sr + half * 64;
+#pragma unroll
+    for (int j = 0; j < 4; j++) kb[j] = *(const u32x4*)(row + j * 16);
+    ks = p.k_scale[blk * p.ks_sp + off];
+  };
+
+  u32x4 kb[4], kn[4];
+  float ks, ksn;
+  load_block(key_begin, kb, ks);
+  for (int key0 = key_begin; key0 < key_end; key0 += 32) {
+    const bool more = key0 + 32 < key_end;
+    if (more) load_block(key0 + 32, kn, ksn);
+    f32x16 c0, c1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) { c0[r] = 0.f; c1[r] = 0.f; }
+#pragma unroll
+    for (int kk = 0; kk < 8; kk++) {
+      const u32x4 v = kb[kk >> 1];
+      const long bop = (kk & 1) ? (long)(((uint64_t)v[3] << 32) | v[2]) : (long)(((uint64_t)v[1] << 32) | v[0]);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[0][kk], bop, c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[1][kk], bop, c1, 0, 0, 0);
+    }
+    float acc = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      acc = fmaf(wr[0][r], fmaxf(c0[r], 0.f), acc);
+      acc = fmaf(wr[1][r], fmaxf(c1[r], 0.f), acc);
+    }
+    acc += xor32(acc);
+    const int key = key0 + key_l;
+    if (half == 0) p.logits[(int64_t)t * p.l_st + key] = key < limit ? acc * ks : -INFINITY;
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) kb[j] = kn[j];
+      ks = ksn;
+    }
+  }
+}
+
+}  // namespace mlahip
+using namespace mlahip;
+
+extern "C" int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_t q_stride_h, const float* weights,
+                                      int64_t w_stride_t, const float* q_scale, int64_t qs_stride_t, const void* k8_cache,
+                                      int64_t k_page_stride, int64_t k_row_stride, const float* k_scale_cache,
+                                      int64_t ks_page_stride, int64_t num_pages, int32_t page_size,
+                                      const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                      const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                                      int32_t max_q_len, int32_t num_heads, int32_t max_seq_len, float* logits,
+                                      int64_t logits_stride, hipStream_t stream) {
+  MLA_REQUIRE(q8 && weights && k8_cache && k_scale_cache && block_table && seq_lens && logits, MLA_ERR_NULL,
+              "dsa_indexer_scores_fp8: null pointer argument");
+  MLA_REQUIRE(num_heads == 64, MLA_ERR_UNSUPPORTED, "dsa_indexer_scores_fp8: 64 index heads only (got %d)", num_heads);
+  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && page_size >= 32 && page_size % 32 == 0 && num_pages >= 1 && max_blocks >= 1 &&
+                  max_seq_len >= 1,
+              MLA_ERR_SHAPE, "dsa_indexer_scores_fp8: batch=%d max_q_len=%d page_size=%d max_seq_len=%d", batch, max_q_len,
+              page_size, max_seq_len);
+  MLA_REQUIRE(q_stride_t % 16 == 0 && q_stride_h % 16 == 0 && k_page_stride % 16 == 0 && k_row_stride % 16 == 0 &&
+                  (uintptr_t)q8 % 16 == 0 && (uintptr_t)k8_cache % 16 == 0,
+              MLA_ERR_SHAPE, "dsa_indexer_scores_fp8: fp8 rows must be 16-byte aligned");
+  MLA_REQUIRE(logits_stride >= (int64_t)((max_seq_len + 31) / 32) * 32, MLA_ERR_SHAPE,
+              "dsa_indexer_scores_fp8: logits rows must hold max_seq_len rounded up to 32 (%lld < %d)",
+              (long long)logits_stride, ((max_seq_len + 31) / 32) * 32);
+  if (batch == 0) return MLA_OK;
+  MLA_REQUIRE((int64_t)batch * max_q_len <= 65535, MLA_ERR_SHAPE, "dsa_indexer_scores_fp8: too many query tokens");
+  IndexerParams p;
+  p.q8 = (const uint8_t*)q8; p.q_st = q_stride_t; p.q_sh = q_stride_h;
+  p.weights = weights; p.w_st = w_stride_t; p.q_scale = q_scale; p.qs_st = qs_stride_t;
+  p.k8 = (const uint8_t*)k8_cache; p.k_sp = k_page_stride; p.k_sr = k_row_stride;
+  p.k_scale = k_scale_cache; p.ks_sp = ks_page_stride;
+  p.block_table = block_table; p.bt_stride = bt_stride; p.max_blocks = max_blocks;
+  p.seq_lens = seq_lens; p.qsl = query_start_loc;
+  p.batch = batch; p.max_q_len = max_q_len; p.num_heads = num_heads; p.page_size = page_size; p.num_pages = num_pages;
+  p.logits = logits; p.l_st = logits_stride;
+  dim3 grid((max_seq_len + kIdxKeysPerWg - 1) / kIdxKeysPerWg, batch * max_q_len);
+  hipLaunchKernelGGL(dsa_indexer_fp8_kernel, grid, dim3(256), 0, stream, p);
+  return check_launch("dsa_indexer_fp8_kernel");
+}

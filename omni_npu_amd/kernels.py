@@ -239,3 +239,123 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
     else:
         raise ValueError(f"decode: unknown phase {phase!r}")
     return out
+
+
+# ------------------------------------------------------------------------------------------------
+# DSA: lightning indexer, top-k, sparse decode
+def indexer_logits_stride(max_seq_len: int) -> int:
+    return (int(max_seq_len) + 31) // 32 * 32
+
+
+def indexer_scores(q8: torch.Tensor, weights: torch.Tensor, k8_cache: torch.Tensor, k_scale_cache: torch.Tensor,
+                   block_table: torch.Tensor, seq_lens: torch.Tensor, logits: torch.Tensor, q_len: int = 1,
+                   q_scale: Optional[torch.Tensor] = None, query_start_loc: Optional[torch.Tensor] = None,
+                   max_seq_len: Optional[int] = None) -> torch.Tensor:
+    """logits[t, s] = k_scale[s] * sum_h w[t,h] (* q_scale[t,h]) * relu(q8[t,h] . k8[s]) for the visible keys s of token t.
+
+    q8 [T,64,128] float8_e4m3fn (or uint8 bits), weights fp32 [T,64], k8_cache [nblk,page,128] fp8, k_scale_cache fp32
+    [nblk,page], logits fp32 [T, >= round_up(max_seq_len, 32)] (reference call site:
+    src/omni_npu/v1/layers/attention/npu_dsa.py:92-103)."""
+    _need_cuda(q8, weights, k8_cache, k_scale_cache, block_table, seq_lens, logits, q_scale)
+    lib = _lib.load()
+    if k8_cache.dim() == 4 and k8_cache.shape[2] == 1:
+        k8_cache = k8_cache.squeeze(2)
+    t, h, d = q8.shape
+    b = seq_lens.numel()
+    if d != 128 or k8_cache.dim() != 3 or k8_cache.shape[-1] != 128 or q8.element_size() != 1 or k8_cache.element_size() != 1:
+        raise ValueError("indexer_scores: q8 [T,H,128] and k8_cache [nblk,page,128] must be 1-byte fp8 tensors")
+    if q8.stride(-1) != 1 or k8_cache.stride(-1) != 1:
+        raise ValueError("indexer_scores: fp8 rows must be contiguous")
+    if weights.dtype != torch.float32 or weights.shape != (t, h) or weights.stride(-1) != 1:
+        raise TypeError("indexer_scores: weights must be fp32 [T,H]")
+    if q_scale is not None and (q_scale.dtype != torch.float32 or q_scale.shape != (t, h) or q_scale.stride(-1) != 1):
+        raise TypeError("indexer_scores: q_scale must be fp32 [T,H]")
+    if k_scale_cache.dtype != torch.float32 or k_scale_cache.shape[:2] != k8_cache.shape[:2] or k_scale_cache.reshape(
+            k8_cache.shape[0], k8_cache.shape[1]).stride(-1) != 1:
+        raise TypeError("indexer_scores: k_scale_cache must be fp32 [nblk,page]")
+    k_scale_cache = k_scale_cache.reshape(k8_cache.shape[0], k8_cache.shape[1])
+    if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32 or logits.dtype != torch.float32:
+        raise TypeError("indexer_scores: int32 tables / lens, fp32 logits")
+    if max_seq_len is None:
+        max_seq_len = min(block_table.shape[1] * k8_cache.shape[1], logits.shape[1])
+    if logits.shape[0] < t or logits.stride(1) != 1 or logits.shape[1] < indexer_logits_stride(max_seq_len):
+        raise ValueError("indexer_scores: logits must be [T, >= round_up(max_seq_len, 32)]")
+    if query_start_loc is None and t != b * q_len:
+        raise ValueError(f"indexer_scores: {t} query tokens != batch {b} x q_len {q_len}")
+    rc = lib.dsa_indexer_scores_fp8(
+        q8.data_ptr(), q8.stride(0), q8.stride(1), weights.data_ptr(), weights.stride(0),
+        q_scale.data_ptr() if q_scale is not None else None, q_scale.stride(0) if q_scale is not None else 0,
+        k8_cache.data_ptr(), k8_cache.stride(0), k8_cache.stride(1), k_scale_cache.data_ptr(), k_scale_cache.stride(0),
+        k8_cache.shape[0], k8_cache.shape[1], block_table.data_ptr(), block_table.stride(0), block_table.shape[1],
+        seq_lens.data_ptr(), query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, h,
+        int(max_seq_len), logits.data_ptr(), logits.stride(0), _stream(q8))
+    _lib.check(rc, "dsa_indexer_scores_fp8")
+    return logits
+
+
+def topk(logits: torch.Tensor, seq_lens: torch.Tensor, k: int, out: torch.Tensor, q_len: int = 1,
+         query_start_loc: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Positions of the k largest logits among each token's visible keys, ties to the lower position, ascending
+    position order, -1 padding; out int32 [T,k] or [T,1,k] (patch_dsv32_indexer.py:133-146)."""
+    _need_cuda(logits, seq_lens, out)
+    lib = _lib.load()
+    o2 = out.reshape(out.shape[0], -1) if out.dim() == 3 else out
+    if o2.data_ptr() != out.data_ptr():
+        raise ValueError("topk: out must be viewable as [T,k]")
+    if logits.dtype != torch.float32 or logits.stride(-1) != 1 or o2.dtype != torch.int32 or o2.stride(-1) != 1 or o2.shape[1] < k:
+        raise TypeError("topk: fp32 logits [T,S], int32 out [T,>=k]")
+    b = seq_lens.numel()
+    rc = lib.dsa_topk(logits.data_ptr(), logits.stride(0), seq_lens.data_ptr(),
+                      query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, k, o2.data_ptr(),
+                      o2.stride(0), _stream(logits))
+    _lib.check(rc, "dsa_topk")
+    return out
+
+
+def build_sparse_rows(indices: torch.Tensor, block_table: torch.Tensor, seq_lens: torch.Tensor, page_size: int,
+                      num_pages: int, rows: torch.Tensor, counts: torch.Tensor, q_len: int = 1,
+                      query_start_loc: Optional[torch.Tensor] = None) -> None:
+    """Translate logical key positions [T,(1,)K] (-1 = unused) into flat cache rows, compacted, plus a count per token."""
+    _need_cuda(indices, block_table, seq_lens, rows, counts)
+    lib = _lib.load()
+    idx = indices.reshape(indices.shape[0], -1)
+    if idx.dtype != torch.int32 or idx.stride(-1) != 1 or rows.dtype != torch.int32 or rows.shape != idx.shape or \
+            rows.stride(-1) != 1 or counts.dtype != torch.int32 or counts.numel() < idx.shape[0] or not counts.is_contiguous():
+        raise TypeError("build_sparse_rows: int32 indices [T,K], rows [T,K], counts [T]")
+    b = seq_lens.numel()
+    rc = lib.dsa_build_rows(idx.data_ptr(), idx.stride(0), block_table.data_ptr(), block_table.stride(0),
+                            block_table.shape[1], seq_lens.data_ptr(),
+                            query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, idx.shape[1],
+                            page_size, num_pages, rows.data_ptr(), rows.stride(0), counts.data_ptr(), _stream(idx))
+    _lib.check(rc, "dsa_build_rows")
+
+
+def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
+                  rows: torch.Tensor, counts: torch.Tensor, scale: float, out: torch.Tensor,
+                  lse_out: Optional[torch.Tensor] = None, num_splits: Optional[int] = None,
+                  workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Absorbed MLA of token t over cache rows rows[t, :counts[t]] (reference: npu_sparse_flash_attention call,
+    src/omni_npu/attention/backends/dsa.py:259-291).  out bf16 viewed as [T,N,512]."""
+    _need_cuda(q_nope, q_rope, nope_cache, rope_cache, rows, counts, out)
+    lib = _lib.load()
+    nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
+    t, n, _ = q_nope.shape
+    if q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, D_NOPE) or rows.shape[0] < t or counts.numel() < t:
+        raise ValueError("sparse_decode: shape mismatch")
+    for x in (q_nope, q_rope, out, nope, rope):
+        if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+            raise TypeError("sparse_decode: bf16 tensors with a contiguous last dim only")
+    if rows.dtype != torch.int32 or counts.dtype != torch.int32 or rows.stride(-1) != 1 or not counts.is_contiguous():
+        raise TypeError("sparse_decode: int32 rows [T,K] and counts [T]")
+    if num_splits is None:
+        num_splits = default_num_splits(t, 1, n, rows.shape[1])
+    need = lib.mla_decode_workspace_bytes(t, 1, n, num_splits)
+    ws = workspace if workspace is not None else _workspace(q_nope.device, need)
+    rc = lib.dsa_sparse_decode_bf16(
+        q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
+        nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[0],
+        nope.shape[1], rows.data_ptr(), rows.stride(0), counts.data_ptr(), t, n, float(scale), out.data_ptr(),
+        out.stride(0), out.stride(1), lse_out.data_ptr() if lse_out is not None else None, ws.data_ptr(),
+        ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
+    _lib.check(rc, "dsa_sparse_decode_bf16")
+    return out

@@ -1,0 +1,145 @@
+"""DSA path on the GPU: lightning-indexer logits, exact top-k, row translation and sparse MLA vs the oracle.
+
+The reference's own tests for these ops are mocks (tests/unit/layers/test_npu_dsa.py:122-138), so the oracle here is
+pinned only against the mathematics (see tests/test_oracle.py); tolerances: logits rel 1e-4 of the row's max |logit|
+(fp32 accumulation order differs), top-k sets bit-exact on identical logits, attention 2e-2 / 2e-3.
+"""
+import pytest
+import torch
+
+from oracle import mla_oracle as O
+from tests.conftest import attn_close
+
+pytestmark = pytest.mark.gpu
+
+
+def make_indexer_case(batch, lo, hi, seed, q_len=1, heads=64, page=128):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(lo, hi + 1, (batch,), generator=g)
+    nblk_seq = (lens + page - 1) // page
+    nblk = int(nblk_seq.sum())
+    perm = torch.randperm(nblk, generator=g)
+    bt = torch.zeros(batch, int(nblk_seq.max()), dtype=torch.int32)
+    o = 0
+    for b in range(batch):
+        n = int(nblk_seq[b])
+        bt[b, :n] = perm[o:o + n].to(torch.int32)
+        o += n
+    k = torch.randn(nblk, page, 128, generator=g)
+    k8, ks = O.fp8_quant_token(k)
+    t = batch * q_len
+    q = torch.randn(t, heads, 128, generator=g)
+    q8, qs = O.fp8_quant_token(q)
+    w = torch.randn(t, heads, generator=g)
+    return dict(seq_lens=lens.to(torch.int32), block_table=bt, k8=k8, k_scale=ks, q8=q8, q_scale=qs, w=w, q_len=q_len)
+
+
+def oracle_logits(c, t):
+    q_len = c["q_len"]
+    b, i = divmod(t, q_len)
+    L = int(c["seq_lens"][b])
+    vis = L - q_len + i + 1
+    rows = O.slots_for(c["block_table"], b, 0, vis)
+    k8 = c["k8"].view(-1, 128)[rows]
+    ks = c["k_scale"].reshape(-1)[rows]
+    return O.indexer_scores(c["q8"][t], c["q_scale"][t], k8, ks, c["w"][t])
+
+
+@pytest.mark.parametrize("batch,lo,hi,q_len", [(3, 1, 200, 1), (4, 1000, 5000, 1), (2, 300, 700, 2)])
+def test_indexer_logits(dev, batch, lo, hi, q_len):
+    from omni_npu_amd import kernels as K
+    c = make_indexer_case(batch, lo, hi, seed=batch, q_len=q_len)
+    t = batch * q_len
+    max_len = int(c["seq_lens"].max())
+    logits = torch.full((t, K.indexer_logits_stride(max_len)), float("nan"), device=dev)
+    K.indexer_scores(c["q8"].to(dev), c["w"].to(dev), c["k8"].to(dev), c["k_scale"].to(dev), c["block_table"].to(dev),
+                     c["seq_lens"].to(dev), logits, q_len=q_len, q_scale=c["q_scale"].to(dev), max_seq_len=max_len)
+    got = logits.cpu()
+    for tt in range(t):
+        ref = oracle_logits(c, tt)
+        n = ref.numel()
+        tol = 1e-4 * ref.abs().max().item() + 1e-6
+        assert (got[tt, :n] - ref).abs().max().item() <= tol
+        pad_end = min((n + 31) // 32 * 32, got.shape[1])
+        assert torch.isinf(got[tt, n:pad_end]).all() and (got[tt, n:pad_end] < 0).all()
+
+
+@pytest.mark.parametrize("n,k", [(5000, 2048), (100, 2048), (2048, 2048), (2049, 2048), (70000, 2048), (3000, 7)])
+def test_topk_bit_exact_sets_and_ties(dev, n, k):
+    """Identical scores in, identical index set out; heavy ties (quantised scores) go to the lower index."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(n)
+    rows = 4
+    x = torch.randn(rows, n, generator=g)
+    x[1] = torch.round(x[1] * 4) / 4                       # many exact ties, including +-0
+    x[1, ::5] = -0.0
+    x[2] = 1.0                                             # all equal: the first k positions win
+    x[3, : n // 2] = x[3, n // 2: 2 * (n // 2)]            # every value twice
+    lens = torch.tensor([n, n, n, max(1, n - 3)], dtype=torch.int32)
+    out = torch.full((rows, 1, k), -7, dtype=torch.int32, device=dev)
+    K.topk(x.to(dev), lens.to(dev), k, out)
+    got = out.cpu().view(rows, k)
+    for r in range(rows):
+        ref = O.topk_stable(x[r], k, int(lens[r]))
+        ref_set = sorted(i for i in ref.tolist() if i >= 0)
+        g_valid = [i for i in got[r].tolist() if i >= 0]
+        assert g_valid == ref_set, f"row {r}: selection differs"
+        assert (got[r, len(g_valid):] == -1).all()
+
+
+def test_topk_on_indexer_logits_then_sparse_decode(dev):
+    """Whole DSA decode chain at small scale: logits -> top-k (set equals the oracle's on the SAME logits) ->
+    rows -> sparse MLA equals the oracle's sparse attention on that index set."""
+    from omni_npu_amd import kernels as K
+    batch, k = 4, 256
+    c = make_indexer_case(batch, 200, 3000, seed=77)
+    dc = O.make_decode_case(batch, 128, 200, 3000, seed=77)
+    dc["seq_lens"], dc["block_table"] = c["seq_lens"], c["block_table"]        # same paging for both caches
+    nblk = c["k8"].shape[0]
+    g = torch.Generator().manual_seed(5)
+    dc["nope"] = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    dc["rope"] = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    max_len = int(c["seq_lens"].max())
+    logits = torch.empty(batch, K.indexer_logits_stride(max_len), device=dev)
+    K.indexer_scores(c["q8"].to(dev), (c["w"] * c["q_scale"]).to(dev), c["k8"].to(dev), c["k_scale"].to(dev),
+                     c["block_table"].to(dev), c["seq_lens"].to(dev), logits, max_seq_len=max_len)
+    idx = torch.empty(batch, 1, k, dtype=torch.int32, device=dev)
+    K.topk(logits, c["seq_lens"].to(dev), k, idx)
+    lg = logits.cpu()
+    for b in range(batch):
+        ref = O.topk_stable(lg[b], k, int(c["seq_lens"][b]))
+        assert sorted(i for i in ref.tolist() if i >= 0) == [i for i in idx[b, 0].tolist() if i >= 0]
+    rows = torch.empty(batch, k, dtype=torch.int32, device=dev)
+    counts = torch.empty(batch, dtype=torch.int32, device=dev)
+    K.build_sparse_rows(idx, c["block_table"].to(dev), c["seq_lens"].to(dev), 128, nblk, rows, counts)
+    assert counts.cpu().tolist() == [min(k, int(l)) for l in c["seq_lens"]]
+    out = torch.empty(batch, 128, 512, dtype=torch.bfloat16, device=dev)
+    K.sparse_decode(dc["q_nope"].to(dev), dc["q_rope"].to(dev), dc["nope"].to(dev), dc["rope"].to(dev), rows, counts,
+                    dc["scale"], out, num_splits=2)
+    ref = O.sparse_decode(dc["q_nope"], dc["q_rope"], dc["nope"], dc["rope"], c["block_table"], c["seq_lens"], idx.cpu(),
+                          dc["scale"])
+    attn_close(out, ref, 2e-2, 2e-3)
+
+
+def test_sparse_decode_with_padding_and_full_coverage(dev):
+    """-1 padding and out-of-range positions are dropped; with k >= L the sparse result equals dense decode."""
+    from omni_npu_amd import kernels as K
+    dc = O.make_decode_case(3, 128, 50, 300, seed=13)
+    k = 512
+    idx = torch.full((3, 1, k), -1, dtype=torch.int32)
+    for b in range(3):
+        L = int(dc["seq_lens"][b])
+        perm = torch.randperm(L, generator=torch.Generator().manual_seed(b)).to(torch.int32)
+        idx[b, 0, 0:2 * L:2] = perm                          # interleaved with -1 holes
+    idx[0, 0, 1] = 100000                                    # beyond the sequence: ignored
+    dev_idx = idx.to(dev)
+    rows = torch.empty(3, k, dtype=torch.int32, device=dev)
+    counts = torch.empty(3, dtype=torch.int32, device=dev)
+    K.build_sparse_rows(dev_idx, dc["block_table"].to(dev), dc["seq_lens"].to(dev), 128, dc["nope"].shape[0], rows, counts)
+    assert counts.cpu().tolist() == dc["seq_lens"].tolist()
+    out = torch.empty(3, 128, 512, dtype=torch.bfloat16, device=dev)
+    K.sparse_decode(dc["q_nope"].to(dev), dc["q_rope"].to(dev), dc["nope"].to(dev), dc["rope"].to(dev), rows, counts,
+                    dc["scale"], out)
+    dense = O.absorbed_decode(dc["q_nope"], dc["q_rope"], dc["nope"], dc["rope"], dc["block_table"], dc["seq_lens"],
+                              dc["scale"])
+    attn_close(out, dense, 2e-2, 2e-3)
