@@ -1,0 +1,145 @@
+/*
+ * libmla_hip.so — C ABI of the gfx950 (MI355X) MLA / DSA attention kernels.
+ *
+ * Conventions for every entry point:
+ *   - plain device pointers, sizes and strides; strides are in ELEMENTS of the tensor's dtype unless a
+ *     parameter name ends in _bytes; the last dimension of every tensor is contiguous;
+ *   - `stream` is a hipStream_t (PyTorch-ROCm: torch.cuda.current_stream().cuda_stream); work is only
+ *     enqueued, nothing synchronises, nothing is allocated or freed, the library owns no memory;
+ *   - returns 0 on success or a negative code (-1 null pointer, -2 bad size/stride/alignment,
+ *     -3 unsupported, -4 workspace too small, -100 launch refused by the HIP runtime) and leaves a
+ *     message for mlahip_last_error_string(); never throws;
+ *   - int32 `seq_lens` / `block_table` / `query_start_loc` live on the device, so a captured HIP graph
+ *     stays valid when their contents change between replays.
+ * Paths cited below are relative to the reference tree (drago1234/omni-npu, src/omni_npu/...).
+ */
+#ifndef MLA_HIP_H
+#define MLA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ihipStream_t* mlahip_stream_t;
+
+int mlahip_version(void);
+const char* mlahip_last_error_string(void);
+
+/* ---- (a6) latent-KV cache write ------------------------------------------------------------------
+ * Replaces torch_npu.npu_scatter_nd_update_ in store_kv, attention/backends/mla.py:868-881 and
+ * attention/backends/dsa.py:359-362:  cache.flatten(0,1)[slot[t]] = src[t]; slot = page * page_size + offset;
+ * negative slots (padding) and slots past the cache are skipped. */
+int mla_cache_write_bf16(const void* kv_c, int64_t kv_c_stride,           /* bf16 [T,512] */
+                         const void* k_pe, int64_t k_pe_stride,           /* bf16 [T,64]  */
+                         const int64_t* slot_mapping, int32_t num_tokens,
+                         void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride, /* bf16 [pages,page,512] */
+                         void* rope_cache, int64_t rope_page_stride, int64_t rope_row_stride, /* bf16 [pages,page,64]  */
+                         int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
+
+/* One cache of any row width (a multiple of 16 bytes): the indexer-K scatter of
+ * vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:116-121 and
+ * v1/layers/attention/npu_dsa.py:134-139. */
+int mla_scatter_rows(const void* src, int64_t src_stride_bytes, int32_t row_bytes, const int64_t* slot_mapping,
+                     int32_t num_tokens, void* cache, int64_t page_stride_bytes, int64_t row_stride_bytes,
+                     int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
+
+/* fp8-e4m3 block-scaled latent cache: one 656-byte row per token = 512 x e4m3 | 4 x fp32 scale
+ * (scale = amax/448 per 128 elements, 1.0 for an all-zero block) | 64 x bf16 rope.  The reference has no fp8 KV
+ * format (attention/ops.py:11-12 accepts and ignores a scale; mla.py:791-792 passes antiquant_mode=0), so the layout
+ * is this library's own. */
+int mla_cache_write_fp8(const void* kv_c, int64_t kv_c_stride, const void* k_pe, int64_t k_pe_stride,
+                        const int64_t* slot_mapping, int32_t num_tokens, void* cache, int64_t page_stride_bytes,
+                        int64_t row_stride_bytes, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
+
+/* ---- (a8, a14) absorbed-MLA paged decode ----------------------------------------------------------
+ * Replaces the decode call of torch.ops.npu.npu_fused_infer_attention_score, attention/backends/mla.py:781-804
+ * (input_layout "TND_NTD", block_size 128, sparse_mode 3): sequence b owns query tokens
+ * [b*max_q_len, (b+1)*max_q_len) or [qsl[b], qsl[b+1]); token i of its s tokens sees keys [0, L_b - s + i].
+ * `out` is addressed as [T, N, 512] through its strides, so the reference's head-major [N,T,512] result is
+ * out_stride_t = 512, out_stride_h = T*512.  Page size is 128.
+ * mla_decode_bf16 = mla_decode_bf16_split (one fp32 partial + log-sum-exp per KV split, into the workspace)
+ * followed by mla_splitkv_reduce (the N-way merge of attention/ops.py:109-141). */
+size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits);
+
+int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h,   /* bf16 [T,N,512] */
+                    const void* q_rope, int64_t qr_stride_t, int64_t qr_stride_h,   /* bf16 [T,N,64]  */
+                    const void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride,
+                    const void* rope_cache, int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                    const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                    const int32_t* seq_lens, const int32_t* query_start_loc /* may be NULL */,
+                    int32_t batch, int32_t max_q_len, int32_t num_heads, float scale,
+                    void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out /* fp32 [T,N] or NULL */,
+                    void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
+
+int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                          int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,
+                          int64_t nope_row_stride, const void* rope_cache, int64_t rope_page_stride,
+                          int64_t rope_row_stride, int64_t num_pages, const int32_t* block_table, int64_t bt_stride,
+                          int32_t max_blocks, const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                          int32_t max_q_len, int32_t num_heads, float scale, void* workspace, size_t workspace_bytes,
+                          int32_t num_splits, mlahip_stream_t stream);
+
+int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* query_start_loc, int32_t batch,
+                       int32_t max_q_len, int32_t num_heads, int32_t num_splits, void* out, int64_t out_stride_t,
+                       int64_t out_stride_h, float* lse_out, mlahip_stream_t stream);
+
+/* ---- (a12, a13) chunked-context helpers -------------------------------------------------------------
+ * mla_gather_paged replaces ops.gather_and_maybe_dequant_cache (attention/ops.py:5-41, which never dequantises):
+ * dst[cu[i] + j] = cat(nope[row], rope[row]) for position seq_starts[i] + j, j < cu[i+1]-cu[i].
+ * mla_merge_states replaces ops.merge_attn_states (attention/ops.py:44-106): +inf lse reads as -inf, both sides
+ * empty gives zeros and -inf.  dtype codes: 0 = bf16, 1 = fp32. */
+int mla_gather_paged(const void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                     int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages, int32_t page_size, void* dst,
+                     int64_t dst_row_stride, int64_t dst_rows, const int32_t* block_table, int64_t bt_stride,
+                     int32_t max_blocks, const int32_t* cu_seq_lens, const int32_t* seq_starts /* may be NULL */,
+                     int32_t batch, int64_t total_rows_hint, mlahip_stream_t stream);
+
+int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_stride_h, const float* prefix_lse,
+                     const void* suffix_out, int64_t so_stride_t, int64_t so_stride_h, const float* suffix_lse,
+                     int32_t in_dtype, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
+                     float* out_lse /* may be NULL */, int32_t tokens, int32_t heads, int32_t dim, mlahip_stream_t stream);
+
+/* ---- (a15) DSA lightning indexer --------------------------------------------------------------------
+ * Replaces torch.ops.custom.npu_lightning_indexer, v1/layers/attention/npu_dsa.py:92-103 and
+ * vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:133-146, in two steps:
+ * dsa_indexer_scores_fp8: logits[t,s] = k_scale[s] * sum_h w[t,h] (* q_scale[t,h]) * relu(q8[t,h,:] . k8[s,:])
+ * for the visible keys s of token t (64 heads, 128-wide float8_e4m3fn rows, fp32 scales);
+ * dsa_topk: positions of the k largest logits, ties to the lower position, ascending order, -1 padding
+ * (int32 [T,k], the reference's [T,1,topk] buffer). */
+int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_t q_stride_h, const float* weights,
+                           int64_t w_stride_t, const float* q_scale /* may be NULL */, int64_t qs_stride_t,
+                           const void* k8_cache, int64_t k_page_stride, int64_t k_row_stride, const float* k_scale_cache,
+                           int64_t ks_page_stride, int64_t num_pages, int32_t page_size, const int32_t* block_table,
+                           int64_t bt_stride, int32_t max_blocks, const int32_t* seq_lens,
+                           const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                           int32_t max_seq_len, float* logits, int64_t logits_stride, mlahip_stream_t stream);
+
+int dsa_topk(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
+             int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
+             mlahip_stream_t stream);
+
+/* ---- (a16) sparse MLA over the selected keys ----------------------------------------------------------
+ * Replaces torch.ops.custom.npu_sparse_flash_attention, attention/backends/dsa.py:259-291 (sparse_block_size 1,
+ * layout_kv "PA_BSND"): dsa_build_rows maps the [T,k] logical positions (-1 = unused,
+ * v1/layers/attention/npu_dsa.py:553-555) through the block table to flat cache rows, compacted, with a count per
+ * token; dsa_sparse_decode_bf16 runs the absorbed-MLA kernel over those rows (cache pages must be contiguous). */
+int dsa_build_rows(const int32_t* indices, int64_t indices_stride, const int32_t* block_table, int64_t bt_stride,
+                   int32_t max_blocks, const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                   int32_t max_q_len, int32_t k, int32_t page_size, int64_t num_pages, int32_t* rows,
+                   int64_t rows_stride, int32_t* counts, mlahip_stream_t stream);
+
+int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                           int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,
+                           int64_t nope_row_stride, const void* rope_cache, int64_t rope_page_stride,
+                           int64_t rope_row_stride, int64_t num_pages, int32_t page_size, const int32_t* sparse_rows,
+                           int64_t sparse_stride, const int32_t* counts, int32_t num_tokens, int32_t num_heads,
+                           float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
+                           void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLA_HIP_H */
