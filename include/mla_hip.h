@@ -102,6 +102,19 @@ int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_str
                      int32_t in_dtype, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
                      float* out_lse /* may be NULL */, int32_t tokens, int32_t heads, int32_t dim, mlahip_stream_t stream);
 
+/* ---- (a10, a11) non-absorbed varlen attention for prefill -------------------------------------------
+ * Replaces the prefill calls of npu_fused_infer_attention_score, attention/backends/mla.py:574-590 (suffix:
+ * right-down causal, sparse_mode 3) and :415-431 (context chunk: no mask, softmax_lse_flag): q_nope [T,N,128],
+ * q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64] shared by all heads (mla.py:579 repeats it), v [Tk,N,128];
+ * cu_q / cu_k int32 [B+1] on the device; out [T,N,128] bf16 (0) or fp32 (1); lse_out fp32 [T,N] or NULL.
+ * Rows with no visible key give zeros and lse = -inf. */
+int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
+                       int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
+                       int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v, int64_t v_stride_t,
+                       int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k, int32_t batch, int32_t num_heads,
+                       int32_t max_q_len, int32_t causal, float scale, void* out, int64_t out_stride_t,
+                       int64_t out_stride_h, int32_t out_dtype, float* lse_out, mlahip_stream_t stream);
+
 /* ---- (a15) DSA lightning indexer --------------------------------------------------------------------
  * Replaces torch.ops.custom.npu_lightning_indexer, v1/layers/attention/npu_dsa.py:92-103 and
  * vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:133-146, in two steps:

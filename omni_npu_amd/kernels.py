@@ -359,3 +359,37 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
         ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
     _lib.check(rc, "dsa_sparse_decode_bf16")
     return out
+
+
+# ------------------------------------------------------------------------------------------------
+def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tensor, k_pe: torch.Tensor, v: torch.Tensor,
+                   cu_q: torch.Tensor, cu_k: torch.Tensor, max_q_len: int, scale: float, causal: bool,
+                   out: torch.Tensor, lse_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Varlen non-absorbed MLA attention (reference: the prefill FIA calls, src/omni_npu/attention/backends/mla.py:574-590
+    and :415-431).  q_nope [T,N,128], q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64] (shared by the heads), v [Tk,N,128],
+    cu_q / cu_k int32 [B+1] device tensors, out [T,N,128] bf16 or fp32, lse_out fp32 [T,N]."""
+    _need_cuda(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, out, lse_out)
+    lib = _lib.load()
+    t, n, p = q_nope.shape
+    k_pe = k_pe.reshape(k_pe.shape[0], -1)
+    if p != 128 or q_pe.shape != (t, n, 64) or k_nope.shape[1:] != (n, 128) or v.shape != k_nope.shape or \
+            k_pe.shape != (k_nope.shape[0], 64) or out.shape != (t, n, 128):
+        raise ValueError("prefill_varlen: shapes must be q_nope [T,N,128], q_pe [T,N,64], k_nope/v [Tk,N,128], k_pe [Tk,64]")
+    for x in (q_nope, q_pe, k_nope, k_pe, v):
+        if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+            raise TypeError("prefill_varlen: bf16 inputs with a contiguous last dim")
+    if out.dtype not in _DT or out.stride(-1) != 1:
+        raise TypeError("prefill_varlen: out must be bf16 or fp32")
+    if cu_q.dtype != torch.int32 or cu_k.dtype != torch.int32 or cu_q.numel() != cu_k.numel() or \
+            not cu_q.is_contiguous() or not cu_k.is_contiguous():
+        raise TypeError("prefill_varlen: cu_q / cu_k must be contiguous int32 [B+1]")
+    if lse_out is not None and (lse_out.dtype != torch.float32 or lse_out.numel() != t * n or not lse_out.is_contiguous()):
+        raise TypeError("prefill_varlen: lse_out must be contiguous fp32 [T,N]")
+    rc = lib.mla_prefill_varlen(q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_pe.data_ptr(), q_pe.stride(0),
+                                q_pe.stride(1), k_nope.data_ptr(), k_nope.stride(0), k_nope.stride(1), k_pe.data_ptr(),
+                                k_pe.stride(0), v.data_ptr(), v.stride(0), v.stride(1), cu_q.data_ptr(), cu_k.data_ptr(),
+                                cu_q.numel() - 1, n, int(max_q_len), 1 if causal else 0, float(scale), out.data_ptr(),
+                                out.stride(0), out.stride(1), _DT[out.dtype],
+                                lse_out.data_ptr() if lse_out is not None else None, _stream(q_nope))
+    _lib.check(rc, "mla_prefill_varlen")
+    return out

@@ -1,0 +1,104 @@
+"""Non-absorbed varlen prefill attention (HIP, through the C-ABI) against the oracle.
+Tolerance: max-abs 2e-2 / mean-rel 2e-3 (the reference's own bar is atol = rtol = 2e-2,
+tests/integration/attention/test_npu_mla_math.py:147-151)."""
+import pytest
+import torch
+
+from oracle import mla_oracle as O
+from tests.conftest import attn_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed, q_lens, k_lens, n):
+    g = torch.Generator().manual_seed(seed)
+    cu_q = [0]
+    cu_k = [0]
+    for a, b in zip(q_lens, k_lens):
+        cu_q.append(cu_q[-1] + a)
+        cu_k.append(cu_k[-1] + b)
+    tq, tk = cu_q[-1], cu_k[-1]
+    q = torch.randn(tq, n, 192, generator=g).bfloat16()
+    kv = (torch.randn(tk, n, 256, generator=g)).bfloat16()          # k_nope | v interleaved per head, as kv_b_proj emits
+    k_pe = torch.randn(tk, 1, 64, generator=g).bfloat16()
+    return q, kv, k_pe, cu_q, cu_k
+
+
+@pytest.mark.parametrize("causal,q_lens,k_lens,n", [
+    (True, [16, 160, 1], [16, 160, 1], 4),           # the reference's shapes (B,S) = (1,16), (8,160) and a 1-token edge
+    (True, [300, 129], [300, 129], 3),               # crosses 128-row and 64-key tile boundaries
+    (False, [16, 48, 7], [32, 100, 64], 4),          # context chunk: no mask, more keys than queries
+    (True, [40, 70], [100, 70], 2),                  # right-down alignment: more keys than queries
+    (False, [5, 9], [0, 33], 2),                     # an empty key range: zeros and lse = -inf
+])
+def test_prefill_varlen_matches_oracle(dev, causal, q_lens, k_lens, n):
+    from omni_npu_amd import kernels as K
+    q, kv, k_pe, cu_q, cu_k = _case(len(q_lens) * 7 + n, q_lens, k_lens, n)
+    scale = 192 ** -0.5
+    ref, ref_lse = O.attention_varlen(q[..., :128], q[..., 128:], kv[..., :128], k_pe.view(-1, 64), kv[..., 128:], cu_q,
+                                      cu_k, scale, causal)
+    dq, dkv, dpe = q.to(dev), kv.to(dev), k_pe.to(dev)
+    out = torch.full((q.shape[0], n, 128), float("nan"), dtype=torch.float32, device=dev)
+    lse = torch.full((q.shape[0], n), float("nan"), dtype=torch.float32, device=dev)
+    K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
+                     torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
+                     max(q_lens), scale, causal, out, lse)
+    attn_close(out, ref, 2e-2, 2e-3)
+    got_lse = lse.cpu()
+    fin = torch.isfinite(ref_lse)
+    assert torch.equal(torch.isfinite(got_lse), fin)
+    assert torch.allclose(got_lse[fin], ref_lse[fin], atol=2e-2)
+    out_bf = torch.empty(q.shape[0], n, 128, dtype=torch.bfloat16, device=dev)
+    K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
+                     torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
+                     max(q_lens), scale, causal, out_bf)
+    attn_close(out_bf, ref, 2e-2, 3e-3)
+
+
+def test_chunked_context_flow_gather_attend_merge(dev):
+    """gather -> up-project -> unmasked attention with LSE -> two-way merges -> merge with the causal suffix
+    (the loop of src/omni_npu/attention/backends/mla.py:377-450 and :573-616) equals the oracle's chunked prefill,
+    on the reference test's schedule: context 48 = chunks [32,16], suffix 16."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(5)
+    bsz, ctx, suf, n = 2, 48, 16, 4
+    w = (torch.randn(512, n * 256, generator=g) * 0.02).bfloat16()
+    nope = torch.randn(bsz, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(bsz, 128, 64, generator=g).bfloat16()
+    bt = torch.tensor([[1], [0]], dtype=torch.int32)
+    q = torch.randn(bsz * suf, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(bsz * suf, 512, generator=g).bfloat16(), torch.randn(bsz * suf, 64, generator=g).bfloat16()
+    cu_q = torch.tensor([0, suf, 2 * suf], dtype=torch.int32)
+    chunks = [(torch.tensor([0, 32, 64], dtype=torch.int32), torch.tensor([0, 0], dtype=torch.int32)),
+              (torch.tensor([0, 16, 32], dtype=torch.int32), torch.tensor([32, 32], dtype=torch.int32))]
+    scale = 192 ** -0.5
+    ref = O.chunked_prefill(q, kvc, kpe, w, nope, rope, bt, cu_q.tolist(), chunks, scale)
+
+    d = lambda x: x.to(dev)
+    dq, dw = d(q), d(w)
+    t = bsz * suf
+    kv_s = (d(kvc) @ dw).view(t, n, 256)
+    out_s = torch.empty(t, n, 128, dtype=torch.bfloat16, device=dev)
+    lse_s = torch.empty(t, n, dtype=torch.float32, device=dev)
+    K.prefill_varlen(dq[..., :128], dq[..., 128:], kv_s[..., :128], d(kpe), kv_s[..., 128:], d(cu_q), d(cu_q), suf, scale,
+                     True, out_s, lse_s)
+    ctx_out = ctx_lse = None
+    ws = torch.empty(64, 576, dtype=torch.bfloat16, device=dev)
+    for cu_k, starts in chunks:
+        toks = int(cu_k[-1])
+        K.gather_paged(d(nope), d(rope), ws, d(bt), d(cu_k), bsz, d(starts), total_rows=toks)
+        kv_c = (ws[:toks, :512] @ dw).view(toks, n, 256)
+        o_i = torch.empty(t, n, 128, dtype=torch.bfloat16, device=dev)
+        l_i = torch.empty(t, n, dtype=torch.float32, device=dev)
+        K.prefill_varlen(dq[..., :128], dq[..., 128:], kv_c[..., :128], ws[:toks, 512:], kv_c[..., 128:], d(cu_q), d(cu_k),
+                         suf, scale, False, o_i, l_i)
+        if ctx_out is None:
+            ctx_out, ctx_lse = o_i, l_i
+        else:
+            o2, l2 = torch.empty_like(o_i), torch.empty_like(l_i)
+            K.merge_states(ctx_out, ctx_lse, o_i, l_i, o2, l2)
+            ctx_out, ctx_lse = o2, l2
+    merged = torch.empty(t, n, 128, dtype=torch.float32, device=dev)
+    K.merge_states(ctx_out, ctx_lse, out_s, lse_s, merged)
+    # the reference's bar for this flow is atol = rtol = 3e-2 (tests/integration/attention/test_mla_chunked_prefill.py:72-76)
+    attn_close(merged.view(t, -1), ref, 3e-2, 6e-3)
