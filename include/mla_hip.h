@@ -86,6 +86,16 @@ int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int3
                        int32_t max_q_len, int32_t num_heads, int32_t num_splits, void* out, int64_t out_stride_t,
                        int64_t out_stride_h, float* lse_out, mlahip_stream_t stream);
 
+/* Same decode over the fp8-e4m3 block-scaled cache written by mla_cache_write_fp8 (row stride exactly 656 bytes,
+ * page size 128).  Tiles are dequantised to bf16 on chip and take the bf16 MFMA path ("dequantise, then attend").
+ * No reference counterpart: attention/backends/mla.py:791-792 passes antiquant_mode=0, antiquant_scale=None. */
+int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope, int64_t qr_stride_t,
+                   int64_t qr_stride_h, const void* cache, int64_t page_stride_bytes, int64_t row_stride_bytes,
+                   int64_t num_pages, const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                   const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch, int32_t max_q_len,
+                   int32_t num_heads, float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
+                   void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
+
 /* ---- (a12, a13) chunked-context helpers -------------------------------------------------------------
  * mla_gather_paged replaces ops.gather_and_maybe_dequant_cache (attention/ops.py:5-41, which never dequantises):
  * dst[cu[i] + j] = cat(nope[row], rope[row]) for position seq_starts[i] + j, j < cu[i+1]-cu[i].

@@ -31,6 +31,12 @@ constexpr int kRopeTileB = kTile * kRopeRowB;      // 8192
 constexpr int kBufB = kNopeTileB + kRopeTileB;     // 73728
 constexpr int kDecodeLdsB = 2 * kBufB;             // 147456
 constexpr int kRowsPerWg = 128;
+// KV source of the kernel: paged bf16 cache, per-token row list over a bf16 cache, paged fp8 block-scaled cache
+constexpr int kModeDense = 0, kModeSparse = 1, kModeFp8 = 2;
+// fp8 mode: one bf16 tile buffer (dequantised) + two raw staging buffers of 44 KiB (64 rows x 656 B, rounded up)
+constexpr int kFp8RowB = 656, kFp8ScaleOff = 512, kFp8RopeOff = 528;
+constexpr int kRawStageB = 44 * 1024;
+constexpr int kFp8LdsB = kBufB + 2 * kRawStageB;      // 163840 = all of the LDS
 #ifndef MLA_QK_AHEAD
 #define MLA_QK_AHEAD 2
 #endif
@@ -74,11 +80,12 @@ struct DecodeParams {
 // Issue the global -> LDS copies of one 64-token tile (18 x 16 B per lane).  Row bases are
 // wave-uniform (scalar registers).  Wave w copies the nope rows r with r % 16 in [4w, 4w+4), so that
 // only four distinct per-lane granule permutations (dma_off, bytes) are needed.
-template <bool kSparse>
+template <int kMode>
 __device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int tile, int L, uint32_t buf, int wave, int lane,
                                            const uint32_t (&dma_off)[4], const uint32_t (&rope_off)[2]) {
   const int tok0 = tile * kTile;
   const int last = L - 1 - tok0;                   // last valid row of this tile (>= 0)
+  constexpr bool kSparse = kMode == kModeSparse;
   if constexpr (kSparse) {
     // every row has its own flat cache row id, read through the scalar cache
     const __attribute__((address_space(4))) int32_t* rows =
@@ -134,7 +141,60 @@ __device__ __forceinline__ void issue_tile(const DecodeParams& p, int b, int til
   }
 }
 
-template <bool kSparse>
+// fp8 mode: a 64-token tile is 64 x 656 contiguous bytes inside its page; copy it linearly (44 wave copies of
+// 1 KiB, 11 per wave; the tail copies re-read the last granule of the tile).
+__device__ __forceinline__ void issue_raw_tile(const DecodeParams& p, int b, int tile, uint32_t stage, int wave, int lane) {
+  const int tok0 = tile * kTile;
+  int page = tok0 / kPage;
+  page = page < p.max_blocks ? page : p.max_blocks - 1;
+  int64_t blk = __builtin_amdgcn_readfirstlane(p.block_table[(int64_t)b * p.bt_stride + page]);
+  blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
+  const char* src = (const char*)p.nope + blk * p.nope_sp + (int64_t)(tok0 % kPage) * kFp8RowB;   // strides in bytes here
+  constexpr int kGranules = kTile * kFp8RowB / 16;   // 2624
+#pragma unroll
+  for (int i = 0; i < 11; i++) {
+    const int wi = i * 4 + wave;
+    int g = wi * 64 + lane;
+    g = g < kGranules ? g : kGranules - 1;
+    dma16_sv(src, (uint32_t)g << 4, stage + wi * 1024);
+  }
+}
+
+// Dequantise the raw tile into the swizzled bf16 tile the MFMA phases read: x = e4m3 * block scale, rounded to
+// bf16; rows past `valid` become zeros (their cache bytes are not defined).
+__device__ __forceinline__ void dequant_tile(const char* raw, char* tile, int valid, int tid) {
+#pragma unroll 2
+  for (int it = 0; it < 8; it++) {
+    const int u = it * 256 + tid;
+    const int r = u >> 5, c = u & 31;                 // row, 16-element chunk
+    const u32x4 w = *(const u32x4*)(raw + r * kFp8RowB + c * 16);
+    const float sc = r < valid ? *(const float*)(raw + r * kFp8RowB + kFp8ScaleOff + (c >> 3) * 4) : 0.f;
+    u32x4 lo, hi;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[j], false);
+      const f32x2 bq = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[j], true);
+      bf16x2 x, y;
+      x[0] = (__bf16)(r < valid ? a[0] * sc : 0.f); x[1] = (__bf16)(r < valid ? a[1] * sc : 0.f);
+      y[0] = (__bf16)(r < valid ? bq[0] * sc : 0.f); y[1] = (__bf16)(r < valid ? bq[1] * sc : 0.f);
+      const uint32_t px = __builtin_bit_cast(uint32_t, x), py = __builtin_bit_cast(uint32_t, y);
+      if (j < 2) { lo[2 * j] = px; lo[2 * j + 1] = py; } else { hi[2 * (j - 2)] = px; hi[2 * (j - 2) + 1] = py; }
+    }
+    const int f = swz_nope(r & 15);
+    *(u32x4*)(tile + r * kNopeRowB + (((2 * c) ^ f) << 4)) = lo;
+    *(u32x4*)(tile + r * kNopeRowB + (((2 * c + 1) ^ f) << 4)) = hi;
+  }
+#pragma unroll
+  for (int it = 0; it < 2; it++) {
+    const int u = it * 256 + tid;
+    const int r = u >> 3, c = u & 7;
+    u32x4 w = *(const u32x4*)(raw + r * kFp8RowB + kFp8RopeOff + c * 16);
+    if (r >= valid) w = u32x4{0, 0, 0, 0};
+    *(u32x4*)(tile + kNopeTileB + r * kRopeRowB + ((c ^ swz_rope(r & 15)) << 4)) = w;
+  }
+}
+
+template <int kMode>
 __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodeParams p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
@@ -183,7 +243,8 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
 #pragma unroll
   for (int j = 0; j < 2; j++) rope_off[j] = (uint32_t)(((lane & 7) ^ swz_rope(j * 8 + (lane >> 3))) << 4);
   const uint32_t lds0 = lds_addr_of(lds);
-  issue_tile<kSparse>(p, b, tile_begin, L, lds0, wave, lane, dma_off, rope_off);
+  if constexpr (kMode == kModeFp8) issue_raw_tile(p, b, tile_begin, lds0 + kBufB, wave, lane);
+  else issue_tile<kMode>(p, b, tile_begin, L, lds0, wave, lane, dma_off, rope_off);
 
   bf16x8 qf[36];
   {
@@ -233,14 +294,28 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
   }
 
   for (int tile = tile_begin; tile < tile_end; tile++) {
-    char* buf = lds + ((tile - tile_begin) & 1) * kBufB;
-    if (tile + 1 < tile_end) {
-      issue_tile<kSparse>(p, b, tile + 1, L, lds0 + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane, dma_off, rope_off);
-      MLA_WAIT_VMCNT(18);
+    char* buf = lds;
+    if constexpr (kMode == kModeFp8) {
+      const int st = (tile - tile_begin) & 1;
+      if (tile + 1 < tile_end) {
+        issue_raw_tile(p, b, tile + 1, lds0 + kBufB + (st ^ 1) * kRawStageB, wave, lane);
+        MLA_WAIT_VMCNT(11);
+      } else {
+        MLA_WAIT_VMCNT(0);
+      }
+      lds_barrier();                                          // raw tile landed for all four waves
+      dequant_tile(lds + kBufB + st * kRawStageB, lds, L - tile * kTile, threadIdx.x);
+      lds_barrier();                                          // bf16 tile complete
     } else {
-      MLA_WAIT_VMCNT(0);
+      buf = lds + ((tile - tile_begin) & 1) * kBufB;
+      if (tile + 1 < tile_end) {
+        issue_tile<kMode>(p, b, tile + 1, L, lds0 + ((tile + 1 - tile_begin) & 1) * kBufB, wave, lane, dma_off, rope_off);
+        MLA_WAIT_VMCNT(18);
+      } else {
+        MLA_WAIT_VMCNT(0);
+      }
+      lds_barrier();                                          // tile visible to all four waves
     }
-    lds_barrier();                                            // tile visible to all four waves
 
     const int tok_base = tile * kTile;
 #pragma unroll 1
@@ -410,7 +485,7 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
                                      const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
                                      int32_t max_q_len, int32_t num_heads, float scale, void* workspace,
                                      size_t workspace_bytes, int32_t num_splits, const int32_t* sparse_rows,
-                                     int64_t sparse_stride, int32_t page_size, hipStream_t stream) {
+                                     int64_t sparse_stride, int32_t page_size, bool fp8, hipStream_t stream) {
   MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && (block_table || sparse_rows) && seq_lens, MLA_ERR_NULL,
               "mla_decode_bf16: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && (sparse_rows || max_blocks >= 1) &&
@@ -449,18 +524,22 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
 
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<false>,
+    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<kModeDense>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLdsB);
     if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                              kDecodeLdsB);
+      e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<kModeSparse>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kDecodeLdsB);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)mla_decode_bf16_kernel<kModeFp8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kFp8LdsB);
     if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_decode_bf16: cannot reserve %d bytes of LDS: %s", kDecodeLdsB,
                                      hipGetErrorString(e));
     attr_set = true;
   }
   dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
-  if (sparse_rows) hipLaunchKernelGGL(mla_decode_bf16_kernel<true>, grid, dim3(256), kDecodeLdsB, stream, p);
-  else hipLaunchKernelGGL(mla_decode_bf16_kernel<false>, grid, dim3(256), kDecodeLdsB, stream, p);
+  if (fp8) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeFp8>, grid, dim3(256), kFp8LdsB, stream, p);
+  else if (sparse_rows) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeSparse>, grid, dim3(256), kDecodeLdsB, stream, p);
+  else hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeDense>, grid, dim3(256), kDecodeLdsB, stream, p);
   return check_launch("mla_decode_bf16_kernel");
 }
 
@@ -477,7 +556,7 @@ extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, in
   return decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
                            nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
                            block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
-                           scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, stream);
+                           scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, false, stream);
 }
 
 // Phase 2: N-way log-sum-exp merge of the workspace partials into the bf16 output (and optional lse).
@@ -545,8 +624,33 @@ extern "C" int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, i
   int rc = decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
                              nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
                              nullptr, 0, 0, counts, nullptr, num_tokens, 1, num_heads, scale, workspace, workspace_bytes,
-                             num_splits, sparse_rows, sparse_stride, page_size, stream);
+                             num_splits, sparse_rows, sparse_stride, page_size, false, stream);
   if (rc != MLA_OK) return rc;
   return mla_splitkv_reduce(workspace, workspace_bytes, nullptr, num_tokens, 1, num_heads, num_splits, out, out_stride_t,
                             out_stride_h, lse_out, stream);
+}
+
+// Absorbed-MLA paged decode over the fp8-e4m3 block-scaled cache written by mla_cache_write_fp8 (656-byte rows,
+// row stride exactly 656, page size 128).  Tiles are dequantised to bf16 in LDS and then take the bf16 MFMA path, so
+// the arithmetic is "dequantise, then attend" as in the CPU restatement.  The reference has no fp8 cache
+// (src/omni_npu/attention/backends/mla.py:791-792 passes antiquant_mode=0, antiquant_scale=None).
+extern "C" int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                              int64_t qr_stride_t, int64_t qr_stride_h, const void* cache, int64_t page_stride_bytes,
+                              int64_t row_stride_bytes, int64_t num_pages, const int32_t* block_table, int64_t bt_stride,
+                              int32_t max_blocks, const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                              int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                              int64_t out_stride_h, float* lse_out, void* workspace, size_t workspace_bytes,
+                              int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(cache && out && block_table, MLA_ERR_NULL, "mla_decode_fp8: null pointer argument");
+  MLA_REQUIRE(row_stride_bytes == kFp8RowB && page_stride_bytes >= (int64_t)kPage * kFp8RowB && page_stride_bytes % 16 == 0,
+              MLA_ERR_UNSUPPORTED, "mla_decode_fp8: rows must be exactly 656 bytes apart, pages 128 rows (got %lld / %lld)",
+              (long long)row_stride_bytes, (long long)page_stride_bytes);
+  // the shared validation wants element strides that are multiples of 8: hand it byte strides that are
+  int rc = decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, cache, page_stride_bytes,
+                             kFp8RowB + 8 /* unused in fp8 mode */, cache, page_stride_bytes, kFp8RowB + 8, num_pages,
+                             block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
+                             scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, true, stream);
+  if (rc != MLA_OK) return rc;
+  return mla_splitkv_reduce(workspace, workspace_bytes, query_start_loc, batch, max_q_len, num_heads, num_splits, out,
+                            out_stride_t, out_stride_h, lse_out, stream);
 }

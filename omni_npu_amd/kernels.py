@@ -393,3 +393,41 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
                                 lse_out.data_ptr() if lse_out is not None else None, _stream(q_nope))
     _lib.check(rc, "mla_prefill_varlen")
     return out
+
+
+def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor,
+               seq_lens: torch.Tensor, scale: float, out: torch.Tensor, q_len: int = 1,
+               query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
+               num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
+               workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Absorbed-MLA paged decode over the fp8 block-scaled cache (uint8 [num_blocks, 128, 656], see cache_write_fp8)."""
+    _need_cuda(q_nope, q_rope, cache, block_table, seq_lens, out)
+    lib = _lib.load()
+    t, n, _ = q_nope.shape
+    b = seq_lens.numel()
+    if cache.dtype != torch.uint8 or cache.dim() != 3 or cache.shape[1:] != (PAGE, FP8_ROW_BYTES) or cache.stride(-1) != 1:
+        raise ValueError(f"decode_fp8: cache must be uint8 [num_blocks, {PAGE}, {FP8_ROW_BYTES}]")
+    if q_nope.shape != (t, n, D_NOPE) or q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, D_NOPE):
+        raise ValueError("decode_fp8: q_nope [T,N,512], q_rope [T,N,64], out [T,N,512]")
+    for x in (q_nope, q_rope, out):
+        if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+            raise TypeError("decode_fp8: bf16 queries / output with a contiguous last dim")
+    if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
+        raise TypeError("decode_fp8: block_table and seq_lens must be int32")
+    if query_start_loc is None and t != b * q_len:
+        raise ValueError(f"decode_fp8: {t} query tokens != batch {b} x q_len {q_len}")
+    if max_seq_len is None:
+        max_seq_len = block_table.shape[1] * PAGE
+    if num_splits is None:
+        num_splits = default_num_splits(b, q_len, n, max_seq_len)
+    need = lib.mla_decode_workspace_bytes(b, q_len, n, num_splits)
+    ws = workspace if workspace is not None else _workspace(q_nope.device, need)
+    rc = lib.mla_decode_fp8(q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0),
+                            q_rope.stride(1), cache.data_ptr(), cache.stride(0), cache.stride(1), cache.shape[0],
+                            block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
+                            query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, n, float(scale),
+                            out.data_ptr(), out.stride(0), out.stride(1),
+                            lse_out.data_ptr() if lse_out is not None else None, ws.data_ptr(),
+                            ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
+    _lib.check(rc, "mla_decode_fp8")
+    return out
