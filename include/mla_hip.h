@@ -140,6 +140,13 @@ int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_t q_stride_
                            const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
                            int32_t max_seq_len, float* logits, int64_t logits_stride, mlahip_stream_t stream);
 
+/* Per-row e4m3 quantisation of 128-wide bf16 rows (scale = amax/448 per row), optionally scattered through a slot
+ * mapping into the paged fp8 indexer-K cache and its scale cache: the indexer-K scatter of patch_dsv32_indexer.py:116-121
+ * with the quantisation fused in; with slot_mapping == NULL it quantises the query rows in place order. */
+int dsa_quant_rows_fp8(const void* src, int64_t src_stride, int64_t rows, const int64_t* slot_mapping /* may be NULL */,
+                       void* dst8, int64_t dst_page_stride_bytes, int64_t dst_row_stride_bytes, float* dst_scale,
+                       int64_t scale_page_stride, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
+
 int dsa_topk(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
              int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
              mlahip_stream_t stream);

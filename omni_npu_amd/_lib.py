@@ -36,6 +36,7 @@ SIGNATURES = {
                                      F32, P, I64, I64, I32, P, P]),
     "dsa_indexer_scores_fp8": (c_int32, [P, I64, I64, P, I64, P, I64, P, I64, I64, P, I64, I64, I32, P, I64, I32, P, P, I32,
                                          I32, I32, I32, P, I64, P]),
+    "dsa_quant_rows_fp8": (c_int32, [P, I64, I64, P, P, I64, I64, P, I64, I32, I64, P]),
     "dsa_topk": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P]),
     "dsa_build_rows": (c_int32, [P, I64, P, I64, I32, P, P, I32, I32, I32, I32, I64, P, I64, P, P]),
     "dsa_sparse_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, I32, P, I64, P, I32, I32,

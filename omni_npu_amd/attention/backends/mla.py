@@ -1,0 +1,311 @@
+"""MLA attention backend for MI355X behind the reference's vLLM plugin contract.
+
+Mirrors src/omni_npu/attention/backends/mla.py (class names, methods, metadata fields, error behaviour) for the
+single-GPU path; every vendor op there is replaced by a HIP kernel of libmla_hip.so:
+  store_kv (mla.py:868-881)                  -> kernels.cache_write / cache_write_fp8   (one launch for both caches)
+  FIA decode (mla.py:781-804)                -> kernels.decode / decode_fp8             (split-KV + reduce)
+  FIA prefill (mla.py:574-590, 415-431)      -> kernels.prefill_varlen
+  gather / merge (ops.py)                    -> kernels.gather_paged / merge_states
+The absorb and up-projection GEMMs stay torch.bmm (hipBLASLt), as in the reference (mla.py:309-315, 900-912).
+Out of scope and rejected loudly: decode context parallelism, static-sink / sliding-window variants, mc2 masks.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import ClassVar, Optional, Tuple
+
+import torch
+
+from ... import kernels as K
+from ..._vllm_compat import (AttentionCGSupport, AttentionType, MLACommonBackend, MLACommonBaseImpl,
+                             MLACommonDecodeMetadata, MLACommonMetadata, MLACommonMetadataBuilder,
+                             MLACommonPrefillMetadata, QueryLenSupport, get_current_vllm_config)
+from .. import ops
+
+FP8_CACHE_DTYPES = ("fp8", "fp8_e4m3")
+
+
+class NPUMLABackend(MLACommonBackend):
+    @staticmethod
+    def get_name() -> str:
+        return "NPUMLA"
+
+    @staticmethod
+    def get_metadata_cls() -> type["NPUMLAMetadata"]:
+        return NPUMLAMetadata
+
+    @staticmethod
+    def get_builder_cls() -> type["NPUMLAMetadataBuilder"]:
+        return NPUMLAMetadataBuilder
+
+    @staticmethod
+    def get_impl_cls() -> type["NPUMLAImpl"]:
+        return NPUMLAImpl
+
+    @staticmethod
+    def reshape_kv_cache(
+        raw_tensor: torch.Tensor,
+        num_blocks: int,
+        block_size: int,
+        num_kv_heads: int,
+        head_size: int,
+        dtype: torch.dtype = torch.bfloat16,
+    ) -> Tuple[torch.Tensor, ...]:
+        """View the per-layer raw allocation as the cache tensors (reference mla.py:59-74): all nope pages
+        [num_blocks, block, 512] first, then all rope pages [num_blocks, block, 64].  With dtype uint8 and head size
+        656 the allocation is one fp8 block-scaled cache [num_blocks, block, 656] (see kernels.cache_write_fp8)."""
+        if dtype == torch.uint8 and head_size == K.FP8_ROW_BYTES:
+            raw = raw_tensor.view(dtype=torch.uint8)
+            if raw.numel() != num_blocks * block_size * K.FP8_ROW_BYTES:
+                raise RuntimeError(f"Raw tensor has {raw.numel()} elements, while the expected size for the fp8 KV cache"
+                                   f" is {num_blocks * block_size * K.FP8_ROW_BYTES}.")
+            return (raw.view(num_blocks, block_size, K.FP8_ROW_BYTES),)
+        raw_tensor = raw_tensor.view(dtype=dtype)
+        shapes = [(num_blocks, block_size, 512), (num_blocks, block_size, 64)]
+        sizes = [math.prod(shape) for shape in shapes]
+        if raw_tensor.numel() != sum(sizes):
+            raise RuntimeError(f"Raw tensor has {raw_tensor.numel()} elements, while"
+                               f" the expected sizes for KV cache are {sizes}.")
+        tensors = torch.split(raw_tensor, sizes)
+        return tuple(t.view(shape) for t, shape in zip(tensors, shapes))
+
+
+@dataclass
+class NPUMLAPrefillMetadata(MLACommonPrefillMetadata):
+    query_cumlens: list = None
+    seq_lens: list = None
+
+
+@dataclass
+class NPUMLADecodeMetadata(MLACommonDecodeMetadata):
+    # Unlike the reference (host lists, mla.py:137-138) the lengths stay on the device so that a captured HIP graph
+    # reads fresh values on every replay; the host copies are kept for callers that want them.
+    query_cumlens: torch.Tensor = None
+    query_start_loc: torch.Tensor = None
+    seq_lens_list: list = None
+    query_cumlens_list: list = None
+    q_len: int = 1
+    max_seq_len: int = 0
+    mc2_mask: torch.Tensor = None
+
+
+@dataclass
+class NPUMLAMetadata(MLACommonMetadata[NPUMLADecodeMetadata]):
+    pass
+
+
+class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
+    _cudagraph_support: ClassVar[AttentionCGSupport] = AttentionCGSupport.ALWAYS
+    supports_uniform_spec_as_decode: ClassVar[bool] = True
+    query_len_support: ClassVar[QueryLenSupport] = QueryLenSupport.VARLEN
+
+    def __init__(self, kv_cache_spec, layer_names, vllm_config, device):
+        super().__init__(kv_cache_spec, layer_names, vllm_config, device, NPUMLAMetadata)
+        self.prefill_metadata_cls = NPUMLAPrefillMetadata
+        if self._use_fi_prefill:
+            raise ValueError("Flashinfer should not be enabled.")
+        if self._use_cudnn_prefill:
+            raise ValueError("CUDNN should not be enabled.")
+        if self.dcp_local_block_size != 1:
+            raise ValueError("DCP only support cp_kv_cache_interleave_size == 1.")
+        if self.dcp_world_size > 1:
+            raise ValueError("Decode context parallelism is not part of the single-GPU build.")
+        if self.aot_schedule:
+            raise ValueError("AOT schedule should be enabled.")
+        if self.compilation_config is not None:
+            cap = getattr(self.compilation_config, "max_cudagraph_capture_size", None) or 0
+            self.reorder_batch_threshold = max(cap, self.reorder_batch_threshold)
+
+    def _build_decode(self, block_table_tensor, seq_lens_cpu, seq_lens_device, query_start_loc_cpu,
+                      query_start_loc_device, num_decode_tokens, dcp_tot_seq_lens_device) -> NPUMLADecodeMetadata:
+        num_decodes = seq_lens_cpu.numel()
+        qlens = (query_start_loc_cpu[1:] - query_start_loc_cpu[:-1])
+        max_q = int(qlens.max()) if num_decodes else 1
+        uniform = num_decodes > 0 and int(qlens.min()) == max_q
+        return NPUMLADecodeMetadata(
+            block_table=block_table_tensor,
+            seq_lens=seq_lens_device.to(torch.int32),
+            dcp_tot_seq_lens=dcp_tot_seq_lens_device,
+            query_cumlens=query_start_loc_device[1:],
+            query_start_loc=None if uniform else query_start_loc_device.to(torch.int32).contiguous(),
+            seq_lens_list=seq_lens_cpu.tolist(),
+            query_cumlens_list=query_start_loc_cpu[1:].tolist(),
+            q_len=max_q,
+            max_seq_len=int(seq_lens_cpu.max()) if num_decodes else 0,
+        )
+
+    def build(self, common_prefix_len: int, common_attn_metadata, fast_build: bool = False) -> NPUMLAMetadata:
+        metadata = super().build(common_prefix_len, common_attn_metadata, fast_build)
+        if metadata.prefill is not None:
+            metadata.prefill.query_start_loc_list = metadata.prefill.query_start_loc.tolist()
+            metadata.prefill.query_cumlens = common_attn_metadata.query_start_loc_cpu[1:].tolist()
+            metadata.prefill.seq_lens = metadata.prefill.query_cumlens
+        return metadata
+
+
+class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
+    can_return_lse_for_decode: bool = True
+
+    def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: int,
+                 alibi_slopes: Optional[list], sliding_window: Optional[int], kv_cache_dtype: str,
+                 logits_soft_cap: Optional[float], attn_type: str, kv_sharing_target_layer_name: Optional[str],
+                 **mla_args) -> None:
+        super().__init__(num_heads, head_size, scale, num_kv_heads, alibi_slopes, sliding_window, kv_cache_dtype,
+                         logits_soft_cap, attn_type, kv_sharing_target_layer_name, **mla_args)
+        cfg = get_current_vllm_config()
+        self.chunked_prefill_workspace_size = (
+            MLACommonMetadataBuilder.determine_chunked_prefill_workspace_size(cfg) if cfg is not None else 0)
+        self.sliding_window = sliding_window
+        unsupported_features = [alibi_slopes, logits_soft_cap]
+        if any(unsupported_features):
+            raise NotImplementedError(
+                "NPUMLAImpl does not support one of the following: "
+                "alibi_slopes, logits_soft_cap")
+        if sliding_window is not None:
+            raise NotImplementedError("NPUMLAImpl: the static-sink / sliding-window variant is not part of this build")
+        if attn_type != AttentionType.DECODER:
+            raise NotImplementedError(
+                "Encoder self-attention and "
+                "encoder/decoder cross-attention "
+                "are not implemented for "
+                "NPUMLAImpl")
+        self.fp8_cache = kv_cache_dtype in FP8_CACHE_DTYPES
+
+    # ---- GEMMs around the kernels (library GEMMs, as in the reference) ----
+    def _v_up_proj(self, x: torch.Tensor) -> torch.Tensor:
+        """[N*T, 512] N-major (or [N,T,512]) -> [T, N*V]  (reference mla.py:309-315)."""
+        x = x.view(self.num_heads, -1, self.kv_lora_rank)
+        out2 = torch.bmm(x, self.W_UV)
+        return out2.transpose(0, 1).contiguous().view(-1, self.num_heads * self.v_head_dim)
+
+    def _kv_up(self, kv_c: torch.Tensor):
+        kv = self.kv_b_proj(kv_c)
+        kv = kv[0] if isinstance(kv, tuple) else kv
+        kv = kv.view(-1, self.num_heads, self.qk_nope_head_dim + self.v_head_dim)
+        return kv[..., :self.qk_nope_head_dim], kv[..., self.qk_nope_head_dim:]
+
+    # ---- prefill ----
+    def _compute_prefill_context(self, q_nope, q_pe, kv_c_cache, k_pe_cache, attn_metadata, k_scale):
+        """Chunked context: gather -> up-project -> unmasked attention with LSE -> running merge (reference mla.py:377-450)."""
+        prefill = attn_metadata.prefill
+        cc = prefill.chunked_context
+        assert cc is not None
+        t, n = q_nope.shape[0], self.num_heads
+        cu_q = prefill.query_start_loc.to(torch.int32).contiguous()
+        output = output_lse = None
+        for i in range(len(cc.seq_tot)):
+            toks = int(cc.seq_tot[i])
+            if toks == 0:
+                continue
+            ops.gather_and_maybe_dequant_cache(src_cache=(kv_c_cache, k_pe_cache), dst=cc.workspace,
+                                               block_table=prefill.block_table, cu_seq_lens=cc.cu_seq_lens[i],
+                                               batch_size=attn_metadata.num_prefills, kv_cache_dtype=self.kv_cache_dtype,
+                                               scale=k_scale, seq_starts=cc.starts[i], total_rows=toks)
+            kv_c_normed = cc.workspace[:toks][..., :self.kv_lora_rank]
+            k_pe = cc.workspace[:toks][..., self.kv_lora_rank:]
+            k_nope, v = self._kv_up(kv_c_normed)
+            attn_output = torch.empty(t, n, self.v_head_dim, dtype=q_nope.dtype, device=q_nope.device)
+            attn_lse = torch.empty(t, n, dtype=torch.float32, device=q_nope.device)
+            K.prefill_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cc.cu_seq_lens[i].to(torch.int32).contiguous(),
+                             prefill.max_query_len, self.scale, False, attn_output, attn_lse)
+            if output is None:
+                output, output_lse = attn_output, attn_lse
+            else:
+                out_tmp, lse_tmp = torch.empty_like(output), torch.empty_like(output_lse)
+                K.merge_states(output, output_lse, attn_output, attn_lse, out_tmp, lse_tmp)
+                output, output_lse = out_tmp, lse_tmp
+        return output, output_lse
+
+    def _forward_prefill(self, q, kv_c_normed, k_pe, kv_cache, attn_metadata, k_scale) -> torch.Tensor:
+        """Causal suffix attention merged with the chunked context (reference mla.py:452-483, 573-616)."""
+        prefill = attn_metadata.prefill
+        assert prefill is not None
+        if self.fp8_cache and prefill.chunked_context is not None:
+            raise NotImplementedError("chunked-context prefill over the fp8 cache is not implemented")
+        t, n = q.shape[0], self.num_heads
+        has_context = prefill.chunked_context is not None
+        q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
+        k_nope, v = self._kv_up(kv_c_normed)
+        cu_q = prefill.query_start_loc.to(torch.int32).contiguous()
+        output = torch.empty(t, n, self.v_head_dim, dtype=q.dtype, device=q.device)
+        output_lse = torch.empty(t, n, dtype=torch.float32, device=q.device) if has_context else None
+        K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
+                         output, output_lse)
+        if has_context:
+            ctx_out, ctx_lse = self._compute_prefill_context(q_nope, q_pe, kv_cache[0], kv_cache[1], attn_metadata, k_scale)
+            if ctx_out is not None:
+                merged = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q.device)
+                K.merge_states(ctx_out, ctx_lse, output, output_lse, merged)
+                output = merged
+        return output.to(torch.bfloat16).flatten(start_dim=-2)
+
+    # ---- decode ----
+    def _forward_decode(self, decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer=None) -> torch.Tensor:
+        """Absorbed paged decode; returns the head-major [N, T, 512] tensor of the reference (mla.py:781-804)."""
+        d = attn_metadata.decode
+        assert d is not None
+        t = decode_ql_nope.shape[0]
+        o = torch.empty(self.num_heads, t, self.kv_lora_rank, dtype=decode_ql_nope.dtype, device=decode_ql_nope.device)
+        kw = dict(q_len=d.q_len, query_start_loc=d.query_start_loc, max_seq_len=d.block_table.shape[1] * K.PAGE)
+        if self.fp8_cache:
+            K.decode_fp8(decode_ql_nope, decode_q_pe, kv_cache[0], d.block_table, d.seq_lens, self.scale,
+                         o.transpose(0, 1), **kw)
+        else:
+            K.decode(decode_ql_nope, decode_q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens, self.scale,
+                     o.transpose(0, 1), **kw)
+        return o
+
+    def forward(self, layer, q: torch.Tensor, k_c_normed: torch.Tensor, k_pe: torch.Tensor,
+                kv_cache: Tuple[torch.Tensor, ...], attn_metadata: NPUMLAMetadata,
+                output: Optional[torch.Tensor] = None, output_scale: Optional[torch.Tensor] = None,
+                output_block_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+        assert output is not None, "Output tensor must be provided."
+        if output_scale is not None or output_block_scale is not None:
+            raise NotImplementedError("fused output quantization is not yet supported for NPUMLAImpl")
+
+        if attn_metadata is None:
+            # profile run: reserve the worst-case up-projection scratch, zero the output (reference mla.py:825-842)
+            _ = torch.empty((self.chunked_prefill_workspace_size, self.num_heads,
+                             self.qk_nope_head_dim + self.v_head_dim), device=k_c_normed.device, dtype=k_c_normed.dtype)
+            return output.fill_(0)
+
+        num_actual_toks = attn_metadata.num_actual_tokens
+        assert isinstance(kv_cache, (list, tuple)), f"{type(kv_cache)=}."
+        want = 1 if self.fp8_cache else 2
+        assert len(kv_cache) == want, f"{len(kv_cache)=}."
+        assert all(isinstance(c, torch.Tensor) and c.numel() > 0 for c in kv_cache), \
+            f"{[getattr(c, 'shape', None) for c in kv_cache]}"
+
+        output_padded = output
+        assert (attn_metadata.num_decodes is not None and attn_metadata.num_prefills is not None
+                and attn_metadata.num_decode_tokens is not None)
+        has_decode = attn_metadata.num_decodes > 0
+        has_prefill = attn_metadata.num_prefills > 0
+        num_decode_tokens = attn_metadata.num_decode_tokens
+        decode_q = q[:num_decode_tokens]
+
+        # write the latent and rope rows of the new tokens (one launch)
+        if self.fp8_cache:
+            K.cache_write_fp8(k_c_normed, k_pe, attn_metadata.slot_mapping, kv_cache[0])
+        else:
+            K.cache_write(k_c_normed, k_pe, attn_metadata.slot_mapping, kv_cache[0], kv_cache[1])
+
+        if has_prefill:
+            output = output[:num_actual_toks, ...]
+            q = q[:num_actual_toks, ...]
+            k_c_normed = k_c_normed[:num_actual_toks, ...]
+            k_pe = k_pe[:num_actual_toks, ...]
+            output[num_decode_tokens:] = self._forward_prefill(
+                q[num_decode_tokens:], k_c_normed[num_decode_tokens:], k_pe[num_decode_tokens:], kv_cache, attn_metadata,
+                getattr(layer, "_k_scale", None))
+
+        if has_decode:
+            assert attn_metadata.decode is not None
+            decode_q_nope, decode_q_pe = decode_q.split([self.qk_nope_head_dim, self.qk_rope_head_dim], dim=-1)
+            # (B, N, P) -> (N, B, P) x (N, P, L) -> (N, B, L) -> (B, N, L) view
+            decode_ql_nope = torch.bmm(decode_q_nope.transpose(0, 1), self.W_UK_T).transpose(0, 1)
+            attn_out = self._forward_decode(decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer)
+            out_proj = self._v_up_proj(attn_out)
+            output[:out_proj.shape[0]].copy_(out_proj)
+        return output_padded

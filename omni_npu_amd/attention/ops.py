@@ -1,0 +1,72 @@
+"""HIP counterparts of the reference's torch helpers (src/omni_npu/attention/ops.py), same names and argument order.
+
+Every function launches a gfx950 kernel through the C-ABI; tensors must live on the GPU.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .. import kernels as K
+
+
+def gather_and_maybe_dequant_cache(
+    src_cache: Tuple[torch.Tensor, torch.Tensor],
+    dst: torch.Tensor,
+    block_table: torch.Tensor,
+    cu_seq_lens: torch.Tensor,
+    batch_size: int,
+    kv_cache_dtype: str,
+    scale: Optional[torch.Tensor],
+    seq_starts: Optional[torch.Tensor] = None,
+    total_rows: Optional[int] = None,
+) -> None:
+    """dst[cu[i]:cu[i+1]] = cat(nope, rope) rows of positions seq_starts[i] .. of sequence i
+    (reference ops.py:5-41).  Like the reference, ``kv_cache_dtype`` and ``scale`` are accepted and unused:
+    no dequantisation happens on this path."""
+    dev = dst.device
+    cu = cu_seq_lens.to(device=dev, dtype=torch.int32).contiguous()
+    st = None if seq_starts is None else seq_starts.to(device=dev, dtype=torch.int32).contiguous()
+    K.gather_paged(src_cache[0], src_cache[1], dst, block_table, cu, batch_size, st, total_rows)
+
+
+def merge_attn_states(
+    output: torch.Tensor,
+    prefix_output: torch.Tensor,
+    prefix_lse: torch.Tensor,
+    suffix_output: torch.Tensor,
+    suffix_lse: torch.Tensor,
+    output_lse: Optional[torch.Tensor] = None,
+) -> None:
+    """Two-way LSE merge of (T, N, D) outputs with (T, N, 1) log-sum-exps (reference ops.py:44-106)."""
+    assert output.dim() == 3, f"output should have 3 dimensions, but got shape {output.shape}."
+    assert prefix_lse.dim() == 3 and prefix_lse.size(-1) == 1, \
+        f"LSE should have 3 dimensions and the last should be 1, but got shape {prefix_lse.shape}."
+    K.merge_states(prefix_output, prefix_lse.float().contiguous(), suffix_output, suffix_lse.float().contiguous(),
+                   output, output_lse)
+
+
+def attention_update_torch(outs, lses):
+    """N-way merge (reference ops.py:109-141): outs [n, T, D] (or list), lses [n, T] -> (out fp32 [T, D], lse fp32 [T]).
+    Folded pairwise with the two-way merge kernel (the merge is associative)."""
+    if type(outs) is list:
+        assert type(lses) is list and len(outs) == len(lses)
+        outs = torch.stack(outs, dim=0)
+        lses = torch.stack(lses, dim=0)
+    assert outs.dim() == 3 and lses.dim() == 2
+    assert outs.size(0) == lses.size(0) and outs.size(1) == lses.size(1)
+    n, t, d = outs.shape
+    acc = outs[0].float().contiguous().view(t, 1, d)
+    acc_lse = lses[0].float().contiguous().view(t, 1)
+    for i in range(1, n):
+        nxt, nxt_lse = torch.empty_like(acc), torch.empty_like(acc_lse)
+        K.merge_states(acc, acc_lse, outs[i].float().contiguous().view(t, 1, d), lses[i].float().contiguous().view(t, 1),
+                       nxt, nxt_lse)
+        acc, acc_lse = nxt, nxt_lse
+    if n == 1:   # same conventions as the merge: +inf reads as -inf, an empty row is zeros
+        z, zl = torch.zeros_like(acc), torch.full_like(acc_lse, float("-inf"))
+        nxt, nxt_lse = torch.empty_like(acc), torch.empty_like(acc_lse)
+        K.merge_states(acc, acc_lse, z, zl, nxt, nxt_lse)
+        acc, acc_lse = nxt, nxt_lse
+    return acc.view(t, d), acc_lse.view(t)

@@ -120,8 +120,50 @@ __global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerPa
   }
 }
 
+// Per-row e4m3 quantisation of 128-wide bf16 rows (one fp32 scale = amax/448 per row, 1.0 for an all-zero row),
+// optionally scattered through a slot mapping into a paged fp8 cache + scale cache: the indexer-K write of
+// src/omni_npu/vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:116-121 with quantisation fused in, and
+// the query quantisation (no slot mapping).  One wavefront per row, lane l owns elements 2l, 2l+1.
+__global__ __launch_bounds__(256) void dsa_quant_rows_kernel(const __bf16* src, int64_t src_stride, int64_t rows,
+                                                             const int64_t* slots, uint8_t* dst8, int64_t d_sp, int64_t d_sr,
+                                                             float* dscale, int64_t s_sp, int32_t page_size,
+                                                             int64_t num_pages) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  int64_t slot = slots ? slots[r] : r;
+  if (slot < 0 || slot >= num_pages * page_size) return;
+  const int64_t pg = slot / page_size, off = slot - pg * page_size;
+  const bf16x2 v = *(const bf16x2*)(src + r * src_stride + lane * 2);
+  const float x0 = (float)v[0], x1 = (float)v[1];
+  float amax = fmaxf(fabsf(x0), fabsf(x1));
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+  const float scale = amax > 0.f ? amax / 448.f : 1.f;
+  const float y0 = fminf(fmaxf(x0 / scale, -448.f), 448.f), y1 = fminf(fmaxf(x1 / scale, -448.f), 448.f);
+  const int w = __builtin_amdgcn_cvt_pk_fp8_f32(y0, y1, 0, false);
+  *(uint16_t*)(dst8 + pg * d_sp + off * d_sr + lane * 2) = (uint16_t)(w & 0xFFFF);
+  if (lane == 0) dscale[pg * s_sp + off] = scale;
+}
+
 }  // namespace mlahip
 using namespace mlahip;
+
+extern "C" int dsa_quant_rows_fp8(const void* src, int64_t src_stride, int64_t rows, const int64_t* slot_mapping,
+                                  void* dst8, int64_t dst_page_stride_bytes, int64_t dst_row_stride_bytes,
+                                  float* dst_scale, int64_t scale_page_stride, int32_t page_size, int64_t num_pages,
+                                  hipStream_t stream) {
+  MLA_REQUIRE(src && dst8 && dst_scale, MLA_ERR_NULL, "dsa_quant_rows_fp8: null pointer argument");
+  MLA_REQUIRE(rows >= 0 && page_size >= 1 && num_pages >= 1 && src_stride % 2 == 0 && dst_row_stride_bytes >= 128 &&
+                  (uintptr_t)src % 4 == 0 && (uintptr_t)dst8 % 2 == 0 && dst_row_stride_bytes % 2 == 0 &&
+                  dst_page_stride_bytes % 2 == 0,
+              MLA_ERR_SHAPE, "dsa_quant_rows_fp8: rows=%lld page_size=%d", (long long)rows, page_size);
+  if (rows == 0) return MLA_OK;
+  hipLaunchKernelGGL(dsa_quant_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, (const __bf16*)src,
+                     src_stride, rows, slot_mapping, (uint8_t*)dst8, dst_page_stride_bytes, dst_row_stride_bytes, dst_scale,
+                     scale_page_stride, page_size, num_pages);
+  return check_launch("dsa_quant_rows_kernel");
+}
 
 extern "C" int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_t q_stride_h, const float* weights,
                                       int64_t w_stride_t, const float* q_scale, int64_t qs_stride_t, const void* k8_cache,

@@ -431,3 +431,36 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
                             ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
     _lib.check(rc, "mla_decode_fp8")
     return out
+
+
+def quant_rows_fp8(x: torch.Tensor, out8: torch.Tensor, out_scale: torch.Tensor,
+                   slot_mapping: Optional[torch.Tensor] = None) -> None:
+    """Per-row e4m3 quantisation of bf16 rows [R,128] (scale = amax/448).  Without ``slot_mapping``: out8 [R,128] (1-byte
+    dtype), out_scale fp32 [R].  With it: out8 is a paged cache [nblk,page,128] and out_scale [nblk,page]; row r goes to
+    flat slot slot_mapping[r] (negative slots skipped) - the fused indexer-K quantise-and-write."""
+    _need_cuda(x, out8, out_scale, slot_mapping)
+    lib = _lib.load()
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.shape[-1] != 128 or x2.dtype != torch.bfloat16 or x2.stride(-1) != 1 or out8.element_size() != 1 or \
+            out_scale.dtype != torch.float32 or out8.stride(-1) != 1:
+        raise TypeError("quant_rows_fp8: bf16 [R,128] in, 1-byte [.,128] and fp32 scales out")
+    if slot_mapping is None:
+        o8, sc = out8.reshape(-1, 128), out_scale.reshape(-1)
+        if o8.data_ptr() != out8.data_ptr() or o8.shape[0] < x2.shape[0] or sc.numel() < x2.shape[0] or not sc.is_contiguous():
+            raise ValueError("quant_rows_fp8: outputs must be contiguous and hold R rows")
+        rc = lib.dsa_quant_rows_fp8(x2.data_ptr(), x2.stride(0), x2.shape[0], None, o8.data_ptr(), 0, o8.stride(0),
+                                    sc.data_ptr(), 0, x2.shape[0], 1, _stream(x))
+    else:
+        if out8.dim() == 4 and out8.shape[2] == 1:
+            out8 = out8.squeeze(2)
+        if out8.dim() != 3 or out_scale.shape[:2] != out8.shape[:2]:
+            raise ValueError("quant_rows_fp8: paged outputs must be [nblk,page,128] and [nblk,page]")
+        sc = out_scale.reshape(out8.shape[0], out8.shape[1])
+        if sc.stride(-1) != 1:
+            raise ValueError("quant_rows_fp8: scale rows must be contiguous")
+        if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+            slot_mapping = slot_mapping.to(torch.int64).contiguous()
+        n = min(x2.shape[0], slot_mapping.numel())
+        rc = lib.dsa_quant_rows_fp8(x2.data_ptr(), x2.stride(0), n, slot_mapping.data_ptr(), out8.data_ptr(), out8.stride(0),
+                                    out8.stride(1), sc.data_ptr(), sc.stride(0), out8.shape[1], out8.shape[0], _stream(x))
+    _lib.check(rc, "dsa_quant_rows_fp8")
