@@ -19,7 +19,9 @@
 //
 // Each workgroup writes a normalised fp32 partial and its log-sum-exp; mla_splitkv_reduce_kernel folds the
 // splits with the N-way merge of src/omni_npu/attention/ops.py:109-141 and writes bf16.
+#include <cstdlib>
 #include "mla_common.hpp"
+#include "decode_v2_params.hpp"
 
 namespace mlahip {
 
@@ -70,7 +72,7 @@ struct DecodeParams {
   int32_t batch, max_q_len, num_heads;
   int64_t num_pages;
   float scale_log2;              // scale * log2(e)
-  float* o_part;                 // [B*S, R_max, 512]
+  _Float16* o_part;              // [B*S, R_max, 512] fp16, normalised
   float* lse_part;               // [B*S, R_max]   (natural log)
   int32_t num_splits;
   // sparse variant: the keys of "sequence" b are the flat cache rows sparse_rows[b, 0 .. seq_lens[b])
@@ -399,21 +401,23 @@ __global__ __launch_bounds__(256, 1) void mla_decode_bf16_kernel(const DecodePar
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (row < r_max) {
     if (half == 0) p.lse_part[part_row] = l_tot > 0.f ? (m_run + fast_log2(l_tot)) * kLn2 : -INFINITY;
-    float* op = p.o_part + part_row * kDNope + 4 * half;
+    _Float16* op = p.o_part + part_row * kDNope + 4 * half;
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 #pragma unroll
     for (int db = 0; db < 16; db++)
 #pragma unroll
       for (int rg = 0; rg < 4; rg++) {
-        f32x4 v = {acc[db][rg * 4 + 0] * inv, acc[db][rg * 4 + 1] * inv, acc[db][rg * 4 + 2] * inv,
-                   acc[db][rg * 4 + 3] * inv};
-        *(f32x4*)(op + db * 32 + rg * 8) = v;
+        h4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = (_Float16)(acc[db][rg * 4 + e] * inv);
+        *(h4*)(op + db * 32 + rg * 8) = v;
       }
   }
 }
 
 // N-way merge over the splits (src/omni_npu/attention/ops.py:109-141): one wavefront per query row.
 struct ReduceParams {
-  const float* o_part; const float* lse_part;
+  const _Float16* o_part; const float* lse_part;
   const int32_t* qsl;
   int32_t batch, max_q_len, num_heads, num_splits;
   __bf16* out; int64_t out_st, out_sh;
@@ -442,27 +446,25 @@ __global__ __launch_bounds__(256) void mla_splitkv_reduce_kernel(const ReducePar
     m = fmaxf(m, l);
   }
   float tot = 0.f;
-  f32x4 a0 = {0, 0, 0, 0}, a1 = {0, 0, 0, 0};
+  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if (m != -INFINITY) {
     for (int s = 0; s < p.num_splits; s++) {
       float l = p.lse_part[base + (int64_t)s * r_max];
       if (l == INFINITY || l == -INFINITY) continue;         // empty split: its partial is never read
       const float w = __expf(l - m);
       tot += w;
-      const float* o = p.o_part + (base + (int64_t)s * r_max) * kDNope;
-      f32x4 v0 = *(const f32x4*)(o + lane * 4);
-      f32x4 v1 = *(const f32x4*)(o + 256 + lane * 4);
-      a0 += v0 * w;
-      a1 += v1 * w;
+      const h8 v = *(const h8*)(p.o_part + (base + (int64_t)s * r_max) * kDNope + lane * 8);
+#pragma unroll
+      for (int e = 0; e < 8; e++) a[e] += (float)v[e] * w;
     }
   }
   const float inv = tot > 0.f ? 1.f / tot : 0.f;
   __bf16* out = p.out + (int64_t)(q0 + t_local) * p.out_st + (int64_t)head * p.out_sh;
-  bf16x4 o0, o1;
+  bf16x8 o8;
 #pragma unroll
-  for (int e = 0; e < 4; e++) { o0[e] = (__bf16)(a0[e] * inv); o1[e] = (__bf16)(a1[e] * inv); }
-  *(bf16x4*)(out + lane * 4) = o0;
-  *(bf16x4*)(out + 256 + lane * 4) = o1;
+  for (int e = 0; e < 8; e++) o8[e] = (__bf16)(a[e] * inv);
+  *(bf16x8*)(out + lane * 8) = o8;
   if (p.lse_out && lane == 0)
     p.lse_out[(int64_t)(q0 + t_local) * p.lse_st + head] = tot > 0.f ? __logf(tot) + m : -INFINITY;
 }
@@ -474,7 +476,7 @@ using namespace mlahip;
 extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits) {
   if (batch <= 0 || max_q_len <= 0 || num_heads <= 0 || num_splits <= 0) return 0;
   const size_t rows = (size_t)batch * num_splits * max_q_len * num_heads;
-  return rows * kDNope * sizeof(float) + rows * sizeof(float);
+  return rows * kDNope * sizeof(_Float16) + rows * sizeof(float);   // fp16 partials + fp32 log-sum-exps
 }
 
 static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
@@ -517,8 +519,8 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   p.seq_lens = seq_lens; p.qsl = query_start_loc;
   p.batch = batch; p.max_q_len = max_q_len; p.num_heads = num_heads; p.num_pages = num_pages;
   p.scale_log2 = scale * kLog2e;
-  p.o_part = (float*)workspace;
-  p.lse_part = (float*)workspace + rows * kDNope;
+  p.o_part = (_Float16*)workspace;
+  p.lse_part = (float*)((_Float16*)workspace + rows * kDNope);
   p.num_splits = num_splits;
   p.sparse_rows = sparse_rows; p.sparse_stride = sparse_stride; p.page_size = page_size;
 
@@ -537,6 +539,17 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
     attr_set = true;
   }
   dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
+  static const bool use_v1 = getenv("MLA_DECODE_V1") != nullptr;     // first-generation kernel, for comparisons
+  if (!fp8 && !use_v1) {
+    DecodeV2Params v;
+    v.q_nope = p.q_nope; v.qn_st = p.qn_st; v.qn_sh = p.qn_sh; v.q_rope = p.q_rope; v.qr_st = p.qr_st; v.qr_sh = p.qr_sh;
+    v.nope = p.nope; v.nope_sp = p.nope_sp; v.nope_sr = p.nope_sr; v.rope = p.rope; v.rope_sp = p.rope_sp; v.rope_sr = p.rope_sr;
+    v.block_table = p.block_table; v.bt_stride = p.bt_stride; v.max_blocks = p.max_blocks; v.seq_lens = p.seq_lens; v.qsl = p.qsl;
+    v.batch = p.batch; v.max_q_len = p.max_q_len; v.num_heads = p.num_heads; v.num_pages = p.num_pages;
+    v.scale_log2 = p.scale_log2; v.o_part = p.o_part; v.lse_part = p.lse_part; v.num_splits = p.num_splits;
+    v.sparse_rows = p.sparse_rows; v.sparse_stride = p.sparse_stride; v.page_size = p.page_size;
+    return launch_decode_v2(v, sparse_rows != nullptr, grid, stream);
+  }
   if (fp8) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeFp8>, grid, dim3(256), kFp8LdsB, stream, p);
   else if (sparse_rows) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeSparse>, grid, dim3(256), kDecodeLdsB, stream, p);
   else hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeDense>, grid, dim3(256), kDecodeLdsB, stream, p);
@@ -566,9 +579,9 @@ extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes,
   MLA_REQUIRE(workspace && out, MLA_ERR_NULL, "mla_splitkv_reduce: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1, MLA_ERR_SHAPE,
               "mla_splitkv_reduce: batch=%d max_q_len=%d num_heads=%d num_splits=%d", batch, max_q_len, num_heads, num_splits);
-  MLA_REQUIRE((out_stride_t % 4 == 0) && (out_stride_h % 4 == 0) && ((uintptr_t)out % 8 == 0) &&
+  MLA_REQUIRE((out_stride_t % 8 == 0) && (out_stride_h % 8 == 0) && ((uintptr_t)out % 16 == 0) &&
                   ((uintptr_t)workspace % 16 == 0),
-              MLA_ERR_SHAPE, "mla_splitkv_reduce: output rows must be 8-byte aligned");
+              MLA_ERR_SHAPE, "mla_splitkv_reduce: output rows must be 16-byte aligned");
   if (batch == 0) return MLA_OK;
   const size_t need = mla_decode_workspace_bytes(batch, max_q_len, num_heads, num_splits);
   MLA_REQUIRE(workspace_bytes >= need, MLA_ERR_WORKSPACE, "mla_splitkv_reduce: workspace %zu bytes < required %zu",
@@ -576,7 +589,8 @@ extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes,
   const int r_max = max_q_len * num_heads;
   const size_t rows = (size_t)batch * num_splits * r_max;
   ReduceParams rp;
-  rp.o_part = (const float*)workspace; rp.lse_part = (const float*)workspace + rows * kDNope; rp.qsl = query_start_loc;
+  rp.o_part = (const _Float16*)workspace; rp.lse_part = (const float*)((const _Float16*)workspace + rows * kDNope);
+  rp.qsl = query_start_loc;
   rp.batch = batch; rp.max_q_len = max_q_len; rp.num_heads = num_heads; rp.num_splits = num_splits;
   rp.out = (__bf16*)out; rp.out_st = out_stride_t; rp.out_sh = out_stride_h;
   rp.lse_out = lse_out; rp.lse_st = num_heads;

@@ -1,0 +1,511 @@
+// Absorbed-MLA paged decode, second-generation kernel for the bf16 cache (dense and row-list sources).
+//
+// Same contract as mla_decode_bf16_kernel in decode.hip (reference call:
+// src/omni_npu/attention/backends/mla.py:781-804); what changed is how a workgroup spends its LDS and MFMA issue slots.
+//
+// A wavefront can issue one LDS instruction per ~17 clocks, and a transposed read delivers only 8 bytes per lane, so
+// "every wave reads all of V^T for its own 32 rows" (two transposed reads per MFMA) makes the P.V phase LDS-issue bound.
+// Here the two products are partitioned differently:
+//   S^T = K Q^T      wave w owns query rows 32w..32w+31 (its 576-wide query stays in registers), all 32 tokens of a block;
+//   O^T += V^T P^T   wave w owns output columns d in [128w, 128w+128) for ALL 128 rows: a V^T fragment is read once and
+//                    feeds four MFMAs (one per row group), and the four P^T blocks (2 KiB each, bf16) plus the rescale
+//                    factors travel through LDS once per block.
+// Per 32 tokens a wave issues 36 + 16 + 8 + ~4 LDS instructions instead of 100, for the same 68 MFMAs.
+//
+// Pipeline (one barrier per 32-token block):  body i = [barrier] QK(i+1) | PV(i) overlapped with softmax(i+1) | publish P(i+1).
+// Blocks live in 4 nope buffers (32 KiB) and 3 rope buffers (4 KiB); the copy of block i+3 is issued right after barrier i, so
+// two blocks are always in flight.
+//
+// No accumulator rescaling in the steady state.  The 256 output accumulators live in the accumulation register file, which
+// vector ALU instructions cannot touch, so the usual online-softmax rescale would cost three instructions per element.
+// Instead every row fixes its reference m_ref at the maximum of the first block in which it sees a key and uses
+// P = exp2(s - m_ref) from then on: bf16 and fp32 share one exponent range, so P may grow to 2^100 without loss of
+// relative precision.  If a later score exceeds m_ref by more than 100 (log2 units; e^69 in weight) the row raises a flag
+// that travels with P, and the whole workgroup restarts its split with the row maxima seen so far as references.  Each
+// restart raises a reference by more than 100, so at most a few can happen; realistic logits never trigger one.
+// Partials are written as fp16 (normalised values, |o| <= max|V|) through an LDS transpose so that global stores are row
+// contiguous; log-sum-exps as fp32.
+#include "decode_v2_params.hpp"
+#include <type_traits>
+
+namespace mlahip {
+
+#ifndef MLA_V2_QK_AHEAD
+#define MLA_V2_QK_AHEAD 3
+#endif
+#ifndef MLA_V2_PV_AHEAD
+#define MLA_V2_PV_AHEAD 2
+#endif
+constexpr int kQkAheadV2 = MLA_V2_QK_AHEAD, kPvAheadV2 = MLA_V2_PV_AHEAD;   // LDS read-ahead depth, in fragments
+constexpr int kBlk = 32;                                   // tokens per block
+constexpr int kV2NopeBufB = kBlk * 1024;                   // 32768
+constexpr int kV2RopeBufB = kBlk * 128;                    // 4096
+constexpr int kV2RopeOff = 4 * kV2NopeBufB;                // 131072
+constexpr int kV2POff = kV2RopeOff + 3 * kV2RopeBufB;      // 143360
+constexpr int kV2PBufB = 8192;                             // 4 row groups x 2 k-blocks x 64 lanes x 16 B
+constexpr int kV2AOff = kV2POff + 2 * kV2PBufB;            // 159744: rescale factors, 2 x 512 B
+constexpr int kV2LdsB = kV2AOff + 2 * 512;                 // 160768
+constexpr float kRestartThreshold = 100.f;                 // log2 units above a row's reference
+
+__device__ __forceinline__ int v2_swz_nope(int r) {
+  int r0 = r & 1, r1 = (r >> 1) & 1, r2 = (r >> 2) & 1, r3 = (r >> 3) & 1;
+  return ((r1 ^ r3) << 3) | (r0 << 2) | (r1 << 1) | r2;
+}
+__device__ __forceinline__ int v2_swz_rope(int r) {
+  int r0 = r & 1, r1 = (r >> 1) & 1, r2 = (r >> 2) & 1, r3 = (r >> 3) & 1;
+  return ((r0 ^ r3) << 2) | (r1 << 1) | r2;
+}
+
+
+// value of the same lane index in the other half of the wavefront, combined with max / add (one VALU swap, no LDS)
+__device__ __forceinline__ float half_max(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+__device__ __forceinline__ float half_sum(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
+typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
+
+template <bool kSparse>
+__global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Params p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int h32 = lane & 31;
+  const int half = lane >> 5;
+  const int split = blockIdx.x, b = blockIdx.y, grp = blockIdx.z;
+
+  const int L = p.seq_lens[b];
+  int q0, qlen;
+  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
+  qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
+  const int rows = qlen * p.num_heads;
+  const int r_max = p.max_q_len * p.num_heads;
+  if (grp * 128 >= r_max) return;
+
+  // this lane's query row for QK / softmax (row group = wave)
+  const int row = grp * 128 + wave * 32 + h32;
+  const bool row_ok = row < rows && L > 0;
+  const int t_local = row / p.num_heads;
+  const int head = row - t_local * p.num_heads;
+  int limit = row_ok ? (L - qlen + t_local + 1) : 0;         // keys [0, limit) are visible to this row
+  limit = limit < 0 ? 0 : limit;
+  const int64_t part_base = ((int64_t)b * p.num_splits + split) * r_max + grp * 128;   // + row index in the group
+
+  // token range of this split, in 32-token blocks (split boundaries on 64-token multiples, as the fp8 kernel)
+  const int tiles_total = (L + 63) / 64;
+  const int tps = (tiles_total + p.num_splits - 1) / p.num_splits;
+  const int blk_begin = split * tps * 2;
+  int blk_end = blk_begin + tps * 2;
+  const int blks_total = (L + kBlk - 1) / kBlk;
+  blk_end = blk_end < blks_total ? blk_end : blks_total;
+
+  if (blk_begin >= blk_end || grp * 128 >= rows) {
+    if (row < r_max && half == 0) p.lse_part[part_base + wave * 32 + h32] = -INFINITY;
+    return;
+  }
+  const int nb = blk_end - blk_begin;
+  const uint32_t lds0 = lds_addr_of(lds);
+
+  // ---- global -> LDS copies: 9 per lane and block (8 nope rows of 1 KiB per wave, one rope instruction of 8 rows) ----
+  // Row r of a block goes to nope buffer row r (granule g at position g ^ swz(r)) and rope buffer row r.  All addresses
+  // are a scalar base plus a per-lane 32-bit offset that does not change from block to block.
+  uint32_t dma_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) dma_off[j] = (uint32_t)((lane ^ v2_swz_nope((wave * 4 + j) & 15)) << 4);
+  const uint32_t rope_off = (uint32_t)(((lane & 7) ^ v2_swz_rope((wave * 8 + (lane >> 3)) & 15)) << 4);
+  const uint32_t n_sr2 = (uint32_t)p.nope_sr * 2u, r_sr2 = (uint32_t)p.rope_sr * 2u;       // row strides in bytes
+  const uint32_t rope_voff = (uint32_t)(lane >> 3) * r_sr2 + rope_off;                      // full blocks: row 8*wave + lane/8
+
+  // dense source: the page of the block being copied and the next one are kept in scalar registers, so the block-table
+  // load is never waited for in the loop
+  ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (kSparse ? 0 : (int64_t)b * p.bt_stride);
+  ConstI32Ptr srows = (ConstI32Ptr)(p.sparse_rows) + (kSparse ? (int64_t)b * p.sparse_stride : 0);
+  const int64_t max_row = p.num_pages * p.page_size - 1;
+  auto load_page = [&](int page) -> int64_t {
+    page = page < p.max_blocks ? page : p.max_blocks - 1;
+    int64_t pg = bt[page];
+    return pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
+  };
+  int page_cur = 0;
+  int64_t pg_cur = 0, pg_nxt = 0;
+  auto issue_reset = [&]() {
+    if constexpr (!kSparse) {
+      page_cur = blk_begin >> 2;
+      pg_cur = load_page(page_cur);
+      pg_nxt = load_page(page_cur + 1);
+    }
+  };
+  auto issue_block = [&](int blk) {
+    const int tok0 = blk * kBlk;
+    const int last = L - 1 - tok0;                            // last valid row of the block (>= 0)
+    const uint32_t nbuf = lds0 + (blk & 3) * kV2NopeBufB;
+    const uint32_t rbuf = lds0 + kV2RopeOff + (blk % 3) * kV2RopeBufB;
+    if constexpr (kSparse) {
+      const char* nope = (const char*)p.nope;
+      const char* rope = (const char*)p.rope;
+      auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
+      if (last >= kBlk - 1) {
+        // full block: the 16 row numbers this wave needs arrive as three scalar vector loads
+        typedef int32_t i4 __attribute__((ext_vector_type(4)));
+        typedef int32_t i8 __attribute__((ext_vector_type(8)));
+        const i4 ra = *(__attribute__((address_space(4))) const i4*)(srows + tok0 + wave * 4);
+        const i4 rb = *(__attribute__((address_space(4))) const i4*)(srows + tok0 + 16 + wave * 4);
+        const i8 rr = *(__attribute__((address_space(4))) const i8*)(srows + tok0 + wave * 8);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          dma16_sv(nope + clampi(ra[j]) * n_sr2, dma_off[j], nbuf + (wave * 4 + j) * 1024);
+          dma16_sv(nope + clampi(rb[j]) * n_sr2, dma_off[j], nbuf + (16 + wave * 4 + j) * 1024);
+        }
+        int32_t mine = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) mine = (lane >> 3) == j ? rr[j] : mine;
+        dma16_v(rope + clampi(mine) * r_sr2 + rope_off, rbuf + wave * 1024);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const int r = q * 16 + wave * 4 + j;
+            const int re = r < last ? r : last;               // rows past the end re-read the last valid row
+            dma16_sv(nope + clampi(srows[tok0 + re]) * n_sr2, dma_off[j], nbuf + r * 1024);
+          }
+        int32_t mine = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const int r = wave * 8 + j;
+          const int32_t sj = srows[tok0 + (r < last ? r : last)];
+          mine = (lane >> 3) == j ? sj : mine;
+        }
+        dma16_v(rope + clampi(mine) * r_sr2 + rope_off, rbuf + wave * 1024);
+      }
+    } else {
+      const int page = blk >> 2;
+      if (page != page_cur) { page_cur = page; pg_cur = pg_nxt; pg_nxt = load_page(page + 1); }
+      const uint32_t row0 = (uint32_t)(blk & 3) * kBlk;
+      const char* np = (const char*)p.nope + pg_cur * p.nope_sp * 2 + (uint64_t)row0 * n_sr2;
+      const char* rp = (const char*)p.rope + pg_cur * p.rope_sp * 2 + (uint64_t)row0 * r_sr2;
+      if (last >= kBlk - 1) {
+        const char* a0 = np + (uint64_t)(wave * 4) * n_sr2;
+        const char* a1 = a0 + (uint64_t)n_sr2 * 16;
+        const uint32_t l0 = nbuf + wave * 4096;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          dma16_sv(a0, dma_off[j], l0 + j * 1024);
+          dma16_sv(a1, dma_off[j], l0 + 16384 + j * 1024);
+          a0 += n_sr2;
+          a1 += n_sr2;
+        }
+        dma16_sv(rp + (uint64_t)(wave * 8) * r_sr2, rope_voff, rbuf + wave * 1024);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const int r = q * 16 + wave * 4 + j;
+            const int re = r < last ? r : last;               // rows past the end re-read the last valid row
+            dma16_sv(np + (uint64_t)re * n_sr2, dma_off[j], nbuf + r * 1024);
+          }
+        const int r = wave * 8 + (lane >> 3);
+        const int re = r < last ? r : last;
+        dma16_sv(rp, (uint32_t)re * r_sr2 + rope_off, rbuf + wave * 1024);
+      }
+    }
+  };
+  auto issue_first_three = [&]() {
+    issue_reset();
+#pragma unroll 1
+    for (int j = 0; j < 3 && j < nb; j++) issue_block(blk_begin + j);
+  };
+
+  // ---- prologue: query loads first (so that the explicit vmcnt waits below count only LDS copies), then three blocks in flight ----
+  bf16x8 qf[36];
+  {
+    const int64_t tq = row_ok ? (q0 + t_local) : q0;
+    const int64_t hq = row_ok ? head : 0;
+    const __bf16* qn = p.q_nope + tq * p.qn_st + hq * p.qn_sh + half * 8;
+    const __bf16* qr = p.q_rope + tq * p.qr_st + hq * p.qr_sh + half * 8;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int kk = 0; kk < 32; kk++) { bf16x8 v = *(const bf16x8*)(qn + kk * 16); qf[kk] = row_ok ? v : zero; }
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) { bf16x8 v = *(const bf16x8*)(qr + kk * 16); qf[32 + kk] = row_ok ? v : zero; }
+#pragma unroll
+    for (int kk = 0; kk < 36; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
+  }
+
+  f32x16 acc[4][4];                                          // [d block of this wave's slice][row group]
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  float m_ref = -INFINITY;       // this row's softmax reference (log2 domain), fixed once finite
+  float m_seen = -INFINITY;      // largest score seen so far (reference of a restart)
+  float l_run = 0.f;
+
+  // ---- per-lane LDS offsets ----
+  // The swizzles are XORs confined to bits 4..7 of a byte offset whose other low bits are zero, so one base register
+  // per access pattern plus an XOR with a compile-time constant reaches every fragment (registers are the scarce
+  // resource here: a single spilled value would be reloaded with a vector-memory wait that also waits for the LDS copies).
+  const int fk = v2_swz_nope(h32 & 15), fr = v2_swz_rope(h32 & 15);
+  const uint32_t kbase = (uint32_t)(h32 * 1024 + ((half ^ fk) << 4));                 // ^ (j << 5), + (kk/8)*256, + buffer
+  const uint32_t rbase = (uint32_t)(kV2RopeOff + h32 * 128 + ((half ^ fr) << 4));     // ^ (j << 5), + buffer
+  const int g16 = lane >> 4, j16 = lane & 15;
+  const int v_row = 4 * (g16 >> 1) + (j16 >> 2);              // + 8*rd + 16*kb
+  const int v_cl = 2 * (g16 & 1) + ((j16 & 3) >> 1);
+  const int v_in = (j16 & 1) * 8;
+  uint32_t vbase[2];                                          // [rd]: ^ (db << 6), + kb*16384, + buffer
+#pragma unroll
+  for (int rd = 0; rd < 2; rd++) {
+    const int rr = v_row + 8 * rd;
+    vbase[rd] = (uint32_t)(rr * 1024 + v_in + wave * 256 + ((v_cl ^ v2_swz_nope(rr & 15)) << 4));
+  }
+  const int p_w_off = kV2POff + (wave * 2 * 64 + lane) * 16;  // + kb*1024 + parity*8192 : this wave's P^T fragments
+  const int p_r_off = kV2POff + lane * 16;                    // + (rg*2 + kb)*1024 + parity*8192
+  const int a_r_off = kV2AOff + h32 * 16;                     // + parity*512: restart flags of rows (rg, h32), 4 floats
+  const int a_w_off = kV2AOff + h32 * 16 + wave * 4;
+
+  // S^T for block `blk`.  The K fragments are read with hand-placed LDS instructions, kQkAheadV2 fragments ahead of the
+  // MFMA that consumes them, and explicit lgkmcnt waits: left to itself the compiler funnels every fragment through one
+  // register quad and waits for each read in full, which exposes the whole LDS latency 36 times per block.  (LDS reads
+  // return in order, so compiler-issued reads around this section only make its own waits stricter, never wrong.)
+  auto qk_block = [&](int blk, f32x16& s) {
+    const uint32_t nb32 = lds0 + (blk & 3) * kV2NopeBufB + kbase;     // buffers are 4 KiB aligned: the XORs below stay exact
+    const uint32_t rb32 = lds0 + (blk % 3) * kV2RopeBufB + rbase;
+    bf16x8 ka[kQkAheadV2];
+#define MLA_K_READ(dst, kk)                                                                                         \
+    do {                                                                                                            \
+      if ((kk) < 32) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(nb32 ^ (uint32_t)(((kk) & 7) << 5)), "i"(((kk) >> 3) * 256)); \
+      else asm volatile("ds_read_b128 %0, %1" : "=v"(dst) : "v"(rb32 ^ (uint32_t)(((kk) & 3) << 5)));              \
+    } while (0)
+#pragma unroll
+    for (int i = 0; i < kQkAheadV2; i++) MLA_K_READ(ka[i], i);
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[r] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < 36; kk++) {
+      // wait until fragment kk has landed: at most min(kQkAheadV2 - 1, 35 - kk) younger reads may still be in flight
+      constexpr int D = kQkAheadV2;
+      const int younger = (36 - 1 - kk) < (D - 1) ? (36 - 1 - kk) : (D - 1);
+      if (younger >= 7) asm volatile("s_waitcnt lgkmcnt(7)" : "+v"(ka[kk % D]));
+      else if (younger == 6) asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(ka[kk % D]));
+      else if (younger == 5) asm volatile("s_waitcnt lgkmcnt(5)" : "+v"(ka[kk % D]));
+      else if (younger == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(ka[kk % D]));
+      else if (younger == 3) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(ka[kk % D]));
+      else if (younger == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(ka[kk % D]));
+      else if (younger == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(ka[kk % D]));
+      else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ka[kk % D]));
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk % D], qf[kk], s, 0, 0, 0);
+      if (kk + D < 36) MLA_K_READ(ka[kk % D], kk + D);
+    }
+#undef MLA_K_READ
+    asm volatile("" : "+v"(s));
+  };
+
+  // Softmax of block `blk` from raw scores s, cut into eight straight-line steps so that it can be interleaved with the
+  // P.V MFMAs of the previous block (step k is called after the k-th group of four MFMAs; the MFMAs run 32 clocks each
+  // while the vector ALU is otherwise idle).  The row maximum is taken over all 32 scores of the block, visible or not:
+  // it only serves as a reference, and any finite reference within 2^100 of the true maximum is as good as another.
+  struct SoftmaxState { float neg_ref, flag; int rel; bf16x8 pb[2]; float psum; };
+  auto softmax_step = [&](int step, int blk, f32x16& s, SoftmaxState& st) {
+    if (step == 0) {
+      float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+      for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(s[r], s[r + 1]));
+      mx = half_max(mx) * p.scale_log2;
+      m_seen = fmaxf(m_seen, mx);
+      if (m_ref == -INFINITY) m_ref = mx;                    // the first block fixes the reference
+      st.flag = mx > m_ref + kRestartThreshold ? -1.f : 1.f; // -1 asks the workgroup to restart with better references
+      st.neg_ref = -m_ref;
+      st.rel = row_ok ? limit - blk * kBlk - 4 * half : 0;   // score r is visible iff 8*(r/4) + r%4 < rel
+      st.psum = 0.f;
+    } else if (step <= 4) {
+#pragma unroll
+      for (int r = 4 * (step - 1); r < 4 * step; r++) {
+        // an overflow to +inf can only happen past the restart threshold, and a restart discards everything accumulated
+        const float e = fast_exp2(__builtin_fmaf(s[r], p.scale_log2, st.neg_ref));
+        s[r] = (8 * (r >> 2) + (r & 3)) < st.rel ? e : 0.f;
+      }
+    } else if (step == 5) {
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.pb[kb][e] = (__bf16)s[kb * 8 + e];
+    } else if (step == 6) {
+      // the row sum uses the ROUNDED probabilities: numerator and denominator then carry the same weights, so the
+      // result is an exact convex combination of cache rows
+#pragma unroll
+      for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) st.psum += (float)st.pb[kb][e];
+    } else {
+      l_run += st.psum;
+      char* base = lds + (blk & 1) * kV2PBufB;
+      *(bf16x8*)(base + p_w_off) = st.pb[0];
+      *(bf16x8*)(base + p_w_off + 1024) = st.pb[1];
+      if (half == 0) *(float*)(lds + (blk & 1) * 512 + a_w_off) = st.flag;
+    }
+  };
+
+  // O^T += V^T P^T for block `blk`: this wave's 128 output columns for all four row groups; with kFused the softmax of
+  // block blk+1 (scores s) rides along
+  auto pv_block = [&](int blk, auto fused, f32x16& s) {
+    constexpr bool kFused = decltype(fused)::value;
+    SoftmaxState st;
+    const char* pbase = lds + (blk & 1) * kV2PBufB;
+    const char* vb = lds + (blk & 3) * kV2NopeBufB;
+    auto v_frag = [&](int stp) -> bf16x8 {                    // stp = 4*kb + db
+      const int db = stp & 3, kb = stp >> 2;
+      bf16x4 lo = lds_read_tr16(vb + kb * 16 * 1024 + (vbase[0] ^ (uint32_t)(db << 6)));
+      bf16x4 hi = lds_read_tr16(vb + kb * 16 * 1024 + (vbase[1] ^ (uint32_t)(db << 6)));
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    bf16x8 va[kPvAheadV2];
+#pragma unroll
+    for (int j = 0; j < kPvAheadV2; j++) va[j] = v_frag(j);
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+      bf16x8 pr[4];
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) pr[rg] = *(const bf16x8*)(pbase + p_r_off + (rg * 2 + kb) * 1024);
+#pragma unroll
+      for (int db = 0; db < 4; db++) {
+        const int stp = kb * 4 + db;
+        const bf16x8 a = va[stp % kPvAheadV2];
+        if (stp + kPvAheadV2 < 8) va[stp % kPvAheadV2] = v_frag(stp + kPvAheadV2);
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++)
+          acc[db][rg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pr[rg], acc[db][rg], 0, 0, 0);
+        if constexpr (kFused) softmax_step(stp, blk + 1, s, st);
+      }
+    }
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) asm volatile("" : "+a"(acc[db][rg]));     // output accumulators stay in AGPRs
+  };
+  auto flags_ask_restart = [&](int blk) -> bool {
+    const f32x4 fl = *(const f32x4*)(lds + (blk & 1) * 512 + a_r_off);
+    // every wave reads the same 128 flags: a uniform decision
+    return __builtin_amdgcn_ballot_w64(fl[0] < 0.f || fl[1] < 0.f || fl[2] < 0.f || fl[3] < 0.f) != 0;
+  };
+
+  bool restart = false;
+  do {
+    if (restart) {
+      // a row outgrew its reference: drain, take the maxima seen so far as references, clear the sums, start over
+      MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      m_ref = m_seen;
+      l_run = 0.f;
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      restart = false;
+    }
+    issue_first_three();
+    // ---- block 0: QK, softmax, publish ----
+    {
+      if (nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      f32x16 s;
+      SoftmaxState st;
+      qk_block(blk_begin, s);
+#pragma unroll
+      for (int step = 0; step < 8; step++) softmax_step(step, blk_begin, s, st);
+    }
+    // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
+    for (int i = 0; i + 1 < nb; i++) {
+      const int blk = blk_begin + i;
+      // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
+      if (i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      if (flags_ask_restart(blk)) { restart = true; break; }
+      if (i + 3 < nb) issue_block(blk + 3);
+      f32x16 s;
+      qk_block(blk + 1, s);
+      pv_block(blk, std::true_type{}, s);
+    }
+    if (!restart) {
+      const int blk = blk_end - 1;
+      MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      if (flags_ask_restart(blk)) restart = true;
+      else { f32x16 s; pv_block(blk, std::false_type{}, s); }
+    }
+  } while (restart);
+
+  // ---- epilogue ----
+  lds_barrier();                                              // all PV done; tile buffers and P buffers are free
+  {
+    const float l_tot = half_sum(l_run);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (half == 0) {
+      *(float*)(lds + a_w_off) = inv;
+      if (row < r_max) p.lse_part[part_base + wave * 32 + h32] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
+    }
+  }
+  lds_barrier();
+  const f32x4 inv4 = *(const f32x4*)(lds + a_r_off);
+  // transpose through this wave's private 32 KiB (nope buffer `wave`): two rounds of 64 rows x 128 columns, fp16
+  char* stage = lds + wave * kV2NopeBufB;
+#pragma unroll
+  for (int round = 0; round < 2; round++) {
+#pragma unroll
+    for (int rgl = 0; rgl < 2; rgl++) {
+      const int rg = round * 2 + rgl;
+      const int srow = rgl * 32 + h32;                        // row inside the staging area, 256 B per row (128 fp16)
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+          typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+          h4 v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] = (_Float16)(acc[db][rg][q4 * 4 + e] * inv4[rg]);
+          const int g8 = db * 8 + q4 * 2 + half;              // 8-byte granule index in the row (32 per row)
+          *(h4*)(stage + srow * 256 + ((g8 ^ (srow & 31)) << 3)) = v;
+        }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // read back: a half-wave reads one row (32 lanes x 8 B = 256 B), 2 rows per instruction, 32 instructions
+#pragma unroll 4
+    for (int it = 0; it < 32; it++) {
+      const int srow = it * 2 + half;
+      const u32x2 v = *(const u32x2*)(stage + srow * 256 + ((h32 ^ (srow & 31)) << 3));
+      const int rg = round * 2 + (srow >> 5);
+      const int r_in_grp = rg * 32 + (srow & 31);
+      if (grp * 128 + r_in_grp < r_max)
+        *(u32x2*)(p.o_part + (part_base + r_in_grp) * kDNope + wave * 128 + h32 * 4) = v;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+}
+
+int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_v2_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kV2LdsB);
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute((const void*)mla_decode_v2_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kV2LdsB);
+    if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_decode_bf16: cannot reserve %d bytes of LDS: %s", kV2LdsB,
+                                     hipGetErrorString(e));
+    attr_set = true;
+  }
+  if (sparse) hipLaunchKernelGGL(mla_decode_v2_kernel<true>, grid, dim3(256), kV2LdsB, stream, p);
+  else hipLaunchKernelGGL(mla_decode_v2_kernel<false>, grid, dim3(256), kV2LdsB, stream, p);
+  return check_launch("mla_decode_v2_kernel");
+}
+
+}  // namespace mlahip

@@ -1,0 +1,27 @@
+// Parameters and launcher of the second-generation absorbed-MLA decode kernel (decode_v2.hip).
+#pragma once
+#include "mla_common.hpp"
+
+namespace mlahip {
+
+struct DecodeV2Params {
+  const __bf16* q_nope; int64_t qn_st, qn_sh;
+  const __bf16* q_rope; int64_t qr_st, qr_sh;
+  const __bf16* nope; int64_t nope_sp, nope_sr;
+  const __bf16* rope; int64_t rope_sp, rope_sr;
+  const int32_t* block_table; int64_t bt_stride; int32_t max_blocks;
+  const int32_t* seq_lens;
+  const int32_t* qsl;
+  int32_t batch, max_q_len, num_heads;
+  int64_t num_pages;
+  float scale_log2;
+  _Float16* o_part;              // [B*S, R_max, 512] fp16
+  float* lse_part;               // [B*S, R_max]
+  int32_t num_splits;
+  const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
+};
+
+// Launches mla_decode_v2_kernel<sparse> on `stream`; returns 0 or a negative error code.
+int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
+
+}  // namespace mlahip
