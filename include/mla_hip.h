@@ -60,8 +60,12 @@ int mla_cache_write_fp8(const void* kv_c, int64_t kv_c_stride, const void* k_pe,
  * [b*max_q_len, (b+1)*max_q_len) or [qsl[b], qsl[b+1]); token i of its s tokens sees keys [0, L_b - s + i].
  * `out` is addressed as [T, N, 512] through its strides, so the reference's head-major [N,T,512] result is
  * out_stride_t = 512, out_stride_h = T*512.  Page size is 128.
- * mla_decode_bf16 = mla_decode_bf16_split (one fp32 partial + log-sum-exp per KV split, into the workspace)
- * followed by mla_splitkv_reduce (the N-way merge of attention/ops.py:109-141). */
+ * mla_decode_bf16 = mla_decode_bf16_split followed by mla_splitkv_reduce (the N-way merge of
+ * attention/ops.py:109-141).  The split phase cuts the 32-token blocks of ALL sequences, laid end to end, into
+ * batch * num_splits chunks of equal size, one workgroup each, so ragged sequence lengths do not unbalance the
+ * launch; a chunk writes one normalised fp16 partial + fp32 log-sum-exp per sequence it touches.  The workspace
+ * therefore holds batch * (num_splits + 1) partials of max_q_len * num_heads rows.  Nothing in the plan is read
+ * back to the host: both phases derive it from seq_lens on the device. */
 size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits);
 
 int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h,   /* bf16 [T,N,512] */
@@ -82,9 +86,12 @@ int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_st
                           int32_t max_q_len, int32_t num_heads, float scale, void* workspace, size_t workspace_bytes,
                           int32_t num_splits, mlahip_stream_t stream);
 
-int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* query_start_loc, int32_t batch,
-                       int32_t max_q_len, int32_t num_heads, int32_t num_splits, void* out, int64_t out_stride_t,
-                       int64_t out_stride_h, float* lse_out, mlahip_stream_t stream);
+/* seq_lens: the array the split phase was given (partials in chunk order); NULL for the [sequence][split] order
+ * that mla_decode_fp8 uses internally.  Output rows must be 16-byte aligned (strides multiples of 8 elements). */
+int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* seq_lens,
+                       const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                       int32_t num_splits, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
+                       mlahip_stream_t stream);
 
 /* Same decode over the fp8-e4m3 block-scaled cache written by mla_cache_write_fp8 (row stride exactly 656 bytes,
  * page size 128).  Tiles are dequantised to bf16 on chip and take the bf16 MFMA path ("dequantise, then attend").

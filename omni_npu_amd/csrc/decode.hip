@@ -475,8 +475,15 @@ using namespace mlahip;
 
 extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits) {
   if (batch <= 0 || max_q_len <= 0 || num_heads <= 0 || num_splits <= 0) return 0;
-  const size_t rows = (size_t)batch * num_splits * max_q_len * num_heads;
+  // batch * num_splits chunks, and one more partial for every sequence boundary inside a chunk: batch * (num_splits + 1) partials in all
+  const size_t rows = (size_t)batch * ((size_t)num_splits + 1) * max_q_len * num_heads;
   return rows * kDNope * sizeof(_Float16) + rows * sizeof(float);   // fp16 partials + fp32 log-sum-exps
+}
+
+// first-generation kernel for the bf16 cache too (comparisons only)
+static bool use_first_generation() {
+  static const bool v = getenv("MLA_DECODE_V1") != nullptr;
+  return v;
 }
 
 static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
@@ -509,7 +516,9 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   MLA_REQUIRE((uintptr_t)workspace % 16 == 0, MLA_ERR_SHAPE, "mla_decode_bf16: workspace must be 16-byte aligned");
 
   const int r_max = max_q_len * num_heads;
-  const size_t rows = (size_t)batch * num_splits * r_max;
+  const size_t rows = (size_t)batch * ((size_t)num_splits + 1) * r_max;
+  MLA_REQUIRE((int64_t)batch * num_splits <= 0x7fffffff / 2 && nope_row_stride < (1 << 28) && rope_row_stride < (1 << 28),
+              MLA_ERR_SHAPE, "mla_decode_bf16: batch * num_splits or a row stride is out of range");
   DecodeParams p;
   p.q_nope = (const __bf16*)q_nope; p.qn_st = qn_stride_t; p.qn_sh = qn_stride_h;
   p.q_rope = (const __bf16*)q_rope; p.qr_st = qr_stride_t; p.qr_sh = qr_stride_h;
@@ -539,16 +548,15 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
     attr_set = true;
   }
   dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
-  static const bool use_v1 = getenv("MLA_DECODE_V1") != nullptr;     // first-generation kernel, for comparisons
-  if (!fp8 && !use_v1) {
+  if (!fp8 && !use_first_generation()) {
     DecodeV2Params v;
     v.q_nope = p.q_nope; v.qn_st = p.qn_st; v.qn_sh = p.qn_sh; v.q_rope = p.q_rope; v.qr_st = p.qr_st; v.qr_sh = p.qr_sh;
     v.nope = p.nope; v.nope_sp = p.nope_sp; v.nope_sr = p.nope_sr; v.rope = p.rope; v.rope_sp = p.rope_sp; v.rope_sr = p.rope_sr;
     v.block_table = p.block_table; v.bt_stride = p.bt_stride; v.max_blocks = p.max_blocks; v.seq_lens = p.seq_lens; v.qsl = p.qsl;
     v.batch = p.batch; v.max_q_len = p.max_q_len; v.num_heads = p.num_heads; v.num_pages = p.num_pages;
-    v.scale_log2 = p.scale_log2; v.o_part = p.o_part; v.lse_part = p.lse_part; v.num_splits = p.num_splits;
+    v.scale_log2 = p.scale_log2; v.o_part = p.o_part; v.lse_part = p.lse_part;
     v.sparse_rows = p.sparse_rows; v.sparse_stride = p.sparse_stride; v.page_size = p.page_size;
-    return launch_decode_v2(v, sparse_rows != nullptr, grid, stream);
+    return launch_decode_v2(v, sparse_rows != nullptr, dim3((unsigned)(batch * num_splits), 1, grid.z), stream);
   }
   if (fp8) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeFp8>, grid, dim3(256), kFp8LdsB, stream, p);
   else if (sparse_rows) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeSparse>, grid, dim3(256), kDecodeLdsB, stream, p);
@@ -573,9 +581,10 @@ extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, in
 }
 
 // Phase 2: N-way log-sum-exp merge of the workspace partials into the bf16 output (and optional lse).
-extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* query_start_loc,
-                                  int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t num_splits, void* out,
-                                  int64_t out_stride_t, int64_t out_stride_h, float* lse_out, hipStream_t stream) {
+extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* seq_lens,
+                                  const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                                  int32_t num_splits, void* out, int64_t out_stride_t, int64_t out_stride_h,
+                                  float* lse_out, hipStream_t stream) {
   MLA_REQUIRE(workspace && out, MLA_ERR_NULL, "mla_splitkv_reduce: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1, MLA_ERR_SHAPE,
               "mla_splitkv_reduce: batch=%d max_q_len=%d num_heads=%d num_splits=%d", batch, max_q_len, num_heads, num_splits);
@@ -587,7 +596,17 @@ extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes,
   MLA_REQUIRE(workspace_bytes >= need, MLA_ERR_WORKSPACE, "mla_splitkv_reduce: workspace %zu bytes < required %zu",
               workspace_bytes, need);
   const int r_max = max_q_len * num_heads;
-  const size_t rows = (size_t)batch * num_splits * r_max;
+  const size_t rows = (size_t)batch * ((size_t)num_splits + 1) * r_max;
+  if (seq_lens && !use_first_generation()) {
+    // partials in chunk order, as the bf16 kernels write them
+    ChunkReduceParams cp;
+    cp.o_part = (const _Float16*)workspace; cp.lse_part = (const float*)((const _Float16*)workspace + rows * kDNope);
+    cp.seq_lens = seq_lens; cp.qsl = query_start_loc;
+    cp.batch = batch; cp.max_q_len = max_q_len; cp.num_heads = num_heads; cp.num_chunks = batch * num_splits;
+    cp.out = (__bf16*)out; cp.out_st = out_stride_t; cp.out_sh = out_stride_h;
+    cp.lse_out = lse_out; cp.lse_st = num_heads;
+    return launch_chunk_reduce(cp, stream);
+  }
   ReduceParams rp;
   rp.o_part = (const _Float16*)workspace; rp.lse_part = (const float*)((const _Float16*)workspace + rows * kDNope);
   rp.qsl = query_start_loc;
@@ -615,8 +634,8 @@ extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t 
                                  num_pages, block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch,
                                  max_q_len, num_heads, scale, workspace, workspace_bytes, num_splits, stream);
   if (rc != MLA_OK) return rc;
-  return mla_splitkv_reduce(workspace, workspace_bytes, query_start_loc, batch, max_q_len, num_heads, num_splits, out,
-                            out_stride_t, out_stride_h, lse_out, stream);
+  return mla_splitkv_reduce(workspace, workspace_bytes, seq_lens, query_start_loc, batch, max_q_len, num_heads, num_splits,
+                            out, out_stride_t, out_stride_h, lse_out, stream);
 }
 
 // Sparse absorbed MLA over a per-token list of cache rows (reference: npu_sparse_flash_attention as called in
@@ -640,8 +659,8 @@ extern "C" int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, i
                              nullptr, 0, 0, counts, nullptr, num_tokens, 1, num_heads, scale, workspace, workspace_bytes,
                              num_splits, sparse_rows, sparse_stride, page_size, false, stream);
   if (rc != MLA_OK) return rc;
-  return mla_splitkv_reduce(workspace, workspace_bytes, nullptr, num_tokens, 1, num_heads, num_splits, out, out_stride_t,
-                            out_stride_h, lse_out, stream);
+  return mla_splitkv_reduce(workspace, workspace_bytes, counts, nullptr, num_tokens, 1, num_heads, num_splits, out,
+                            out_stride_t, out_stride_h, lse_out, stream);
 }
 
 // Absorbed-MLA paged decode over the fp8-e4m3 block-scaled cache written by mla_cache_write_fp8 (656-byte rows,
@@ -665,6 +684,7 @@ extern "C" int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t q
                              block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
                              scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, true, stream);
   if (rc != MLA_OK) return rc;
-  return mla_splitkv_reduce(workspace, workspace_bytes, query_start_loc, batch, max_q_len, num_heads, num_splits, out,
-                            out_stride_t, out_stride_h, lse_out, stream);
+  // the fp8 kernel writes its partials in [sequence][split] order: no sequence lengths, no chunk arithmetic
+  return mla_splitkv_reduce(workspace, workspace_bytes, nullptr, query_start_loc, batch, max_q_len, num_heads, num_splits,
+                            out, out_stride_t, out_stride_h, lse_out, stream);
 }

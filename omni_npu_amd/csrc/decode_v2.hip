@@ -31,7 +31,7 @@
 namespace mlahip {
 
 #ifndef MLA_V2_QK_AHEAD
-#define MLA_V2_QK_AHEAD 3
+#define MLA_V2_QK_AHEAD 6
 #endif
 #ifndef MLA_V2_PV_AHEAD
 #define MLA_V2_PV_AHEAD 2
@@ -69,6 +69,23 @@ __device__ __forceinline__ float half_sum(float v) {
   return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
 }
 
+__device__ __forceinline__ int v2_num_blocks(int len) { return len > 0 ? (len + kBlk - 1) / kBlk : 0; }
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+  return v;
+}
+__device__ __forceinline__ int wave_max_i32(int v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v = max(v, __shfl_xor(v, d, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_incl_scan_i32(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) { const int t = __shfl_up(v, d, 64); v += lane >= d ? t : 0; }
+  return v;
+}
+
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
 template <bool kSparse>
@@ -78,15 +95,58 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h32 = lane & 31;
   const int half = lane >> 5;
-  const int split = blockIdx.x, b = blockIdx.y, grp = blockIdx.z;
+  const int chunk = blockIdx.x, grp = blockIdx.z;
+  const int r_max = p.max_q_len * p.num_heads;
+  if (grp * 128 >= r_max) return;
+  const uint32_t lds0 = lds_addr_of(lds);
 
+  // ---- which blocks are mine ----
+  // The 32-token blocks of all sequences, laid end to end, are cut into gridDim.x chunks of equal size (to within one
+  // block), whatever the individual sequence lengths: chunk c covers global blocks [c*T/G, (c+1)*T/G).  A chunk that
+  // crosses a sequence boundary is processed as two (or more) segments; the segment of sequence b in chunk c writes
+  // partial number c + b, so the partials of one sequence are consecutive and mla_chunk_reduce_kernel finds them with
+  // the same arithmetic.  Every wavefront derives the plan by itself from the sequence lengths (two passes: total, scan).
+  int seg_b, seg_off, remaining;
+  {
+    int tot = 0;
+    for (int i = lane; i < p.batch; i += 64) tot += v2_num_blocks(p.seq_lens[i]);
+    tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
+    const int64_t cb = (int64_t)chunk * tot / gridDim.x, ce = (int64_t)(chunk + 1) * tot / gridDim.x;
+    if (cb == ce) return;
+    int carry = 0, b0 = 0, pb0 = 0;
+    for (int base = 0; base < p.batch; base += 64) {
+      const int i = base + lane;
+      const int c = i < p.batch ? v2_num_blocks(p.seq_lens[i]) : 0;
+      const int pe = wave_incl_scan_i32(c, lane) + carry;     // blocks of sequences 0..i
+      const bool le = i < p.batch && pe <= cb;                // sequence i ends at or before my first block
+      b0 += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+      pb0 = max(pb0, wave_max_i32(le ? pe : 0));
+      carry = __builtin_amdgcn_readlane(pe, 63);
+    }
+    seg_b = __builtin_amdgcn_readfirstlane(b0) - 1;
+    seg_off = (int)cb - __builtin_amdgcn_readfirstlane(pb0);
+    remaining = (int)(ce - cb);
+  }
+
+  while (remaining > 0) {
+  seg_b++;
+  if (seg_b >= p.batch) break;
+  const int b = seg_b;
   const int L = p.seq_lens[b];
+  const int blk_begin = seg_off;
+  seg_off = 0;
+  int take = v2_num_blocks(L) - blk_begin;
+  take = take < remaining ? take : remaining;
+  if (take <= 0) continue;
+  remaining -= take;
+  const int blk_end = blk_begin + take;
+  const int nb = take;
+  lds_barrier();                                              // the previous segment's epilogue is done with the buffers
+
   int q0, qlen;
   if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
   qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
   const int rows = qlen * p.num_heads;
-  const int r_max = p.max_q_len * p.num_heads;
-  if (grp * 128 >= r_max) return;
 
   // this lane's query row for QK / softmax (row group = wave)
   const int row = grp * 128 + wave * 32 + h32;
@@ -95,22 +155,12 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const int head = row - t_local * p.num_heads;
   int limit = row_ok ? (L - qlen + t_local + 1) : 0;         // keys [0, limit) are visible to this row
   limit = limit < 0 ? 0 : limit;
-  const int64_t part_base = ((int64_t)b * p.num_splits + split) * r_max + grp * 128;   // + row index in the group
+  const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
 
-  // token range of this split, in 32-token blocks (split boundaries on 64-token multiples, as the fp8 kernel)
-  const int tiles_total = (L + 63) / 64;
-  const int tps = (tiles_total + p.num_splits - 1) / p.num_splits;
-  const int blk_begin = split * tps * 2;
-  int blk_end = blk_begin + tps * 2;
-  const int blks_total = (L + kBlk - 1) / kBlk;
-  blk_end = blk_end < blks_total ? blk_end : blks_total;
-
-  if (blk_begin >= blk_end || grp * 128 >= rows) {
+  if (grp * 128 >= rows) {
     if (row < r_max && half == 0) p.lse_part[part_base + wave * 32 + h32] = -INFINITY;
-    return;
+    continue;
   }
-  const int nb = blk_end - blk_begin;
-  const uint32_t lds0 = lds_addr_of(lds);
 
   // ---- global -> LDS copies: 9 per lane and block (8 nope rows of 1 KiB per wave, one rope instruction of 8 rows) ----
   // Row r of a block goes to nope buffer row r (granule g at position g ^ swz(r)) and rope buffer row r.  All addresses
@@ -141,100 +191,94 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       pg_nxt = load_page(page_cur + 1);
     }
   };
-  auto issue_block = [&](int blk) {
-    const int tok0 = blk * kBlk;
-    const int last = L - 1 - tok0;                            // last valid row of the block (>= 0)
-    const uint32_t nbuf = lds0 + (blk & 3) * kV2NopeBufB;
-    const uint32_t rbuf = lds0 + kV2RopeOff + (blk % 3) * kV2RopeBufB;
+  // The nine copies of a block are issued one at a time ("pieces" 0..8) so that they can be spread over the MFMAs of the
+  // QK phase: piece k copies nope rows 4*wave + k/2 (+16 for odd k) for k < 8, piece 8 the wave's eight rope rows.  Rows
+  // past the end of the sequence re-read its last row (their scores are masked).
+  struct IssueCtx { const char* np; const char* rp; const char* a0; const char* a1; uint32_t nbuf, rbuf; int last, tok0; };
+  auto issue_begin = [&](int blk) -> IssueCtx {
+    IssueCtx c;
+    c.tok0 = blk * kBlk;
+    c.last = L - 1 - c.tok0;                                  // last valid row of the block (>= 0)
+    c.nbuf = lds0 + (blk & 3) * kV2NopeBufB;
+    c.rbuf = lds0 + kV2RopeOff + (blk % 3) * kV2RopeBufB;
     if constexpr (kSparse) {
-      const char* nope = (const char*)p.nope;
-      const char* rope = (const char*)p.rope;
-      auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
-      if (last >= kBlk - 1) {
-        // full block: the 16 row numbers this wave needs arrive as three scalar vector loads
-        typedef int32_t i4 __attribute__((ext_vector_type(4)));
-        typedef int32_t i8 __attribute__((ext_vector_type(8)));
-        const i4 ra = *(__attribute__((address_space(4))) const i4*)(srows + tok0 + wave * 4);
-        const i4 rb = *(__attribute__((address_space(4))) const i4*)(srows + tok0 + 16 + wave * 4);
-        const i8 rr = *(__attribute__((address_space(4))) const i8*)(srows + tok0 + wave * 8);
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          dma16_sv(nope + clampi(ra[j]) * n_sr2, dma_off[j], nbuf + (wave * 4 + j) * 1024);
-          dma16_sv(nope + clampi(rb[j]) * n_sr2, dma_off[j], nbuf + (16 + wave * 4 + j) * 1024);
-        }
-        int32_t mine = 0;
-#pragma unroll
-        for (int j = 0; j < 8; j++) mine = (lane >> 3) == j ? rr[j] : mine;
-        dma16_v(rope + clampi(mine) * r_sr2 + rope_off, rbuf + wave * 1024);
-      } else {
-#pragma unroll
-        for (int q = 0; q < 2; q++)
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const int r = q * 16 + wave * 4 + j;
-            const int re = r < last ? r : last;               // rows past the end re-read the last valid row
-            dma16_sv(nope + clampi(srows[tok0 + re]) * n_sr2, dma_off[j], nbuf + r * 1024);
-          }
-        int32_t mine = 0;
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-          const int r = wave * 8 + j;
-          const int32_t sj = srows[tok0 + (r < last ? r : last)];
-          mine = (lane >> 3) == j ? sj : mine;
-        }
-        dma16_v(rope + clampi(mine) * r_sr2 + rope_off, rbuf + wave * 1024);
-      }
+      c.np = (const char*)p.nope;
+      c.rp = (const char*)p.rope;
     } else {
       const int page = blk >> 2;
       if (page != page_cur) { page_cur = page; pg_cur = pg_nxt; pg_nxt = load_page(page + 1); }
       const uint32_t row0 = (uint32_t)(blk & 3) * kBlk;
-      const char* np = (const char*)p.nope + pg_cur * p.nope_sp * 2 + (uint64_t)row0 * n_sr2;
-      const char* rp = (const char*)p.rope + pg_cur * p.rope_sp * 2 + (uint64_t)row0 * r_sr2;
-      if (last >= kBlk - 1) {
-        const char* a0 = np + (uint64_t)(wave * 4) * n_sr2;
-        const char* a1 = a0 + (uint64_t)n_sr2 * 16;
-        const uint32_t l0 = nbuf + wave * 4096;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          dma16_sv(a0, dma_off[j], l0 + j * 1024);
-          dma16_sv(a1, dma_off[j], l0 + 16384 + j * 1024);
-          a0 += n_sr2;
-          a1 += n_sr2;
-        }
-        dma16_sv(rp + (uint64_t)(wave * 8) * r_sr2, rope_voff, rbuf + wave * 1024);
+      c.np = (const char*)p.nope + pg_cur * p.nope_sp * 2 + (uint64_t)row0 * n_sr2;
+      c.rp = (const char*)p.rope + pg_cur * p.rope_sp * 2 + (uint64_t)row0 * r_sr2;
+    }
+    c.a0 = c.np + (uint64_t)(wave * 4) * n_sr2;               // full dense blocks: running row addresses
+    c.a1 = c.a0 + (uint64_t)n_sr2 * 16;
+    return c;
+  };
+  // kFull: every row of the block exists and the source is the paged cache: plain pointer increments
+  auto issue_piece = [&](IssueCtx& c, int k, auto full) {
+    constexpr bool kFull = decltype(full)::value && !kSparse;
+    auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
+    if (k < 8) {
+      const int j = k >> 1;
+      const int r = (k & 1) * 16 + wave * 4 + j;
+      if constexpr (kFull) {
+        if ((k & 1) == 0) dma16_sv(c.a0, dma_off[j], c.nbuf + r * 1024);
+        else { dma16_sv(c.a1, dma_off[j], c.nbuf + r * 1024); c.a0 += n_sr2; c.a1 += n_sr2; }
       } else {
+        const int re = r < c.last ? r : c.last;
+        if constexpr (kSparse) dma16_sv(c.np + clampi(srows[c.tok0 + re]) * n_sr2, dma_off[j], c.nbuf + r * 1024);
+        else dma16_sv(c.np + (uint64_t)re * n_sr2, dma_off[j], c.nbuf + r * 1024);
+      }
+    } else {
+      if constexpr (kSparse) {
+        int32_t mine = 0;                                     // lane's row = 8*wave + lane/8, picked from 8 scalar loads
 #pragma unroll
-        for (int q = 0; q < 2; q++)
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const int r = q * 16 + wave * 4 + j;
-            const int re = r < last ? r : last;               // rows past the end re-read the last valid row
-            dma16_sv(np + (uint64_t)re * n_sr2, dma_off[j], nbuf + r * 1024);
-          }
+        for (int j = 0; j < 8; j++) {
+          const int r = wave * 8 + j;
+          const int32_t sj = srows[c.tok0 + (r < c.last ? r : c.last)];
+          mine = (lane >> 3) == j ? sj : mine;
+        }
+        dma16_v(c.rp + clampi(mine) * r_sr2 + rope_off, c.rbuf + wave * 1024);
+      } else if constexpr (kFull) {
+        dma16_sv(c.rp + (uint64_t)(wave * 8) * r_sr2, rope_voff, c.rbuf + wave * 1024);
+      } else {
         const int r = wave * 8 + (lane >> 3);
-        const int re = r < last ? r : last;
-        dma16_sv(rp, (uint32_t)re * r_sr2 + rope_off, rbuf + wave * 1024);
+        const int re = r < c.last ? r : c.last;
+        dma16_sv(c.rp, (uint32_t)re * r_sr2 + rope_off, c.rbuf + wave * 1024);
       }
     }
   };
-  auto issue_first_three = [&]() {
+  auto issue_block = [&](int blk) {
+    IssueCtx c = issue_begin(blk);
+#pragma unroll
+    for (int k = 0; k < 9; k++) issue_piece(c, k, std::false_type{});
+  };
+  auto issue_first = [&]() {
     issue_reset();
+    issue_block(blk_begin);
+  };
+  auto issue_next_two = [&]() {
 #pragma unroll 1
-    for (int j = 0; j < 3 && j < nb; j++) issue_block(blk_begin + j);
+    for (int j = 1; j < 3 && j < nb; j++) issue_block(blk_begin + j);
   };
 
-  // ---- prologue: query loads first (so that the explicit vmcnt waits below count only LDS copies), then three blocks in flight ----
+  // ---- prologue: the first block's copies go out, then the query loads; both are waited for together ----
+  issue_first();
   bf16x8 qf[36];
   {
+    // All 36 loads go out back to back and are waited for once (written as assembly: the compiler, short of registers,
+    // would wait for each load before issuing the next).  Rows that do not exist read row 0 of the sequence instead:
+    // their results are finite and never stored.
     const int64_t tq = row_ok ? (q0 + t_local) : q0;
     const int64_t hq = row_ok ? head : 0;
     const __bf16* qn = p.q_nope + tq * p.qn_st + hq * p.qn_sh + half * 8;
     const __bf16* qr = p.q_rope + tq * p.qr_st + hq * p.qr_sh + half * 8;
-    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int kk = 0; kk < 32; kk++) { bf16x8 v = *(const bf16x8*)(qn + kk * 16); qf[kk] = row_ok ? v : zero; }
+    for (int kk = 0; kk < 32; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[kk]) : "v"(qn), "i"(kk * 32));
 #pragma unroll
-    for (int kk = 0; kk < 4; kk++) { bf16x8 v = *(const bf16x8*)(qr + kk * 16); qf[32 + kk] = row_ok ? v : zero; }
+    for (int kk = 0; kk < 4; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[32 + kk]) : "v"(qr), "i"(kk * 32));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
     for (int kk = 0; kk < 36; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
   }
@@ -276,9 +320,18 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   // MFMA that consumes them, and explicit lgkmcnt waits: left to itself the compiler funnels every fragment through one
   // register quad and waits for each read in full, which exposes the whole LDS latency 36 times per block.  (LDS reads
   // return in order, so compiler-issued reads around this section only make its own waits stricter, never wrong.)
-  auto qk_block = [&](int blk, f32x16& s) {
+  // The MFMAs of this phase are written as assembly with the scores in ordinary vector registers: the compiler would
+  // put every MFMA result into the accumulation file, which is full of output accumulators, and shuffle 48 registers
+  // per block to make room.  Hazards the compiler would otherwise pad: none between dependent MFMAs of one shape with
+  // identical C and D; the wait after the last one (MFMA result read by the vector ALU) is the s_nop pair at the end.
+  // With kIssue the nine copies of block `blk_issue` are spread over the MFMAs.
+  auto qk_block = [&](int blk, f32x16& s, auto issue, int blk_issue, auto&& mid_hook) {
+    constexpr int kIssueMode = decltype(issue)::value;       // 0: no copies; 1: any block; 2: a full block of the paged cache
+    constexpr bool kIssue = kIssueMode != 0;
     const uint32_t nb32 = lds0 + (blk & 3) * kV2NopeBufB + kbase;     // buffers are 4 KiB aligned: the XORs below stay exact
     const uint32_t rb32 = lds0 + (blk % 3) * kV2RopeBufB + rbase;
+    IssueCtx ic;
+    if constexpr (kIssue) ic = issue_begin(blk_issue);
     bf16x8 ka[kQkAheadV2];
 #define MLA_K_READ(dst, kk)                                                                                         \
     do {                                                                                                            \
@@ -287,8 +340,6 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     } while (0)
 #pragma unroll
     for (int i = 0; i < kQkAheadV2; i++) MLA_K_READ(ka[i], i);
-#pragma unroll
-    for (int r = 0; r < 16; r++) s[r] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < 36; kk++) {
       // wait until fragment kk has landed: at most min(kQkAheadV2 - 1, 35 - kk) younger reads may still be in flight
@@ -302,19 +353,22 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       else if (younger == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(ka[kk % D]));
       else if (younger == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(ka[kk % D]));
       else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(ka[kk % D]));
-      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk % D], qf[kk], s, 0, 0, 0);
+      if (kk == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(ka[kk % D]), "v"(qf[kk]));
+      else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(ka[kk % D]), "v"(qf[kk]));
       if (kk + D < 36) MLA_K_READ(ka[kk % D], kk + D);
+      if constexpr (kIssue) if ((kk & 3) == 1) issue_piece(ic, kk >> 2, std::integral_constant<bool, kIssueMode == 2>{});
+      if (kk == 27) mid_hook();
     }
 #undef MLA_K_READ
-    asm volatile("" : "+v"(s));
+    asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s));
   };
 
   // Softmax of block `blk` from raw scores s, cut into eight straight-line steps so that it can be interleaved with the
   // P.V MFMAs of the previous block (step k is called after the k-th group of four MFMAs; the MFMAs run 32 clocks each
   // while the vector ALU is otherwise idle).  The row maximum is taken over all 32 scores of the block, visible or not:
   // it only serves as a reference, and any finite reference within 2^100 of the true maximum is as good as another.
-  struct SoftmaxState { float neg_ref, flag; int rel; bf16x8 pb[2]; float psum; };
-  auto softmax_step = [&](int step, int blk, f32x16& s, SoftmaxState& st) {
+  struct SoftmaxState { float neg_ref, flag; bf16x8 pb[2]; float psum; };
+  auto softmax_step = [&](int step, f32x16& s, SoftmaxState& st) {
     if (step == 0) {
       float mx = fmaxf(s[0], s[1]);
 #pragma unroll
@@ -324,41 +378,68 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       if (m_ref == -INFINITY) m_ref = mx;                    // the first block fixes the reference
       st.flag = mx > m_ref + kRestartThreshold ? -1.f : 1.f; // -1 asks the workgroup to restart with better references
       st.neg_ref = -m_ref;
-      st.rel = row_ok ? limit - blk * kBlk - 4 * half : 0;   // score r is visible iff 8*(r/4) + r%4 < rel
       st.psum = 0.f;
     } else if (step <= 4) {
 #pragma unroll
       for (int r = 4 * (step - 1); r < 4 * step; r++) {
         // an overflow to +inf can only happen past the restart threshold, and a restart discards everything accumulated
-        const float e = fast_exp2(__builtin_fmaf(s[r], p.scale_log2, st.neg_ref));
-        s[r] = (8 * (r >> 2) + (r & 3)) < st.rel ? e : 0.f;
+        s[r] = fast_exp2(__builtin_fmaf(s[r], p.scale_log2, st.neg_ref));
+        st.psum += s[r];
       }
     } else if (step == 5) {
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
         for (int e = 0; e < 8; e++) st.pb[kb][e] = (__bf16)s[kb * 8 + e];
-    } else if (step == 6) {
-      // the row sum uses the ROUNDED probabilities: numerator and denominator then carry the same weights, so the
-      // result is an exact convex combination of cache rows
+    }
+  };
+  // After the steps: the last blocks of a sequence hold keys that some rows must not see (causal multi-token queries,
+  // rows past the end of the sequence); only those blocks pay for the masking.  Then P^T and the flag go to LDS.
+  auto softmax_finish = [&](int blk, f32x16& s, SoftmaxState& st) {
+    if ((blk + 1) * kBlk > L - p.max_q_len + 1) {
+      const int rel = row_ok ? limit - blk * kBlk - 4 * half : 0;   // score r is visible iff 8*(r/4) + r%4 < rel
+      st.psum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        s[r] = (8 * (r >> 2) + (r & 3)) < rel ? s[r] : 0.f;
+        st.psum += s[r];
+      }
 #pragma unroll
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) st.psum += (float)st.pb[kb][e];
-    } else {
-      l_run += st.psum;
-      char* base = lds + (blk & 1) * kV2PBufB;
-      *(bf16x8*)(base + p_w_off) = st.pb[0];
-      *(bf16x8*)(base + p_w_off + 1024) = st.pb[1];
-      if (half == 0) *(float*)(lds + (blk & 1) * 512 + a_w_off) = st.flag;
+        for (int e = 0; e < 8; e++) st.pb[kb][e] = (__bf16)s[kb * 8 + e];
     }
+    l_run += st.psum;
+    char* base = lds + (blk & 1) * kV2PBufB;
+    *(bf16x8*)(base + p_w_off) = st.pb[0];
+    *(bf16x8*)(base + p_w_off + 1024) = st.pb[1];
+    if (half == 0) *(float*)(lds + (blk & 1) * 512 + a_w_off) = st.flag;
   };
 
   // O^T += V^T P^T for block `blk`: this wave's 128 output columns for all four row groups; with kFused the softmax of
   // block blk+1 (scores s) rides along
-  auto pv_block = [&](int blk, auto fused, f32x16& s) {
+  // First operands of the P.V phase of block `blk`, read with hand-placed instructions from inside the QK phase (they do
+  // not depend on it), so that the first P.V MFMA finds them in registers.
+  struct PvHead { bf16x8 pr[4]; bf16x4 v[4]; };
+  auto pv_head_read = [&](int blk, PvHead& h) {
+    const uint32_t pb32 = lds0 + (blk & 1) * kV2PBufB + p_r_off;
+    const uint32_t vb32 = lds0 + (blk & 3) * kV2NopeBufB;
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(h.pr[rg]) : "v"(pb32), "i"(rg * 2 * 1024));
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(h.v[2 * j]) : "v"(vb32 + (vbase[0] ^ (uint32_t)(j << 6))));
+      asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(h.v[2 * j + 1]) : "v"(vb32 + (vbase[1] ^ (uint32_t)(j << 6))));
+    }
+  };
+  auto pv_head_wait = [&](PvHead& h) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(h.pr[0]), "+v"(h.pr[1]), "+v"(h.pr[2]), "+v"(h.pr[3]), "+v"(h.v[0]), "+v"(h.v[1]),
+                 "+v"(h.v[2]), "+v"(h.v[3]));
+  };
+  auto pv_block = [&](int blk, auto fused, f32x16& s, SoftmaxState& st, auto preloaded, PvHead& head) {
     constexpr bool kFused = decltype(fused)::value;
-    SoftmaxState st;
+    constexpr bool kPre = decltype(preloaded)::value;
+    static_assert(kPvAheadV2 == 2, "the preloaded head holds two V^T fragments");
     const char* pbase = lds + (blk & 1) * kV2PBufB;
     const char* vb = lds + (blk & 3) * kV2NopeBufB;
     auto v_frag = [&](int stp) -> bf16x8 {                    // stp = 4*kb + db
@@ -368,13 +449,22 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     };
     bf16x8 va[kPvAheadV2];
+    if constexpr (kPre) {
+      pv_head_wait(head);
 #pragma unroll
-    for (int j = 0; j < kPvAheadV2; j++) va[j] = v_frag(j);
+      for (int j = 0; j < 2; j++) va[j] = __builtin_shufflevector(head.v[2 * j], head.v[2 * j + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kPvAheadV2; j++) va[j] = v_frag(j);
+    }
 #pragma unroll
     for (int kb = 0; kb < 2; kb++) {
       bf16x8 pr[4];
 #pragma unroll
-      for (int rg = 0; rg < 4; rg++) pr[rg] = *(const bf16x8*)(pbase + p_r_off + (rg * 2 + kb) * 1024);
+      for (int rg = 0; rg < 4; rg++) {
+        if (kPre && kb == 0) pr[rg] = head.pr[rg];
+        else pr[rg] = *(const bf16x8*)(pbase + p_r_off + (rg * 2 + kb) * 1024);
+      }
 #pragma unroll
       for (int db = 0; db < 4; db++) {
         const int stp = kb * 4 + db;
@@ -383,7 +473,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
 #pragma unroll
         for (int rg = 0; rg < 4; rg++)
           acc[db][rg] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pr[rg], acc[db][rg], 0, 0, 0);
-        if constexpr (kFused) softmax_step(stp, blk + 1, s, st);
+        if constexpr (kFused) softmax_step(stp, s, st);
       }
     }
 #pragma unroll
@@ -391,9 +481,10 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
 #pragma unroll
       for (int rg = 0; rg < 4; rg++) asm volatile("" : "+a"(acc[db][rg]));     // output accumulators stay in AGPRs
   };
-  auto flags_ask_restart = [&](int blk) -> bool {
-    const f32x4 fl = *(const f32x4*)(lds + (blk & 1) * 512 + a_r_off);
-    // every wave reads the same 128 flags: a uniform decision
+  // every wave reads the same 128 flags: a uniform decision.  The read is issued right after the barrier and tested after
+  // the QK phase, when it has long landed; acting late is harmless because a restart discards everything.
+  auto flags_read = [&](int blk) -> f32x4 { return *(const f32x4*)(lds + (blk & 1) * 512 + a_r_off); };
+  auto flags_ask_restart = [&](const f32x4& fl) -> bool {
     return __builtin_amdgcn_ballot_w64(fl[0] < 0.f || fl[1] < 0.f || fl[2] < 0.f || fl[3] < 0.f) != 0;
   };
 
@@ -411,18 +502,20 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
         for (int j = 0; j < 4; j++)
 #pragma unroll
           for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      issue_first();
       restart = false;
     }
-    issue_first_three();
+    issue_next_two();
     // ---- block 0: QK, softmax, publish ----
     {
       if (nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
       lds_barrier();
       f32x16 s;
       SoftmaxState st;
-      qk_block(blk_begin, s);
+      qk_block(blk_begin, s, std::integral_constant<int, 0>{}, 0, [] {});
 #pragma unroll
-      for (int step = 0; step < 8; step++) softmax_step(step, blk_begin, s, st);
+      for (int step = 0; step < 6; step++) softmax_step(step, s, st);
+      softmax_finish(blk_begin, s, st);
     }
     // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
     for (int i = 0; i + 1 < nb; i++) {
@@ -430,18 +523,24 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
       if (i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
       lds_barrier();
-      if (flags_ask_restart(blk)) { restart = true; break; }
-      if (i + 3 < nb) issue_block(blk + 3);
+      const f32x4 fl = flags_read(blk);
       f32x16 s;
-      qk_block(blk + 1, s);
-      pv_block(blk, std::true_type{}, s);
+      PvHead head;
+      auto hook = [&] { pv_head_read(blk, head); };
+      if (i + 3 >= nb) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0, hook);
+      else if (kSparse || L - 1 - (blk + 3) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + 3, hook);
+      else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + 3, hook);
+      if (flags_ask_restart(fl)) { restart = true; break; }
+      SoftmaxState st;
+      pv_block(blk, std::true_type{}, s, st, std::true_type{}, head);
+      softmax_finish(blk + 1, s, st);
     }
     if (!restart) {
       const int blk = blk_end - 1;
       MLA_WAIT_VMCNT(0);
       lds_barrier();
-      if (flags_ask_restart(blk)) restart = true;
-      else { f32x16 s; pv_block(blk, std::false_type{}, s); }
+      if (flags_ask_restart(flags_read(blk))) restart = true;
+      else { f32x16 s; SoftmaxState st; PvHead head; pv_block(blk, std::false_type{}, s, st, std::false_type{}, head); }
     }
   } while (restart);
 
@@ -490,6 +589,79 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
+  }  // segments
+}
+
+// N-way merge of the partials of one query row (src/omni_npu/attention/ops.py:109-141), for the chunk layout written
+// by mla_decode_v2_kernel: one wavefront per row.  The partials of sequence b are those of the chunks that overlap its
+// blocks, numbered chunk + b.
+__global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
+  const int lane = threadIdx.x & 63;
+  const int r_max = p.max_q_len * p.num_heads;
+  const int64_t gr = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gr >= (int64_t)p.batch * r_max) return;
+  const int b = gr / r_max;
+  const int row = gr - (int64_t)b * r_max;
+  int q0, qlen;
+  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
+  qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
+  if (row >= qlen * p.num_heads) return;
+  const int t_local = row / p.num_heads;
+  const int head = row - t_local * p.num_heads;
+
+  int tot_blocks = 0, before = 0;
+  for (int i = lane; i < p.batch; i += 64) {
+    const int c = v2_num_blocks(p.seq_lens[i]);
+    tot_blocks += c;
+    before += i < b ? c : 0;
+  }
+  tot_blocks = wave_sum_i32(tot_blocks);
+  before = wave_sum_i32(before);
+  const int mine = v2_num_blocks(p.seq_lens[b]);
+  const int64_t G = p.num_chunks, T = tot_blocks;
+
+  float m = -INFINITY;
+  float tot = 0.f;
+  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (mine > 0) {
+    // chunk c starts at block floor(c*T/G): the chunk holding block x is the largest c with c*T < (x+1)*G
+    const int c_first = (int)((((int64_t)before + 1) * G - 1) / T);
+    const int c_last = (int)((((int64_t)before + mine) * G - 1) / T);
+    for (int c = c_first; c <= c_last; c++) {
+      if (c * T / G == (c + 1) * T / G) continue;            // empty chunk: wrote nothing
+      float l = p.lse_part[(int64_t)(c + b) * r_max + row];
+      l = l == INFINITY ? -INFINITY : l;
+      m = fmaxf(m, l);
+    }
+    if (m != -INFINITY) {
+      for (int c = c_first; c <= c_last; c++) {
+        if (c * T / G == (c + 1) * T / G) continue;
+        const int64_t pr = (int64_t)(c + b) * r_max + row;
+        const float l = p.lse_part[pr];
+        if (l == INFINITY || l == -INFINITY) continue;       // nothing visible in that segment
+        const float w = __expf(l - m);
+        tot += w;
+        const h8 v = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) a[e] += (float)v[e] * w;
+      }
+    }
+  }
+  const float inv = tot > 0.f ? 1.f / tot : 0.f;
+  __bf16* out = p.out + (int64_t)(q0 + t_local) * p.out_st + (int64_t)head * p.out_sh;
+  bf16x8 o8;
+#pragma unroll
+  for (int e = 0; e < 8; e++) o8[e] = (__bf16)(a[e] * inv);
+  *(bf16x8*)(out + lane * 8) = o8;
+  if (p.lse_out && lane == 0)
+    p.lse_out[(int64_t)(q0 + t_local) * p.lse_st + head] = tot > 0.f ? __logf(tot) + m : -INFINITY;
+}
+
+int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
+  const int64_t nrows = (int64_t)p.batch * p.max_q_len * p.num_heads;
+  hipLaunchKernelGGL(mla_chunk_reduce_kernel, dim3((unsigned)((nrows + 3) / 4)), dim3(256), 0, stream, p);
+  return check_launch("mla_chunk_reduce_kernel");
 }
 
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream) {

@@ -15,11 +15,19 @@ struct DecodeV2Params {
   int32_t batch, max_q_len, num_heads;
   int64_t num_pages;
   float scale_log2;
-  _Float16* o_part;              // [B*S, R_max, 512] fp16
-  float* lse_part;               // [B*S, R_max]
-  int32_t num_splits;
+  _Float16* o_part;              // [chunks + B, R_max, 512] fp16, normalised
+  float* lse_part;               // [chunks + B, R_max], natural log
   const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
 };
+
+struct ChunkReduceParams {
+  const _Float16* o_part; const float* lse_part;
+  const int32_t* seq_lens; const int32_t* qsl;
+  int32_t batch, max_q_len, num_heads, num_chunks;
+  __bf16* out; int64_t out_st, out_sh;
+  float* lse_out; int64_t lse_st;      // optional [T, N]
+};
+int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream);
 
 // Launches mla_decode_v2_kernel<sparse> on `stream`; returns 0 or a negative error code.
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);

@@ -233,7 +233,7 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
     elif phase == "split":
         _lib.check(lib.mla_decode_bf16_split(*front, *ws_args, num_splits, st), "mla_decode_bf16_split")
     elif phase == "reduce":
-        rc = lib.mla_splitkv_reduce(*ws_args, qsl, b, q_len, n, num_splits, out.data_ptr(), out.stride(0), out.stride(1),
+        rc = lib.mla_splitkv_reduce(*ws_args, seq_lens.data_ptr(), qsl, b, q_len, n, num_splits, out.data_ptr(), out.stride(0), out.stride(1),
                                     lse_p, st)
         _lib.check(rc, "mla_splitkv_reduce")
     else:
