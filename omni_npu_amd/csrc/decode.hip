@@ -477,7 +477,8 @@ extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, i
   if (batch <= 0 || max_q_len <= 0 || num_heads <= 0 || num_splits <= 0) return 0;
   // batch * num_splits chunks, and one more partial for every sequence boundary inside a chunk: batch * (num_splits + 1) partials in all
   const size_t rows = (size_t)batch * ((size_t)num_splits + 1) * max_q_len * num_heads;
-  return rows * kDNope * sizeof(_Float16) + rows * sizeof(float);   // fp16 partials + fp32 log-sum-exps
+  // fp16 partials, fp32 log-sum-exps, and per row a correction record (fp32 factor + cache address)
+  return rows * kDNope * sizeof(_Float16) + rows * (2 * sizeof(float) + sizeof(void*));
 }
 
 // first-generation kernel for the bf16 cache too (comparisons only)
@@ -555,6 +556,7 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
     v.block_table = p.block_table; v.bt_stride = p.bt_stride; v.max_blocks = p.max_blocks; v.seq_lens = p.seq_lens; v.qsl = p.qsl;
     v.batch = p.batch; v.max_q_len = p.max_q_len; v.num_heads = p.num_heads; v.num_pages = p.num_pages;
     v.scale_log2 = p.scale_log2; v.o_part = p.o_part; v.lse_part = p.lse_part;
+    v.corr_scale = p.lse_part + rows; v.corr_row = (const __bf16**)(p.lse_part + 2 * rows);
     v.sparse_rows = p.sparse_rows; v.sparse_stride = p.sparse_stride; v.page_size = p.page_size;
     return launch_decode_v2(v, sparse_rows != nullptr, dim3((unsigned)(batch * num_splits), 1, grid.z), stream);
   }
@@ -601,6 +603,7 @@ extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes,
     // partials in chunk order, as the bf16 kernels write them
     ChunkReduceParams cp;
     cp.o_part = (const _Float16*)workspace; cp.lse_part = (const float*)((const _Float16*)workspace + rows * kDNope);
+    cp.corr_scale = cp.lse_part + rows; cp.corr_row = (const __bf16* const*)(cp.lse_part + 2 * rows);
     cp.seq_lens = seq_lens; cp.qsl = query_start_loc;
     cp.batch = batch; cp.max_q_len = max_q_len; cp.num_heads = num_heads; cp.num_chunks = batch * num_splits;
     cp.out = (__bf16*)out; cp.out_st = out_stride_t; cp.out_sh = out_stride_h;

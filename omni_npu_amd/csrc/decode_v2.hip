@@ -63,6 +63,10 @@ __device__ __forceinline__ float half_max(float v) {
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
 }
+__device__ __forceinline__ int half_max_i32(int v) {
+  const auto r = __builtin_amdgcn_permlane32_swap((uint32_t)v, (uint32_t)v, false, false);
+  return max((int)r[0], (int)r[1]);
+}
 __device__ __forceinline__ float half_sum(float v) {
   const uint32_t u = __builtin_bit_cast(uint32_t, v);
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
@@ -158,7 +162,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
 
   if (grp * 128 >= rows) {
-    if (row < r_max && half == 0) p.lse_part[part_base + wave * 32 + h32] = -INFINITY;
+    if (row < r_max && half == 0) { p.lse_part[part_base + wave * 32 + h32] = -INFINITY; p.corr_scale[part_base + wave * 32 + h32] = 0.f; }
     continue;
   }
 
@@ -278,7 +282,9 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     for (int kk = 0; kk < 32; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[kk]) : "v"(qn), "i"(kk * 32));
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[32 + kk]) : "v"(qr), "i"(kk * 32));
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // (a builtin, so that the compiler's own bookkeeping of outstanding loads is cleared too: otherwise it would guard
+    // the first use of any earlier load inside the main loop with a full wait, on every iteration)
+    __builtin_amdgcn_s_waitcnt(0x0F70);                                         // vmcnt(0)
 #pragma unroll
     for (int kk = 0; kk < 36; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
   }
@@ -293,6 +299,8 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   float m_ref = -INFINITY;       // this row's softmax reference (log2 domain), fixed once finite
   float m_seen = -INFINITY;      // largest score seen so far (reference of a restart)
   float l_run = 0.f;
+  float top_p = 0.f;             // largest probability (relative to m_ref) among the visible keys so far ...
+  int top_tok = -1;              // ... and the position of that key in the sequence's key list
 
   // ---- per-lane LDS offsets ----
   // The swizzles are XORs confined to bits 4..7 of a byte offset whose other low bits are zero, so one base register
@@ -311,10 +319,14 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     const int rr = v_row + 8 * rd;
     vbase[rd] = (uint32_t)(rr * 1024 + v_in + wave * 256 + ((v_cl ^ v2_swz_nope(rr & 15)) << 4));
   }
-  const int p_w_off = kV2POff + (wave * 2 * 64 + lane) * 16;  // + kb*1024 + parity*8192 : this wave's P^T fragments
-  const int p_r_off = kV2POff + lane * 16;                    // + (rg*2 + kb)*1024 + parity*8192
-  const int a_r_off = kV2AOff + h32 * 16;                     // + parity*512: restart flags of rows (rg, h32), 4 floats
-  const int a_w_off = kV2AOff + h32 * 16 + wave * 4;
+  // P^T fragments and restart flags in LDS.  These offsets are recomputed from the hardware lane number wherever they are
+  // used instead of living in registers across the loop: every register counts (a spilled value would be reloaded with
+  // a vector-memory wait that also waits for the copies in flight).
+  auto lane_now = [] { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); };
+  auto p_w_off = [&] { return kV2POff + (wave * 2 * 64 + lane_now()) * 16; };   // + kb*1024 + parity*8192: this wave's fragments
+  auto p_r_off = [&] { return kV2POff + lane_now() * 16; };                     // + (rg*2 + kb)*1024 + parity*8192
+  auto a_r_off = [&] { return kV2AOff + (lane_now() & 31) * 16; };              // + parity*512: flags of rows (rg, h32), 4 floats
+  auto a_w_off = [&] { return kV2AOff + (lane_now() & 31) * 16 + wave * 4; };
 
   // S^T for block `blk`.  The K fragments are read with hand-placed LDS instructions, kQkAheadV2 fragments ahead of the
   // MFMA that consumes them, and explicit lgkmcnt waits: left to itself the compiler funnels every fragment through one
@@ -367,17 +379,36 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   // P.V MFMAs of the previous block (step k is called after the k-th group of four MFMAs; the MFMAs run 32 clocks each
   // while the vector ALU is otherwise idle).  The row maximum is taken over all 32 scores of the block, visible or not:
   // it only serves as a reference, and any finite reference within 2^100 of the true maximum is as good as another.
-  struct SoftmaxState { float neg_ref, flag; bf16x8 pb[2]; float psum; };
+  // Which of the row's 32 probabilities is the largest: the element number travels in the five low mantissa bits of the
+  // (positive) values through an unsigned maximum, so no compare-and-select chain and no branch is needed.  Two values
+  // closer than 2^-18 relative may swap places, which only matters to a correction that is itself a rounding error.
+  auto argmax_pack = [&](const f32x16& s) -> uint32_t {
+    // (plain assembly without side effects: the optimiser mangles the equivalent C++ reduction)
+    const uint32_t keep = ~31u;
+    uint32_t u[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(u[r]) : "v"(s[r]), "s"(keep), "n"(r));
+    uint32_t pk = u[0];
+#pragma unroll
+    for (int r = 1; r < 15; r += 2) asm("v_max3_u32 %0, %1, %2, %3" : "=v"(pk) : "v"(pk), "v"(u[r]), "v"(u[r + 1]));
+    asm("v_max_u32 %0, %1, %2" : "=v"(pk) : "v"(pk), "v"(u[15]));
+    pk |= (uint32_t)(lane_now() >> 1) & 16u;                 // bit 4: upper half of the wavefront
+    const auto sw = __builtin_amdgcn_permlane32_swap(pk, pk, false, false);
+    return max((uint32_t)sw[0], (uint32_t)sw[1]);
+  };
+  struct SoftmaxState { float neg_ref, flag, pm; uint32_t pk; bf16x8 pb[2]; float psum; };
   auto softmax_step = [&](int step, f32x16& s, SoftmaxState& st) {
     if (step == 0) {
       float mx = fmaxf(s[0], s[1]);
 #pragma unroll
       for (int r = 2; r < 16; r += 2) mx = fmaxf(mx, fmaxf(s[r], s[r + 1]));
-      mx = half_max(mx) * p.scale_log2;
+      const float mx_raw = half_max(mx);
+      mx = mx_raw * p.scale_log2;
       m_seen = fmaxf(m_seen, mx);
       if (m_ref == -INFINITY) m_ref = mx;                    // the first block fixes the reference
       st.flag = mx > m_ref + kRestartThreshold ? -1.f : 1.f; // -1 asks the workgroup to restart with better references
       st.neg_ref = -m_ref;
+      st.pm = fast_exp2(__builtin_fmaf(mx_raw, p.scale_log2, st.neg_ref));   // bit-identical to that score's probability below
       st.psum = 0.f;
     } else if (step <= 4) {
 #pragma unroll
@@ -391,13 +422,17 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
         for (int e = 0; e < 8; e++) st.pb[kb][e] = (__bf16)s[kb * 8 + e];
+    } else if (step == 6) {
+      st.pk = argmax_pack(s);
     }
   };
   // After the steps: the last blocks of a sequence hold keys that some rows must not see (causal multi-token queries,
   // rows past the end of the sequence); only those blocks pay for the masking.  Then P^T and the flag go to LDS.
   auto softmax_finish = [&](int blk, f32x16& s, SoftmaxState& st) {
     if ((blk + 1) * kBlk > L - p.max_q_len + 1) {
-      const int rel = row_ok ? limit - blk * kBlk - 4 * half : 0;   // score r is visible iff 8*(r/4) + r%4 < rel
+      int blk_s = blk;                                        // opaque: keeps the compiler from carrying `rel` as a loop
+      asm volatile("" : "+s"(blk_s));                         // variable of its own (one more register across the loop)
+      const int rel = limit - blk_s * kBlk - ((lane_now() >> 3) & 4);   // score r is visible iff 8*(r/4) + r%4 < rel
       st.psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
@@ -408,12 +443,26 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       for (int kb = 0; kb < 2; kb++)
 #pragma unroll
         for (int e = 0; e < 8; e++) st.pb[kb][e] = (__bf16)s[kb * 8 + e];
+      float pv = fmaxf(s[0], s[1]);                           // largest VISIBLE probability of the row in this block
+#pragma unroll
+      for (int r = 2; r < 16; r += 2) pv = fmaxf(pv, fmaxf(s[r], s[r + 1]));
+      st.pm = half_max(pv);
+      st.pk = argmax_pack(s);
+    }
+    // Remember the row's most probable key: the bf16 rounding of its probability is the largest single error of the
+    // P.V product when the softmax is peaked, and the merge kernel takes it out again.
+    {
+      const bool nw = st.pm > top_p;
+      top_p = nw ? st.pm : top_p;
+      const int e = (int)(st.pk & 15u);
+      top_tok = nw ? blk * kBlk + (int)((st.pk >> 2) & 4u) + 8 * (e >> 2) + (e & 3) : top_tok;
     }
     l_run += st.psum;
     char* base = lds + (blk & 1) * kV2PBufB;
-    *(bf16x8*)(base + p_w_off) = st.pb[0];
-    *(bf16x8*)(base + p_w_off + 1024) = st.pb[1];
-    if (half == 0) *(float*)(lds + (blk & 1) * 512 + a_w_off) = st.flag;
+    const int pw = p_w_off();
+    *(bf16x8*)(base + pw) = st.pb[0];
+    *(bf16x8*)(base + pw + 1024) = st.pb[1];
+    if (lane_now() < 32) *(float*)(lds + (blk & 1) * 512 + a_w_off()) = st.flag;
   };
 
   // O^T += V^T P^T for block `blk`: this wave's 128 output columns for all four row groups; with kFused the softmax of
@@ -422,7 +471,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   // not depend on it), so that the first P.V MFMA finds them in registers.
   struct PvHead { bf16x8 pr[4]; bf16x4 v[4]; };
   auto pv_head_read = [&](int blk, PvHead& h) {
-    const uint32_t pb32 = lds0 + (blk & 1) * kV2PBufB + p_r_off;
+    const uint32_t pb32 = lds0 + (blk & 1) * kV2PBufB + p_r_off();
     const uint32_t vb32 = lds0 + (blk & 3) * kV2NopeBufB;
 #pragma unroll
     for (int rg = 0; rg < 4; rg++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(h.pr[rg]) : "v"(pb32), "i"(rg * 2 * 1024));
@@ -463,7 +512,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
 #pragma unroll
       for (int rg = 0; rg < 4; rg++) {
         if (kPre && kb == 0) pr[rg] = head.pr[rg];
-        else pr[rg] = *(const bf16x8*)(pbase + p_r_off + (rg * 2 + kb) * 1024);
+        else pr[rg] = *(const bf16x8*)(pbase + p_r_off() + (rg * 2 + kb) * 1024);
       }
 #pragma unroll
       for (int db = 0; db < 4; db++) {
@@ -483,7 +532,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   };
   // every wave reads the same 128 flags: a uniform decision.  The read is issued right after the barrier and tested after
   // the QK phase, when it has long landed; acting late is harmless because a restart discards everything.
-  auto flags_read = [&](int blk) -> f32x4 { return *(const f32x4*)(lds + (blk & 1) * 512 + a_r_off); };
+  auto flags_read = [&](int blk) -> f32x4 { return *(const f32x4*)(lds + (blk & 1) * 512 + a_r_off()); };
   auto flags_ask_restart = [&](const f32x4& fl) -> bool {
     return __builtin_amdgcn_ballot_w64(fl[0] < 0.f || fl[1] < 0.f || fl[2] < 0.f || fl[3] < 0.f) != 0;
   };
@@ -496,6 +545,8 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       lds_barrier();
       m_ref = m_seen;
       l_run = 0.f;
+      top_p = 0.f;
+      top_tok = -1;
 #pragma unroll
       for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -514,9 +565,15 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       SoftmaxState st;
       qk_block(blk_begin, s, std::integral_constant<int, 0>{}, 0, [] {});
 #pragma unroll
-      for (int step = 0; step < 6; step++) softmax_step(step, s, st);
+      for (int step = 0; step < 7; step++) softmax_step(step, s, st);
       softmax_finish(blk_begin, s, st);
     }
+    // Everything the loop keeps in registers is touched here: a value that was parked in scratch during the prologue is
+    // brought back (and waited for) now, not at its first use inside the loop, where the wait would recur every iteration
+    // and stall on the copies in flight.
+    asm volatile("" :: "v"(limit), "v"(kbase), "v"(rbase), "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(m_seen), "v"(l_run),
+                 "v"(top_p), "v"(top_tok), "v"(dma_off[0]), "v"(dma_off[1]), "v"(dma_off[2]), "v"(dma_off[3]), "v"(rope_off),
+                 "v"(rope_voff));
     // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
     for (int i = 0; i + 1 < nb; i++) {
       const int blk = blk_begin + i;
@@ -549,13 +606,36 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   {
     const float l_tot = half_sum(l_run);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    // Rows whose most probable key carries more than 1/16 of the weight leave a note for the merge kernel: the rounding
+    // error of that key's probability (already divided by l) and the address of its latent vector in the cache.
+    float corr = 0.f;
+    const __bf16* vrow = p.nope;
+    if (row_ok && top_tok >= 0 && top_p * 16.f > l_tot) {
+      corr = (top_p - (float)(__bf16)top_p) * inv;
+      if constexpr (kSparse) {
+        int64_t slot = p.sparse_rows[(int64_t)b * p.sparse_stride + top_tok];
+        slot = slot < 0 ? 0 : (slot > max_row ? max_row : slot);
+        vrow = p.nope + slot * p.nope_sr;
+      } else {
+        int page = top_tok / kPage;
+        page = page < p.max_blocks ? page : p.max_blocks - 1;
+        int64_t pg = p.block_table[(int64_t)b * p.bt_stride + page];
+        pg = pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
+        vrow = p.nope + pg * p.nope_sp + (int64_t)(top_tok % kPage) * p.nope_sr;
+      }
+    }
     if (half == 0) {
-      *(float*)(lds + a_w_off) = inv;
-      if (row < r_max) p.lse_part[part_base + wave * 32 + h32] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
+      *(float*)(lds + kV2POff + h32 * 16 + wave * 4) = inv;
+      if (row < r_max) {
+        const int64_t pr = part_base + wave * 32 + h32;
+        p.lse_part[pr] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        p.corr_scale[pr] = corr;
+        p.corr_row[pr] = vrow;
+      }
     }
   }
   lds_barrier();
-  const f32x4 inv4 = *(const f32x4*)(lds + a_r_off);
+  const f32x4 inv4 = *(const f32x4*)(lds + kV2POff + h32 * 16);
   // transpose through this wave's private 32 KiB (nope buffer `wave`): two rounds of 64 rows x 128 columns, fp16
   char* stage = lds + wave * kV2NopeBufB;
 #pragma unroll
@@ -645,6 +725,13 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
         const h8 v = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
 #pragma unroll
         for (int e = 0; e < 8; e++) a[e] += (float)v[e] * w;
+        // the split kernel rounded this segment's dominant probability to bf16: put the difference back
+        const float cs = p.corr_scale[pr];
+        if (cs != 0.f) {
+          const bf16x8 kv = *(const bf16x8*)(p.corr_row[pr] + lane * 8);
+#pragma unroll
+          for (int e = 0; e < 8; e++) a[e] += (float)kv[e] * (w * cs);
+        }
       }
     }
   }

@@ -17,11 +17,13 @@ struct DecodeV2Params {
   float scale_log2;
   _Float16* o_part;              // [chunks + B, R_max, 512] fp16, normalised
   float* lse_part;               // [chunks + B, R_max], natural log
+  float* corr_scale;             // [chunks + B, R_max]: (p - bf16(p)) / l of the row's dominant key, or 0
+  const __bf16** corr_row;       // [chunks + B, R_max]: that key's latent vector in the cache
   const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
 };
 
 struct ChunkReduceParams {
-  const _Float16* o_part; const float* lse_part;
+  const _Float16* o_part; const float* lse_part; const float* corr_scale; const __bf16* const* corr_row;
   const int32_t* seq_lens; const int32_t* qsl;
   int32_t batch, max_q_len, num_heads, num_chunks;
   __bf16* out; int64_t out_st, out_sh;
