@@ -154,9 +154,14 @@ int dsa_quant_rows_fp8(const void* src, int64_t src_stride, int64_t rows, const 
                        void* dst8, int64_t dst_page_stride_bytes, int64_t dst_row_stride_bytes, float* dst_scale,
                        int64_t scale_page_stride, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
 
+/* With a workspace of dsa_topk_workspace_bytes() the selection of a token is spread over several workgroups (three
+ * launches that meet in the workspace: slice histograms, boundary-bin gather, ordered write), which is what a
+ * decode step with few tokens and long rows needs; with workspace == NULL one workgroup per token does everything and
+ * no scratch memory is touched.  Both give identical results. */
+size_t dsa_topk_workspace_bytes(int32_t batch, int32_t max_q_len, int64_t logits_stride);
 int dsa_topk(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
              int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
-             mlahip_stream_t stream);
+             void* workspace /* may be NULL */, size_t workspace_bytes, mlahip_stream_t stream);
 
 /* ---- (a16) sparse MLA over the selected keys ----------------------------------------------------------
  * Replaces torch.ops.custom.npu_sparse_flash_attention, attention/backends/dsa.py:259-291 (sparse_block_size 1,

@@ -158,8 +158,8 @@ def merge_states(prefix_out: torch.Tensor, prefix_lse: torch.Tensor, suffix_out:
 _workspaces: dict = {}
 
 
-def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
-    key = (dev.index, )
+def _workspace(dev: torch.device, nbytes: int, tag: str = "decode") -> torch.Tensor:
+    key = (dev.index, tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
@@ -294,9 +294,11 @@ def indexer_scores(q8: torch.Tensor, weights: torch.Tensor, k8_cache: torch.Tens
 
 
 def topk(logits: torch.Tensor, seq_lens: torch.Tensor, k: int, out: torch.Tensor, q_len: int = 1,
-         query_start_loc: Optional[torch.Tensor] = None) -> torch.Tensor:
+         query_start_loc: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+         single_workgroup: bool = False) -> torch.Tensor:
     """Positions of the k largest logits among each token's visible keys, ties to the lower position, ascending
-    position order, -1 padding; out int32 [T,k] or [T,1,k] (patch_dsv32_indexer.py:133-146)."""
+    position order, -1 padding; out int32 [T,k] or [T,1,k] (patch_dsv32_indexer.py:133-146).
+    single_workgroup=True runs the variant that needs no scratch memory (one workgroup per token)."""
     _need_cuda(logits, seq_lens, out)
     lib = _lib.load()
     o2 = out.reshape(out.shape[0], -1) if out.dim() == 3 else out
@@ -305,9 +307,14 @@ def topk(logits: torch.Tensor, seq_lens: torch.Tensor, k: int, out: torch.Tensor
     if logits.dtype != torch.float32 or logits.stride(-1) != 1 or o2.dtype != torch.int32 or o2.stride(-1) != 1 or o2.shape[1] < k:
         raise TypeError("topk: fp32 logits [T,S], int32 out [T,>=k]")
     b = seq_lens.numel()
+    ws_ptr, ws_bytes = None, 0
+    if not single_workgroup:
+        need = lib.dsa_topk_workspace_bytes(b, q_len, logits.stride(0))
+        ws = workspace if workspace is not None else _workspace(logits.device, need, tag="topk")
+        ws_ptr, ws_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
     rc = lib.dsa_topk(logits.data_ptr(), logits.stride(0), seq_lens.data_ptr(),
                       query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, k, o2.data_ptr(),
-                      o2.stride(0), _stream(logits))
+                      o2.stride(0), ws_ptr, ws_bytes, _stream(logits))
     _lib.check(rc, "dsa_topk")
     return out
 

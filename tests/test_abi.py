@@ -20,7 +20,7 @@ def test_header_declares_the_path():
     syms = declared_symbols()
     for must in ("mla_cache_write_bf16", "mla_cache_write_fp8", "mla_decode_bf16", "mla_splitkv_reduce",
                  "mla_decode_workspace_bytes", "mla_gather_paged", "mla_merge_states", "dsa_indexer_scores_fp8",
-                 "dsa_topk", "dsa_sparse_decode_bf16", "mlahip_version", "mlahip_last_error_string"):
+                 "dsa_topk", "dsa_topk_workspace_bytes", "dsa_sparse_decode_bf16", "mlahip_version", "mlahip_last_error_string"):
         assert must in syms
 
 
@@ -44,7 +44,7 @@ def test_bad_arguments_return_codes_not_crashes():
     p = ctypes.addressof(buf) // 16 * 16 + 16
     rc = lib.mla_cache_write_bf16(p, 513, p, 64, p, 4, p, 65536, 512, p, 8192, 64, 128, 1, None)   # odd row stride
     assert rc == -2
-    rc = lib.dsa_topk(p, 1 << 23, p, None, 1, 1, 16, p, 16, None)                                  # too many keys per row
+    rc = lib.dsa_topk(p, 1 << 23, p, None, 1, 1, 16, p, 16, None, 0, None)                                  # too many keys per row
     assert rc == -2
     rc = lib.mla_merge_states(p, 1, 1, p, p, 1, 1, p, 7, p, 1, 1, 0, None, 1, 1, 1, None)          # unknown dtype code
     assert rc == -3

@@ -64,20 +64,27 @@ def test_indexer_logits(dev, batch, lo, hi, q_len):
         assert torch.isinf(got[tt, n:pad_end]).all() and (got[tt, n:pad_end] < 0).all()
 
 
-@pytest.mark.parametrize("n,k", [(5000, 2048), (100, 2048), (2048, 2048), (2049, 2048), (70000, 2048), (3000, 7)])
-def test_topk_bit_exact_sets_and_ties(dev, n, k):
-    """Identical scores in, identical index set out; heavy ties (quantised scores) go to the lower index."""
+@pytest.mark.parametrize("single_workgroup", [False, True], ids=["multi-workgroup", "single-workgroup"])
+@pytest.mark.parametrize("n,k", [(5000, 2048), (100, 2048), (2048, 2048), (2049, 2048), (70000, 2048), (3000, 7), (20000, 2048),
+                                 (9001, 300), (131071, 2048)])
+def test_topk_bit_exact_sets_and_ties(dev, n, k, single_workgroup):
+    """Identical scores in, identical index set out; heavy ties (quantised scores) go to the lower index.  Rows 1-3
+    are the degenerate inputs (few distinct values) that take the radix-select paths of both variants; row 4 carries
+    infinities and a huge outlier, which the linear binning must survive."""
     from omni_npu_amd import kernels as K
     g = torch.Generator().manual_seed(n)
-    rows = 4
+    rows = 5
     x = torch.randn(rows, n, generator=g)
+    x[4, 1::97] = float("inf")
+    x[4, 2::89] = float("-inf")
+    x[4, 3] = 1e30
     x[1] = torch.round(x[1] * 4) / 4                       # many exact ties, including +-0
     x[1, ::5] = -0.0
     x[2] = 1.0                                             # all equal: the first k positions win
     x[3, : n // 2] = x[3, n // 2: 2 * (n // 2)]            # every value twice
-    lens = torch.tensor([n, n, n, max(1, n - 3)], dtype=torch.int32)
+    lens = torch.tensor([n, n, n, max(1, n - 3), n], dtype=torch.int32)
     out = torch.full((rows, 1, k), -7, dtype=torch.int32, device=dev)
-    K.topk(x.to(dev), lens.to(dev), k, out)
+    K.topk(x.to(dev), lens.to(dev), k, out, single_workgroup=single_workgroup)
     got = out.cpu().view(rows, k)
     for r in range(rows):
         ref = O.topk_stable(x[r], k, int(lens[r]))
