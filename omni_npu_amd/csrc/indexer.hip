@@ -7,7 +7,7 @@
 // q8 / k8 are float8_e4m3fn (OCP), 128 wide; w already carries the per-(token, head) q scale unless a
 // separate q_scale is passed.  The selection half is dsa_topk (topk.hip).
 //
-// Pure streaming kernel, no LDS: a wavefront walks blocks of 32 keys.  Lane (key = l % 32, half = l / 32)
+// Pure streaming kernel, no LDS: a wavefront walks blocks of 32 keys (its equal share of all blocks of the launch).  Lane (key = l % 32, half = l / 32)
 // loads bytes [64*half, 64*half + 64) of its key row straight from the paged cache and uses them as the B
 // operand of 8 MFMA 32x32x16 fp8 steps per head block (the k order inside a step is free as long as A
 // uses the same one).  A = the query's 64 heads x 128, held in 32 registers.  In the accumulator layout
@@ -18,8 +18,7 @@
 namespace mlahip {
 
 constexpr int kIdxDim = 128;
-constexpr int kIdxKeysPerWave = 512;                  // 16 blocks of 32 keys
-constexpr int kIdxKeysPerWg = 4 * kIdxKeysPerWave;    // 2048
+constexpr int kIdxAhead = 6;                          // key blocks held in registers (5 requested ahead)
 
 struct IndexerParams {
   const uint8_t* q8; int64_t q_st, q_sh;              // bytes
@@ -34,22 +33,76 @@ struct IndexerParams {
   float* logits; int64_t l_st;                        // [T, l_st]
 };
 
-__global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerParams p) {
+__device__ __forceinline__ int idx_wave_sum(int v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+  return v;
+}
+__device__ __forceinline__ int idx_wave_max(int v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v = max(v, __shfl_xor(v, d, 64));
+  return v;
+}
+
+// The 32-key blocks of all query tokens, laid end to end, are dealt out to the wavefronts of the launch in equal
+// contiguous shares (to within one block), whatever the individual context lengths; a share that crosses a token
+// boundary is processed as two (or more) segments.  Every wavefront derives its share from the sequence lengths by
+// itself (two passes: total, scan); there is no LDS and no barrier in this kernel, so wavefronts are independent.
+__global__ __launch_bounds__(256, 1) void dsa_indexer_fp8_kernel(const IndexerParams p) {
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int key_l = lane & 31, half = lane >> 5;
-  const int b = blockIdx.y / p.max_q_len;
-  const int ti = blockIdx.y - b * p.max_q_len;        // query token inside the request
-  int q0, qlen;
-  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
-  if (ti >= qlen) return;
-  const int t = q0 + ti;
-  const int L = p.seq_lens[b];
-  int limit = L - qlen + ti + 1;                       // visible keys (right-down causal)
-  limit = limit < 0 ? 0 : limit;
-  const int key_begin = blockIdx.x * kIdxKeysPerWg + wave * kIdxKeysPerWave;
-  if (key_begin >= limit) return;
-  int key_end = key_begin + kIdxKeysPerWave;
+  const int slots = p.batch * p.max_q_len;
+  // visible keys of token slot s = (request, token inside the request); 0 for slots past a request's length
+  auto limit_of = [&](int s) -> int {
+    const int bb = s / p.max_q_len, tt = s - bb * p.max_q_len;
+    const int ql0 = p.qsl ? p.qsl[bb + 1] - p.qsl[bb] : p.max_q_len;
+    const int ql = ql0 < p.max_q_len ? ql0 : p.max_q_len;
+    if (tt >= ql) return 0;
+    const int lim = p.seq_lens[bb] - ql + tt + 1;
+    return lim < 0 ? 0 : lim;
+  };
+  int seg_s, seg_off, remaining;
+  {
+    int tot = 0;
+    for (int i = lane; i < slots; i += 64) tot += (limit_of(i) + 31) >> 5;
+    tot = __builtin_amdgcn_readfirstlane(idx_wave_sum(tot));
+    const int64_t nw = (int64_t)gridDim.x * 4, me = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t ub = me * tot / nw, ue = (me + 1) * tot / nw;
+    if (ub == ue) return;
+    int carry = 0, s0 = 0, pb0 = 0;
+    for (int base = 0; base < slots; base += 64) {
+      const int i = base + lane;
+      const int c = i < slots ? (limit_of(i) + 31) >> 5 : 0;
+      int pe = c;                                         // inclusive scan
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) { const int v = __shfl_up(pe, d, 64); pe += lane >= d ? v : 0; }
+      pe += carry;
+      const bool le = i < slots && pe <= ub;              // slot i ends at or before my first block
+      s0 += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+      pb0 = max(pb0, idx_wave_max(le ? pe : 0));
+      carry = __builtin_amdgcn_readlane(pe, 63);
+    }
+    seg_s = __builtin_amdgcn_readfirstlane(s0) - 1;
+    seg_off = (int)ub - __builtin_amdgcn_readfirstlane(pb0);
+    remaining = (int)(ue - ub);
+  }
+
+  while (remaining > 0) {
+  seg_s++;
+  if (seg_s >= slots) break;
+  const int b = seg_s / p.max_q_len;
+  const int ti = seg_s - b * p.max_q_len;              // query token inside the request
+  const int limit = limit_of(seg_s);                   // visible keys (right-down causal)
+  const int blk_begin = seg_off;
+  seg_off = 0;
+  int take = ((limit + 31) >> 5) - blk_begin;
+  take = take < remaining ? take : remaining;
+  if (take <= 0) continue;
+  remaining -= take;
+  const int t = (p.qsl ? p.qsl[b] : b * p.max_q_len) + ti;
+  const int key_begin = blk_begin * 32;
+  int key_end = key_begin + take * 32;
   key_end = key_end < limit ? key_end : limit;
 
   // A operand: head = hb*32 + key_l (as row index), bytes [64*half, +64) of that head's query row
@@ -73,51 +126,77 @@ __global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerPa
     }
   }
 
-  auto load_block = [&](int key0, u32x4 (&kb)[4], float& ks) {
+  // Key blocks are requested kIdxAhead - 1 blocks ahead of their use: a block is 4 KiB per wavefront, and only what is in
+  // flight hides the memory latency.  When pages hold a whole number of 32-key blocks the page number of a block is a
+  // scalar (one scalar load of the block table, no dependent vector load in front of the key loads).
+  const bool block_paged = (p.page_size & 31) == 0;
+  int nxt_key0 = key_begin;                             // next block to request; its page and row offset when block_paged
+  int nxt_pg = key_begin / p.page_size;
+  int nxt_off = key_begin - nxt_pg * p.page_size;
+  auto load_block = [&](u32x4 (&kb)[4], float& ks) {
+    const int key0 = nxt_key0;
     int key = key0 + key_l;
-    key = key < limit ? key : limit - 1;               // tail lanes re-read the last visible key
-    int pg = key / p.page_size;
-    const int off = key - pg * p.page_size;
-    pg = pg < p.max_blocks ? pg : p.max_blocks - 1;
-    int64_t blk = p.block_table[(int64_t)b * p.bt_stride + pg];
-    blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
-    const uint8_t* row = p.k8 + blk * p.k_sp + (int64_t)off * p.k_sr + half * 64;
+    key = key < limit ? key : limit - 1;               // tail lanes re-read the last visible key (same block)
+    const uint8_t* row;
+    const float* sc;
+    if (block_paged) {
+      const int pgc = nxt_pg < p.max_blocks ? nxt_pg : p.max_blocks - 1;
+      int64_t blk = ((const __attribute__((address_space(4))) int32_t*)p.block_table)[(int64_t)b * p.bt_stride + pgc];
+      blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
+      const int off = nxt_off + (key - key0);
+      row = p.k8 + blk * p.k_sp + (int64_t)off * p.k_sr + half * 64;
+      sc = p.k_scale + blk * p.ks_sp + off;
+      nxt_off += 32;
+      if (nxt_off >= p.page_size) { nxt_off = 0; nxt_pg++; }
+    } else {
+      int pg = key / p.page_size;
+      const int off = key - pg * p.page_size;
+      pg = pg < p.max_blocks ? pg : p.max_blocks - 1;
+      int64_t blk = p.block_table[(int64_t)b * p.bt_stride + pg];
+      blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
+      row = p.k8 + blk * p.k_sp + (int64_t)off * p.k_sr + half * 64;
+      sc = p.k_scale + blk * p.ks_sp + off;
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) kb[j] = *(const u32x4*)(row + j * 16);
-    ks = p.k_scale[blk * p.ks_sp + off];
+    ks = *sc;
+    nxt_key0 += 32;
   };
 
-  u32x4 kb[4], kn[4];
-  float ks, ksn;
-  load_block(key_begin, kb, ks);
-  for (int key0 = key_begin; key0 < key_end; key0 += 32) {
-    const bool more = key0 + 32 < key_end;
-    if (more) load_block(key0 + 32, kn, ksn);
-    f32x16 c0, c1;
+  u32x4 kb[kIdxAhead][4];
+  float ks[kIdxAhead];
 #pragma unroll
-    for (int r = 0; r < 16; r++) { c0[r] = 0.f; c1[r] = 0.f; }
+  for (int i = 0; i < kIdxAhead - 1; i++)
+    if (key_begin + 32 * i < key_end) load_block(kb[i], ks[i]);
+  for (int g = 0; key_begin + 32 * g < key_end; g += kIdxAhead) {
 #pragma unroll
-    for (int kk = 0; kk < 8; kk++) {
-      const u32x4 v = kb[kk >> 1];
-      const long bop = (kk & 1) ? (long)(((uint64_t)v[3] << 32) | v[2]) : (long)(((uint64_t)v[1] << 32) | v[0]);
-      c0 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[0][kk], bop, c0, 0, 0, 0);
-      c1 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[1][kk], bop, c1, 0, 0, 0);
-    }
-    float acc = 0.f;
+    for (int st = 0; st < kIdxAhead; st++) {                // ring slot = step: g is a multiple of kIdxAhead
+      const int key0 = key_begin + 32 * (g + st);
+      if (key0 >= key_end) break;
+      if (key0 + 32 * (kIdxAhead - 1) < key_end)
+        load_block(kb[(st + kIdxAhead - 1) % kIdxAhead], ks[(st + kIdxAhead - 1) % kIdxAhead]);
+      f32x16 c0, c1;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      acc = fmaf(wr[0][r], fmaxf(c0[r], 0.f), acc);
-      acc = fmaf(wr[1][r], fmaxf(c1[r], 0.f), acc);
-    }
-    acc += xor32(acc);
-    const int key = key0 + key_l;
-    if (half == 0) p.logits[(int64_t)t * p.l_st + key] = key < limit ? acc * ks : -INFINITY;
-    if (more) {
+      for (int r = 0; r < 16; r++) { c0[r] = 0.f; c1[r] = 0.f; }
 #pragma unroll
-      for (int j = 0; j < 4; j++) kb[j] = kn[j];
-      ks = ksn;
+      for (int kk = 0; kk < 8; kk++) {
+        const u32x4 v = kb[st][kk >> 1];
+        const long bop = (kk & 1) ? (long)(((uint64_t)v[3] << 32) | v[2]) : (long)(((uint64_t)v[1] << 32) | v[0]);
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[0][kk], bop, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[1][kk], bop, c1, 0, 0, 0);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        acc = fmaf(wr[0][r], fmaxf(c0[r], 0.f), acc);
+        acc = fmaf(wr[1][r], fmaxf(c1[r], 0.f), acc);
+      }
+      acc += xor32(acc);
+      const int key = key0 + key_l;
+      if (half == 0) p.logits[(int64_t)t * p.l_st + key] = key < limit ? acc * ks[st] : -INFINITY;
     }
   }
+  }  // segments
 }
 
 // Per-row e4m3 quantisation of 128-wide bf16 rows (one fp32 scale = amax/448 per row, 1.0 for an all-zero row),
@@ -197,7 +276,18 @@ extern "C" int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_
   p.seq_lens = seq_lens; p.qsl = query_start_loc;
   p.batch = batch; p.max_q_len = max_q_len; p.num_heads = num_heads; p.page_size = page_size; p.num_pages = num_pages;
   p.logits = logits; p.l_st = logits_stride;
-  dim3 grid((max_seq_len + kIdxKeysPerWg - 1) / kIdxKeysPerWg, batch * max_q_len);
-  hipLaunchKernelGGL(dsa_indexer_fp8_kernel, grid, dim3(256), 0, stream, p);
+  // two workgroups per compute unit (what the register budget allows), never more wavefronts than 32-key blocks
+  static int num_cus = 0;
+  if (num_cus == 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&num_cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        num_cus <= 0)
+      num_cus = 256;
+  }
+  const int64_t max_blocks_total = (int64_t)batch * max_q_len * ((max_seq_len + 31) / 32);
+  int64_t wgs = 2 * (int64_t)num_cus;
+  if (wgs * 4 > max_blocks_total) wgs = (max_blocks_total + 3) / 4;
+  if (wgs < 1) wgs = 1;
+  hipLaunchKernelGGL(dsa_indexer_fp8_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p);
   return check_launch("dsa_indexer_fp8_kernel");
 }
