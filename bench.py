@@ -41,6 +41,85 @@ def algorithmic_bytes(case, heads):
     return dict(kv=kv, q=q, out=o, cache_write=wr, tables=tables, total=kv + q + o + wr + tables)
 
 
+def bench_dsa(K, dev, args):
+    """configs[3]: lightning indexer (64 fp8 heads x 128) over contexts uniform[32768, 65536], batch 32, top-2048,
+    sparse absorbed MLA over the selected rows.  Per-stage device times (HIP events on the launch stream)."""
+    g = torch.Generator().manual_seed(args.seed)
+    B, H, N, k = 32, 64, 128, 2048
+    lens = torch.randint(32768, 65537, (B,), generator=g).to(torch.int32)
+    nblk_seq = (lens + 127) // 128
+    nblk = int(nblk_seq.sum())
+    perm = torch.randperm(nblk, generator=g)
+    bt = torch.zeros(B, int(nblk_seq.max()), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        n = int(nblk_seq[b])
+        bt[b, :n] = perm[o:o + n].to(torch.int32)
+        o += n
+    # fp8-e4m3 bit patterns of finite positive values for keys and queries, fp32 scales and head weights N(0,1)
+    k8 = torch.randint(0, 120, (nblk, 128, 128), dtype=torch.uint8, generator=g).to(dev)
+    ks = torch.rand(nblk, 128, generator=g).to(dev)
+    q8 = torch.randint(0, 120, (B, H, 128), dtype=torch.uint8, generator=g).to(dev)
+    w = torch.randn(B, H, generator=g).to(dev)
+    nope = torch.randn(nblk, 128, 512, device=dev).bfloat16()
+    rope = torch.randn(nblk, 128, 64, device=dev).bfloat16()
+    qn = torch.randn(B, N, 512, device=dev).bfloat16()
+    qr = torch.randn(B, N, 64, device=dev).bfloat16()
+    btd, lensd = bt.to(dev), lens.to(dev)
+    max_len = int(lens.max())
+    logits = torch.empty(B, K.indexer_logits_stride(max_len), device=dev)
+    idx = torch.empty(B, k, dtype=torch.int32, device=dev)
+    rows = torch.empty(B, k, dtype=torch.int32, device=dev)
+    counts = torch.empty(B, dtype=torch.int32, device=dev)
+    out = torch.empty(B, N, 512, dtype=torch.bfloat16, device=dev)
+    splits = args.splits or K.default_num_splits(B, 1, N, k)
+    stages = [
+        ("indexer", lambda: K.indexer_scores(q8, w, k8, ks, btd, lensd, logits, max_seq_len=max_len)),
+        ("topk", lambda: K.topk(logits, lensd, k, idx)),
+        ("build_rows", lambda: K.build_sparse_rows(idx, btd, lensd, 128, nblk, rows, counts)),
+        ("sparse_decode", lambda: K.sparse_decode(qn, qr, nope, rope, rows, counts, 192 ** -0.5, out, num_splits=splits)),
+    ]
+
+    def whole():
+        for _, f in stages:
+            f()
+
+    def ev_time(fn, n):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(e) * 1e3 / n
+
+    total = ev_time(whole, args.steps)
+    # a stage timed alone in a launch loop is bounded below by the host's launch rate (about 10 us a call): the small
+    # stages read high here, the per-kernel durations of a rocprofv3 kernel trace are the better figure for them
+    per_stage = {name: round(ev_time(f, args.steps), 2) for name, f in stages}
+    sum_l = int(lens.sum())
+    idx_bytes = sum_l * (128 + 4) + B * H * (128 + 4) + sum_l * 4          # fp8 keys + scales, queries + weights, logits out
+    sparse_bytes = B * k * 576 * 2 + B * N * (576 + 512) * 2
+    ideal_us = (idx_bytes + sum_l * 4 + sparse_bytes) / (HBM_PEAK_GBS * 1e9) * 1e6
+    return {
+        "metric": "DSA decode us/layer (B=32, ctx 32k-64k, indexer 64 fp8 heads + top-2048 + sparse MLA 128 heads)",
+        "value": round(total, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "fp8 (indexer) / bf16 (attention)", "data": "synthetic",
+        "config": {"workload": "configs[3]: DSA sparse decode path", "batch": B, "index_heads": H, "heads": N, "topk": k,
+                   "seq_lens": "uniform[32768,65536]", "sum_seq_len": sum_l, "kv_splits": splits, "seed": args.seed},
+        "stage_us_launch_loop": per_stage, "launch": "eager launches",
+        "roofline": {"kernel": "dsa_indexer_fp8_kernel", "bound": "hbm",
+                     "achieved": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": idx_bytes},
+        "chain_roofline": {"hbm_bytes": idx_bytes + sum_l * 4 + sparse_bytes, "ideal_us_at_8TBs": round(ideal_us, 2),
+                           "frac": round(ideal_us / total, 4)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -54,6 +133,14 @@ def main():
     ap.add_argument("--q-len", type=int, default=1)
     ap.add_argument("--splits", type=int, default=0, help="KV splits per sequence (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true",
+                    help="replay the step as a captured HIP graph instead of launching its kernels one by one (measured "
+                         "slower on this ROCm: replay adds more between kernels than the launches it saves)")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
+                         "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -65,6 +152,16 @@ def main():
 
     from omni_npu_amd import kernels as K
     dev = torch.device("cuda:0")
+    if args.copy_probe:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    if args.workload == "dsa":
+        print(json.dumps(bench_dsa(K, dev, args)))
+        return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len
     t = b * q_len
@@ -79,6 +176,17 @@ def main():
         K.cache_write(g["new_c"], g["new_r"], g["slot_mapping"], g["nope"], g["rope"])
         K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], g["block_table"], g["seq_lens"], case["scale"], out_v,
                  q_len=q_len, num_splits=splits, workspace=ws)
+
+    eager_step = step
+    if args.graph:
+        # the product's decode path can replay a captured HIP graph (compilation/acl_graph.py)
+        for _ in range(3):
+            eager_step()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            eager_step()
+        step = graph.replay
 
     for _ in range(args.warmup):
         step()
@@ -120,12 +228,12 @@ def main():
                    "q_len": q_len, "seq_lens": f"uniform[{args.len_lo},{args.len_hi}]", "sum_seq_len": sum_l,
                    "page": 128, "kv_splits": splits, "seed": args.seed},
         "step_us": {"host_wall": round(us_per_step, 2), "device_avg": round(dev_step_avg, 2),
-                    "device_median": round(dev_step_med, 2)},
+                    "device_median": round(dev_step_med, 2), "launch": "hip graph replay" if args.graph else "eager launches"},
         "step_tflops": round(flops / (dev_step_avg * 1e-6) / 1e12, 1),
         "step_hbm_gbs": round(ab["total"] / (dev_step_avg * 1e-6) / 1e9, 1),
         "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                                     / (dev_step_avg * 1e-6), 4),
-        "roofline": {"kernel": "mla_decode_bf16_kernel", "bound": "hbm", "achieved": round(achieved, 1),
+        "roofline": {"kernel": "mla_decode_v2_kernel<false>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                      "kernel_us_avg": round(k_avg, 2), "kernel_us_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),

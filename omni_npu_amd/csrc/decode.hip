@@ -478,7 +478,8 @@ extern "C" size_t mla_decode_workspace_bytes(int32_t batch, int32_t max_q_len, i
   // batch * num_splits chunks, and one more partial for every sequence boundary inside a chunk: batch * (num_splits + 1) partials in all
   const size_t rows = (size_t)batch * ((size_t)num_splits + 1) * max_q_len * num_heads;
   // fp16 partials, fp32 log-sum-exps, and per row a correction record (fp32 factor + cache address)
-  return rows * kDNope * sizeof(_Float16) + rows * (2 * sizeof(float) + sizeof(void*));
+  // ... and two partial numbers per sequence
+  return rows * kDNope * sizeof(_Float16) + rows * (2 * sizeof(float) + sizeof(void*)) + (size_t)batch * 2 * sizeof(int32_t);
 }
 
 // first-generation kernel for the bf16 cache too (comparisons only)
@@ -557,6 +558,7 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
     v.batch = p.batch; v.max_q_len = p.max_q_len; v.num_heads = p.num_heads; v.num_pages = p.num_pages;
     v.scale_log2 = p.scale_log2; v.o_part = p.o_part; v.lse_part = p.lse_part;
     v.corr_scale = p.lse_part + rows; v.corr_row = (const __bf16**)(p.lse_part + 2 * rows);
+    v.seg_ids = (int32_t*)(p.lse_part + 4 * rows);
     v.sparse_rows = p.sparse_rows; v.sparse_stride = p.sparse_stride; v.page_size = p.page_size;
     return launch_decode_v2(v, sparse_rows != nullptr, dim3((unsigned)(batch * num_splits), 1, grid.z), stream);
   }
@@ -604,6 +606,7 @@ extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes,
     ChunkReduceParams cp;
     cp.o_part = (const _Float16*)workspace; cp.lse_part = (const float*)((const _Float16*)workspace + rows * kDNope);
     cp.corr_scale = cp.lse_part + rows; cp.corr_row = (const __bf16* const*)(cp.lse_part + 2 * rows);
+    cp.seg_ids = (const int32_t*)(cp.lse_part + 4 * rows);
     cp.seq_lens = seq_lens; cp.qsl = query_start_loc;
     cp.batch = batch; cp.max_q_len = max_q_len; cp.num_heads = num_heads; cp.num_chunks = batch * num_splits;
     cp.out = (__bf16*)out; cp.out_st = out_stride_t; cp.out_sh = out_stride_h;

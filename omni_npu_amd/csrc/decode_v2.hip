@@ -74,6 +74,8 @@ __device__ __forceinline__ float half_sum(float v) {
 }
 
 __device__ __forceinline__ int v2_num_blocks(int len) { return len > 0 ? (len + kBlk - 1) / kBlk : 0; }
+constexpr int kSegCost = 8;                                // start-up cost of a segment, in blocks (about 19 us / 2.3 us)
+__device__ __forceinline__ int v2_work_units(int len) { return len > 0 ? (len + kBlk - 1) / kBlk + kSegCost : 0; }
 __device__ __forceinline__ int wave_sum_i32(int v) {
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
@@ -105,46 +107,57 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const uint32_t lds0 = lds_addr_of(lds);
 
   // ---- which blocks are mine ----
-  // The 32-token blocks of all sequences, laid end to end, are cut into gridDim.x chunks of equal size (to within one
-  // block), whatever the individual sequence lengths: chunk c covers global blocks [c*T/G, (c+1)*T/G).  A chunk that
+  // Work is measured in units of one 32-token block; starting a segment (query load, first copies, epilogue, partial
+  // write) costs about kSegCost of them.  Every non-empty sequence is laid out as kSegCost units of start-up followed by
+  // its blocks, the sequences end to end, and that line is cut into gridDim.x chunks of equal length: chunk c covers
+  // units [c*T/G, (c+1)*T/G), and a chunk that holds the start of a sequence gets that many fewer blocks.  A chunk that
   // crosses a sequence boundary is processed as two (or more) segments; the segment of sequence b in chunk c writes
   // partial number c + b, so the partials of one sequence are consecutive and mla_chunk_reduce_kernel finds them with
   // the same arithmetic.  Every wavefront derives the plan by itself from the sequence lengths (two passes: total, scan).
-  int seg_b, seg_off, remaining;
+  int seg_b;
+  int64_t v_cur, v_end, v_seq;                                // my units [v_cur, v_end); first unit of sequence seg_b + 1
   {
     int tot = 0;
-    for (int i = lane; i < p.batch; i += 64) tot += v2_num_blocks(p.seq_lens[i]);
+    for (int i = lane; i < p.batch; i += 64) tot += v2_work_units(p.seq_lens[i]);
     tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
     const int64_t cb = (int64_t)chunk * tot / gridDim.x, ce = (int64_t)(chunk + 1) * tot / gridDim.x;
     if (cb == ce) return;
     int carry = 0, b0 = 0, pb0 = 0;
     for (int base = 0; base < p.batch; base += 64) {
       const int i = base + lane;
-      const int c = i < p.batch ? v2_num_blocks(p.seq_lens[i]) : 0;
-      const int pe = wave_incl_scan_i32(c, lane) + carry;     // blocks of sequences 0..i
-      const bool le = i < p.batch && pe <= cb;                // sequence i ends at or before my first block
+      const int c = i < p.batch ? v2_work_units(p.seq_lens[i]) : 0;
+      const int pe = wave_incl_scan_i32(c, lane) + carry;     // units of sequences 0..i
+      const bool le = i < p.batch && pe <= cb;                // sequence i ends at or before my first unit
       b0 += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
       pb0 = max(pb0, wave_max_i32(le ? pe : 0));
       carry = __builtin_amdgcn_readlane(pe, 63);
     }
     seg_b = __builtin_amdgcn_readfirstlane(b0) - 1;
-    seg_off = (int)cb - __builtin_amdgcn_readfirstlane(pb0);
-    remaining = (int)(ce - cb);
+    v_seq = __builtin_amdgcn_readfirstlane(pb0);
+    v_cur = cb;
+    v_end = ce;
   }
 
-  while (remaining > 0) {
+  while (v_cur < v_end) {
   seg_b++;
   if (seg_b >= p.batch) break;
   const int b = seg_b;
   const int L = p.seq_lens[b];
-  const int blk_begin = seg_off;
-  seg_off = 0;
-  int take = v2_num_blocks(L) - blk_begin;
-  take = take < remaining ? take : remaining;
-  if (take <= 0) continue;
-  remaining -= take;
-  const int blk_end = blk_begin + take;
-  const int nb = take;
+  const int64_t v_b = v_seq;                                  // first unit of sequence b
+  v_seq += v2_work_units(L);
+  const int64_t v_hi = v_seq < v_end ? v_seq : v_end;
+  int blk_begin = (int)(v_cur - v_b) - kSegCost;
+  int blk_end = (int)(v_hi - v_b) - kSegCost;
+  blk_begin = blk_begin < 0 ? 0 : blk_begin;
+  blk_end = blk_end < 0 ? 0 : blk_end;
+  v_cur = v_hi;
+  const int nb = blk_end - blk_begin;
+  if (nb <= 0) continue;
+  // the merge kernel finds the partials of a sequence between the numbers its first and its last segment leave here
+  if (threadIdx.x == 0) {
+    if (blk_begin == 0) p.seg_ids[2 * b] = chunk + b;
+    if (blk_end == v2_num_blocks(L)) p.seg_ids[2 * b + 1] = chunk + b;
+  }
   lds_barrier();                                              // the previous segment's epilogue is done with the buffers
 
   int q0, qlen;
@@ -672,82 +685,133 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   }  // segments
 }
 
-// N-way merge of the partials of one query row (src/omni_npu/attention/ops.py:109-141), for the chunk layout written
-// by mla_decode_v2_kernel: one wavefront per row.  The partials of sequence b are those of the chunks that overlap its
-// blocks, numbered chunk + b.
+// N-way merge of the partials of the query rows (src/omni_npu/attention/ops.py:109-141), for the chunk layout written
+// by mla_decode_v2_kernel.  The partials of sequence b are those of the chunks that hold blocks of it, numbered
+// chunk + b.  A wavefront merges kRedRows consecutive rows of one sequence (lane l owns columns 8l..8l+7): it derives
+// the chunk list once, then asks for everything it needs of up to kRedParts partials of all its rows before it uses
+// any of it - the kernel is a chain of dependent memory round trips, and this keeps the chain at two.
+constexpr int kRedRows = 2;
+constexpr int kRedParts = 6;
 __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
   const int lane = threadIdx.x & 63;
   const int r_max = p.max_q_len * p.num_heads;
-  const int64_t gr = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (gr >= (int64_t)p.batch * r_max) return;
-  const int b = gr / r_max;
-  const int row = gr - (int64_t)b * r_max;
+  const int groups = (r_max + kRedRows - 1) / kRedRows;     // row groups per sequence
+  const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (gw >= (int64_t)p.batch * groups) return;
+  const int b = (int)(gw / groups);
+  const int row0 = (int)(gw - (int64_t)b * groups) * kRedRows;
   int q0, qlen;
   if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
   qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
-  if (row >= qlen * p.num_heads) return;
-  const int t_local = row / p.num_heads;
-  const int head = row - t_local * p.num_heads;
+  const int rows = qlen * p.num_heads;
+  if (row0 >= rows) return;
 
-  int tot_blocks = 0, before = 0;
+  int tot_units = 0, before = 0;
   for (int i = lane; i < p.batch; i += 64) {
-    const int c = v2_num_blocks(p.seq_lens[i]);
-    tot_blocks += c;
+    const int c = v2_work_units(p.seq_lens[i]);
+    tot_units += c;
     before += i < b ? c : 0;
   }
-  tot_blocks = wave_sum_i32(tot_blocks);
-  before = wave_sum_i32(before);
-  const int mine = v2_num_blocks(p.seq_lens[b]);
-  const int64_t G = p.num_chunks, T = tot_blocks;
+  tot_units = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot_units));
+  before = __builtin_amdgcn_readfirstlane(wave_sum_i32(before));
+  const int mine = v2_work_units(p.seq_lens[b]);
+  const int64_t G = p.num_chunks, T = tot_units;
+  // does chunk c hold blocks of this sequence (units [before, before + mine), the first kSegCost of them start-up)?
+  auto holds_blocks = [&](int64_t c) -> bool {
+    const int64_t cb = c * T / G, ce = (c + 1) * T / G;
+    const int64_t lo = cb > before ? cb : before, hi = ce < before + mine ? ce : before + mine;
+    int64_t rlo = lo - before - kSegCost, rhi = hi - before - kSegCost;
+    rlo = rlo < 0 ? 0 : rlo;
+    rhi = rhi < 0 ? 0 : rhi;
+    return rhi > rlo;
+  };
 
-  float m = -INFINITY;
-  float tot = 0.f;
   typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-  float a[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  float m[kRedRows], tot[kRedRows], a[kRedRows][8];
+#pragma unroll
+  for (int j = 0; j < kRedRows; j++) {
+    m[j] = -INFINITY;
+    tot[j] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) a[j][e] = 0.f;
+  }
   if (mine > 0) {
-    // chunk c starts at block floor(c*T/G): the chunk holding block x is the largest c with c*T < (x+1)*G
-    const int c_first = (int)((((int64_t)before + 1) * G - 1) / T);
-    const int c_last = (int)((((int64_t)before + mine) * G - 1) / T);
-    for (int c = c_first; c <= c_last; c++) {
-      if (c * T / G == (c + 1) * T / G) continue;            // empty chunk: wrote nothing
-      float l = p.lse_part[(int64_t)(c + b) * r_max + row];
-      l = l == INFINITY ? -INFINITY : l;
-      m = fmaxf(m, l);
+    // With at least one unit per chunk every chunk between the sequence's first and last segment holds blocks of it, and
+    // the split kernel left those two partial numbers behind.  Otherwise (tiny workloads) some chunks are empty and the
+    // chunk boundaries are worked out here: chunk c starts at unit floor(c*T/G), the chunk holding unit x is the
+    // largest c with c*T < (x+1)*G.
+    const bool dense_chunks = T >= G;
+    int c, c_last;
+    if (dense_chunks) {
+      c = p.seg_ids[2 * b] - b;
+      c_last = p.seg_ids[2 * b + 1] - b;
+    } else {
+      c = (int)((((int64_t)before + 1) * G - 1) / T);
+      c_last = (int)((((int64_t)before + mine) * G - 1) / T);
     }
-    if (m != -INFINITY) {
-      for (int c = c_first; c <= c_last; c++) {
-        if (c * T / G == (c + 1) * T / G) continue;
-        const int64_t pr = (int64_t)(c + b) * r_max + row;
-        const float l = p.lse_part[pr];
-        if (l == INFINITY || l == -INFINITY) continue;       // nothing visible in that segment
-        const float w = __expf(l - m);
-        tot += w;
-        const h8 v = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
+    while (c <= c_last) {
+      int64_t part[kRedParts];                               // partial numbers of this round (uniform), -1 = none
+      int np = 0;
 #pragma unroll
-        for (int e = 0; e < 8; e++) a[e] += (float)v[e] * w;
-        // the split kernel rounded this segment's dominant probability to bf16: put the difference back
-        const float cs = p.corr_scale[pr];
-        if (cs != 0.f) {
-          const bf16x8 kv = *(const bf16x8*)(p.corr_row[pr] + lane * 8);
-#pragma unroll
-          for (int e = 0; e < 8; e++) a[e] += (float)kv[e] * (w * cs);
-        }
+      for (int q = 0; q < kRedParts; q++) {
+        while (c <= c_last && !dense_chunks && !holds_blocks(c)) c++;     // wrote nothing for this sequence
+        part[q] = c <= c_last ? (int64_t)(c + b) * r_max + row0 : -1;
+        if (c <= c_last) { np++; c++; }
       }
+      float lse[kRedRows][kRedParts], cs[kRedRows][kRedParts];
+      h8 v[kRedRows][kRedParts];
+#pragma unroll
+      for (int q = 0; q < kRedParts; q++)
+#pragma unroll
+        for (int j = 0; j < kRedRows; j++) {
+          const bool on = q < np && row0 + j < rows;
+          const int64_t pr = on ? part[q] + j : 0;
+          lse[j][q] = on ? p.lse_part[pr] : -INFINITY;
+          cs[j][q] = on ? p.corr_scale[pr] : 0.f;
+          v[j][q] = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
+        }
+#pragma unroll
+      for (int q = 0; q < kRedParts; q++)
+#pragma unroll
+        for (int j = 0; j < kRedRows; j++) {
+          float l = lse[j][q];
+          if (l == INFINITY || l == -INFINITY) continue;     // nothing visible in that segment (or no such partial)
+          const float mn = fmaxf(m[j], l);
+          const float so = __expf(m[j] - mn), w = __expf(l - mn);   // m = -inf at first: exp(-inf) = 0 rescales the zeros
+          m[j] = mn;
+          tot[j] = tot[j] * so + w;
+#pragma unroll
+          for (int e = 0; e < 8; e++) a[j][e] = a[j][e] * so + (float)v[j][q][e] * w;
+          // the split kernel rounded this segment's dominant probability to bf16: put the difference back
+          if (cs[j][q] != 0.f) {
+            const bf16x8 kv = *(const bf16x8*)(p.corr_row[part[q] + j] + lane * 8);
+#pragma unroll
+            for (int e = 0; e < 8; e++) a[j][e] += (float)kv[e] * (w * cs[j][q]);
+          }
+        }
     }
   }
-  const float inv = tot > 0.f ? 1.f / tot : 0.f;
-  __bf16* out = p.out + (int64_t)(q0 + t_local) * p.out_st + (int64_t)head * p.out_sh;
-  bf16x8 o8;
 #pragma unroll
-  for (int e = 0; e < 8; e++) o8[e] = (__bf16)(a[e] * inv);
-  *(bf16x8*)(out + lane * 8) = o8;
-  if (p.lse_out && lane == 0)
-    p.lse_out[(int64_t)(q0 + t_local) * p.lse_st + head] = tot > 0.f ? __logf(tot) + m : -INFINITY;
+  for (int j = 0; j < kRedRows; j++) {
+    const int row = row0 + j;
+    if (row >= rows) break;
+    const int t_local = row / p.num_heads;
+    const int head = row - t_local * p.num_heads;
+    const float inv = tot[j] > 0.f ? 1.f / tot[j] : 0.f;
+    __bf16* out = p.out + (int64_t)(q0 + t_local) * p.out_st + (int64_t)head * p.out_sh;
+    bf16x8 o8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o8[e] = (__bf16)(a[j][e] * inv);
+    *(bf16x8*)(out + lane * 8) = o8;
+    if (p.lse_out && lane == 0)
+      p.lse_out[(int64_t)(q0 + t_local) * p.lse_st + head] = tot[j] > 0.f ? __logf(tot[j]) + m[j] : -INFINITY;
+  }
 }
 
 int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
-  const int64_t nrows = (int64_t)p.batch * p.max_q_len * p.num_heads;
-  hipLaunchKernelGGL(mla_chunk_reduce_kernel, dim3((unsigned)((nrows + 3) / 4)), dim3(256), 0, stream, p);
+  const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
+  const int64_t waves = (int64_t)p.batch * ((r_max + kRedRows - 1) / kRedRows);
+  hipLaunchKernelGGL(mla_chunk_reduce_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, p);
   return check_launch("mla_chunk_reduce_kernel");
 }
 

@@ -19,11 +19,13 @@ struct DecodeV2Params {
   float* lse_part;               // [chunks + B, R_max], natural log
   float* corr_scale;             // [chunks + B, R_max]: (p - bf16(p)) / l of the row's dominant key, or 0
   const __bf16** corr_row;       // [chunks + B, R_max]: that key's latent vector in the cache
+  int32_t* seg_ids;              // [B][2]: partial number of the sequence's first / last segment
   const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
 };
 
 struct ChunkReduceParams {
   const _Float16* o_part; const float* lse_part; const float* corr_scale; const __bf16* const* corr_row;
+  const int32_t* seg_ids;
   const int32_t* seq_lens; const int32_t* qsl;
   int32_t batch, max_q_len, num_heads, num_chunks;
   __bf16* out; int64_t out_st, out_sh;

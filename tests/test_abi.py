@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol():
 def test_bad_arguments_return_codes_not_crashes():
     from omni_npu_amd import _lib
     lib = _lib.load()
-    assert lib.mla_decode_workspace_bytes(64, 1, 128, 4) == 64 * (4 + 1) * 128 * (512 * 2 + 4 + 4 + 8)
+    assert lib.mla_decode_workspace_bytes(64, 1, 128, 4) == 64 * (4 + 1) * 128 * (512 * 2 + 4 + 4 + 8) + 64 * 8
     assert lib.mla_decode_workspace_bytes(0, 1, 128, 4) == 0
     rc = lib.mla_cache_write_bf16(None, 512, None, 64, None, 4, None, 0, 0, None, 0, 0, 128, 1, None)
     assert rc == -1 and b"null" in lib.mlahip_last_error_string()
