@@ -120,6 +120,75 @@ def bench_dsa(K, dev, args):
     }
 
 
+def bench_prefill(K, dev, args):
+    """configs[2]: non-absorbed chunked prefill, 4 sequences, a 2048-token query chunk each over 16384 cached tokens,
+    128 heads (qk 128 + 64 rope, v 128).  Times the attention kernels (context part, causal suffix, merge) and, beside
+    them, the latent gather and the torch GEMM that up-projects the latent to K/V."""
+    g = torch.Generator().manual_seed(args.seed)
+    B, N, Q, C = 4, 128, 2048, 16384
+    scale = 192 ** -0.5
+    bf = lambda *shape: torch.randn(*shape, generator=g).bfloat16().to(dev)
+    qn, qp = bf(B * Q, N, 128), bf(B * Q, N, 64)
+    # suffix (the chunk's own keys) and context (the cached prefix), already up-projected
+    ks_n, ks_p, vs = bf(B * Q, N, 128), bf(B * Q, 64), bf(B * Q, N, 128)
+    kc_n = torch.randn(B * C, N, 128, device=dev).bfloat16()
+    kc_p = torch.randn(B * C, 64, device=dev).bfloat16()
+    vc = torch.randn(B * C, N, 128, device=dev).bfloat16()
+    cu_q = torch.arange(0, (B + 1) * Q, Q, dtype=torch.int32, device=dev)
+    cu_c = torch.arange(0, (B + 1) * C, C, dtype=torch.int32, device=dev)
+    o_s = torch.empty(B * Q, N, 128, dtype=torch.bfloat16, device=dev)
+    o_c = torch.empty_like(o_s)
+    o = torch.empty_like(o_s)
+    l_s = torch.empty(B * Q, N, dtype=torch.float32, device=dev)
+    l_c = torch.empty_like(l_s)
+    # latent cache of the prefix for the gather + up-projection leg
+    pages = B * C // 128
+    nope = torch.randn(pages, 128, 512, device=dev).bfloat16()
+    rope = torch.randn(pages, 128, 64, device=dev).bfloat16()
+    bt = torch.randperm(pages, generator=g).to(torch.int32).view(B, C // 128).to(dev)
+    gathered = torch.empty(B * C, 576, dtype=torch.bfloat16, device=dev)
+    w_up = (torch.randn(512, N * 256, generator=g) * 0.02).bfloat16().to(dev)
+
+    stages = [
+        ("context_attention", lambda: K.prefill_varlen(qn, qp, kc_n, kc_p, vc, cu_q, cu_c, Q, scale, False, o_c, l_c)),
+        ("suffix_attention", lambda: K.prefill_varlen(qn, qp, ks_n, ks_p, vs, cu_q, cu_q, Q, scale, True, o_s, l_s)),
+        ("merge", lambda: K.merge_states(o_c, l_c, o_s, l_s, o)),
+        ("gather_latent", lambda: K.gather_paged(nope, rope, gathered, bt, cu_c, B)),
+        ("kv_up_proj_torch_gemm", lambda: torch.matmul(gathered[:, :512], w_up)),
+    ]
+
+    def ev_time(fn, n):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(e) * 1e3 / n
+
+    n = max(3, min(args.steps, 10))
+    per = {name: round(ev_time(f, n), 1) for name, f in stages}
+    fl_c = B * N * Q * C * 2 * (192 + 128)
+    fl_s = B * N * Q * (Q + 1) // 2 * 2 * (192 + 128)
+    attn_us = per["context_attention"] + per["suffix_attention"] + per["merge"]
+    return {
+        "metric": "MLA chunked prefill us/layer (4 x 2048-token chunk over 16384 cached tokens, 128 heads, bf16, attention kernels)",
+        "value": round(attn_us, 1), "unit": "us/layer", "n_gpus": 1, "steps": n, "warmup": 2, "higher_is_better": False,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[2]: non-absorbed chunked prefill", "sequences": B, "chunk": Q, "prefix": C, "heads": N,
+                   "seed": args.seed},
+        "stage_us": per,
+        "roofline": {"kernel": "mla_prefill_varlen_kernel", "bound": "mfma",
+                     "achieved": round((fl_c + fl_s) / ((per["context_attention"] + per["suffix_attention"]) * 1e-6) / 1e12, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round((fl_c + fl_s) / ((per["context_attention"] + per["suffix_attention"]) * 1e-6) / 1e12
+                                   / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "algorithmic_flops": fl_c + fl_s},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,8 +208,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa"],
-                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -161,6 +230,9 @@ def main():
         del src, dst
     if args.workload == "dsa":
         print(json.dumps(bench_dsa(K, dev, args)))
+        return
+    if args.workload == "prefill":
+        print(json.dumps(bench_prefill(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len
