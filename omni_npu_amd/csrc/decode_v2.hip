@@ -8,23 +8,24 @@
 // Here the two products are partitioned differently:
 //   S^T = K Q^T      wave w owns query rows 32w..32w+31 (its 576-wide query stays in registers), all 32 tokens of a block;
 //   O^T += V^T P^T   wave w owns output columns d in [128w, 128w+128) for ALL 128 rows: a V^T fragment is read once and
-//                    feeds four MFMAs (one per row group), and the four P^T blocks (2 KiB each, bf16) plus the rescale
-//                    factors travel through LDS once per block.
+//                    feeds four MFMAs (one per row group), and the four P^T blocks (2 KiB each, bf16) plus a restart
+//                    flag per row travel through LDS once per block.
 // Per 32 tokens a wave issues 36 + 16 + 8 + ~4 LDS instructions instead of 100, for the same 68 MFMAs.
 //
 // Pipeline (one barrier per 32-token block):  body i = [barrier] QK(i+1) | PV(i) overlapped with softmax(i+1) | publish P(i+1).
-// Blocks live in 4 nope buffers (32 KiB) and 3 rope buffers (4 KiB); the copy of block i+3 is issued right after barrier i, so
-// two blocks are always in flight.
+// Blocks live in 4 nope buffers (32 KiB) and 3 rope buffers (4 KiB); the copies of block i+3 are spread over the QK phase of
+// body i, so two blocks are always in flight.
 //
 // No accumulator rescaling in the steady state.  The 256 output accumulators live in the accumulation register file, which
 // vector ALU instructions cannot touch, so the usual online-softmax rescale would cost three instructions per element.
-// Instead every row fixes its reference m_ref at the maximum of the first block in which it sees a key and uses
+// Instead every row fixes its reference m_ref at the largest score of its first block and uses
 // P = exp2(s - m_ref) from then on: bf16 and fp32 share one exponent range, so P may grow to 2^100 without loss of
 // relative precision.  If a later score exceeds m_ref by more than 100 (log2 units; e^69 in weight) the row raises a flag
-// that travels with P, and the whole workgroup restarts its split with the row maxima seen so far as references.  Each
+// that travels with P, and the whole workgroup restarts its segment with the row maxima seen so far as references.  Each
 // restart raises a reference by more than 100, so at most a few can happen; realistic logits never trigger one.
 // Partials are written as fp16 (normalised values, |o| <= max|V|) through an LDS transpose so that global stores are row
-// contiguous; log-sum-exps as fp32.
+// contiguous; log-sum-exps as fp32.  With a fixed reference a row's most probable key no longer has probability exactly 1,
+// so its bf16 rounding error is recorded beside the partial and taken out again by mla_chunk_reduce_kernel.
 #include "decode_v2_params.hpp"
 #include <type_traits>
 
@@ -750,7 +751,7 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
       c_last = (int)((((int64_t)before + mine) * G - 1) / T);
     }
     while (c <= c_last) {
-      int64_t part[kRedParts];                               // partial numbers of this round (uniform), -1 = none
+      int64_t part[kRedParts];                               // partial numbers of this pass (uniform), -1 = none
       int np = 0;
 #pragma unroll
       for (int q = 0; q < kRedParts; q++) {
