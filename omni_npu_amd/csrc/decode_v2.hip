@@ -28,6 +28,7 @@
 // so its bf16 rounding error is recorded beside the partial and taken out again by mla_chunk_reduce_kernel.
 #include "decode_v2_params.hpp"
 #include <type_traits>
+#include <cstdlib>
 
 namespace mlahip {
 
@@ -46,6 +47,10 @@ constexpr int kV2POff = kV2RopeOff + 3 * kV2RopeBufB;      // 143360
 constexpr int kV2PBufB = 8192;                             // 4 row groups x 2 k-blocks x 64 lanes x 16 B
 constexpr int kV2AOff = kV2POff + 2 * kV2PBufB;            // 159744: rescale factors, 2 x 512 B
 constexpr int kV2LdsB = kV2AOff + 2 * 512;                 // 160768
+#ifndef MLA_V2_LEAD
+#define MLA_V2_LEAD 3
+#endif
+constexpr int kLead = MLA_V2_LEAD;                          // block i + kLead is copied while block i is consumed (2 or 3)
 constexpr float kRestartThreshold = 100.f;                 // log2 units above a row's reference
 
 __device__ __forceinline__ int v2_swz_nope(int r) {
@@ -278,7 +283,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   };
   auto issue_next_two = [&]() {
 #pragma unroll 1
-    for (int j = 1; j < 3 && j < nb; j++) issue_block(blk_begin + j);
+    for (int j = 1; j < kLead && j < nb; j++) issue_block(blk_begin + j);
   };
 
   // ---- prologue: the first block's copies go out, then the query loads; both are waited for together ----
@@ -573,7 +578,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     issue_next_two();
     // ---- block 0: QK, softmax, publish ----
     {
-      if (nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
+      if (kLead > 2 && nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
       lds_barrier();
       f32x16 s;
       SoftmaxState st;
@@ -592,15 +597,15 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     for (int i = 0; i + 1 < nb; i++) {
       const int blk = blk_begin + i;
       // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
-      if (i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
+      if (kLead > 2 && i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
       lds_barrier();
       const f32x4 fl = flags_read(blk);
       f32x16 s;
       PvHead head;
       auto hook = [&] { pv_head_read(blk, head); };
-      if (i + 3 >= nb) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0, hook);
-      else if (kSparse || L - 1 - (blk + 3) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + 3, hook);
-      else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + 3, hook);
+      if (i + kLead >= nb) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0, hook);
+      else if (kSparse || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead, hook);
+      else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + kLead, hook);
       if (flags_ask_restart(fl)) { restart = true; break; }
       SoftmaxState st;
       pv_block(blk, std::true_type{}, s, st, std::true_type{}, head);
@@ -697,15 +702,14 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
   const int lane = threadIdx.x & 63;
   const int r_max = p.max_q_len * p.num_heads;
   const int groups = (r_max + kRedRows - 1) / kRedRows;     // row groups per sequence
-  const int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (gw >= (int64_t)p.batch * groups) return;
+  for (int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); gw < (int64_t)p.batch * groups; gw += (int64_t)gridDim.x * 4) {
   const int b = (int)(gw / groups);
   const int row0 = (int)(gw - (int64_t)b * groups) * kRedRows;
   int q0, qlen;
   if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
   qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
   const int rows = qlen * p.num_heads;
-  if (row0 >= rows) return;
+  if (row0 >= rows) continue;
 
   int tot_units = 0, before = 0;
   for (int i = lane; i < p.batch; i += 64) {
@@ -807,12 +811,16 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
     if (p.lse_out && lane == 0)
       p.lse_out[(int64_t)(q0 + t_local) * p.lse_st + head] = tot[j] > 0.f ? __logf(tot[j]) + m[j] : -INFINITY;
   }
+  }  // row groups of this wavefront
 }
 
 int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
   const int64_t waves = (int64_t)p.batch * ((r_max + kRedRows - 1) / kRedRows);
-  hipLaunchKernelGGL(mla_chunk_reduce_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, stream, p);
+  int64_t wgs = (waves + 3) / 4;
+  static const int64_t cap = getenv("MLA_REDUCE_WGS") ? atoll(getenv("MLA_REDUCE_WGS")) : (1ll << 30);
+  if (wgs > cap) wgs = cap;
+  hipLaunchKernelGGL(mla_chunk_reduce_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p);
   return check_launch("mla_chunk_reduce_kernel");
 }
 

@@ -62,6 +62,69 @@ def test_decode_single_key_returns_the_row(dev):
         assert torch.equal(got[b].cpu(), row.view(1, -1).expand(128, -1))
 
 
+def _plant(case, b, pos, head, gain):
+    """Overwrite the latent row of key `pos` of sequence b with gain * (query of `head`): its score for that head jumps
+    by about gain * |q|^2 * scale ~ 37 * gain (natural units), far beyond anything N(0,1) data produces."""
+    page = case["block_table"][b, pos // 128].long()
+    case["nope"][page, pos % 128] = (gain * case["q_nope"][b * case["q_len"], head].float()).bfloat16()
+
+
+@pytest.mark.parametrize("num_splits", [1, 4])
+def test_decode_scores_that_outgrow_the_first_block(dev, num_splits):
+    """The kernel fixes each row's softmax reference at its first block and restarts a segment when a later score exceeds
+    it by more than 2^100: keys planted late in the sequences with scores ~110 and ~220 (natural units) above the
+    rest exercise one and two restarts, a planted key in the very first block exercises a reference that is already
+    the maximum, and a moderately dominant key (weight ~0.5) exercises the correction of the dominant probability."""
+    case = O.make_decode_case(4, 128, 1500, 2500, seed=21)
+    lens = case["seq_lens"].tolist()
+    _plant(case, 0, lens[0] - 40, 3, 3.0)                      # one restart, late in the last chunk
+    _plant(case, 1, 700, 5, 3.0)
+    _plant(case, 1, 1400, 5, 6.0)                              # two restarts for head 5 of sequence 1
+    _plant(case, 2, 7, 9, 4.0)                                 # the maximum sits in the first block
+    _plant(case, 3, 900, 11, 0.17)                             # about e^6 above the crowd: weight of the order of 0.5
+    ref = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"])
+    got, _ = _run(case, dev, num_splits)
+    got = got.float().cpu()
+    # the planted rows dominate their heads completely: the output is that latent row (values up to ~25, so the bf16
+    # rounding of the output alone exceeds the absolute bar: these three (sequence, head) pairs are checked relatively)
+    for b, pos, head in ((0, lens[0] - 40, 3), (1, 1400, 5), (2, 7, 9)):
+        row = case["nope"][case["block_table"][b, pos // 128].long(), pos % 128].float()
+        assert (got[b, head] - row).abs().max().item() <= 2 ** -8 * row.abs().max().item()
+        assert (ref[b, head] - row).abs().max().item() <= 1e-3 * row.abs().max().item()
+    # the planted rows hold values up to ~25 and leak into other heads of their sequences, so the absolute bar is scaled by
+    # the magnitude of each output row (it is the unchanged 2e-2 wherever the outputs are of order one)
+    err = (got - ref).abs()
+    bar = MAX_ABS * ref.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    assert (err <= bar).all(), f"worst excess {(err / bar).max().item():.3f} x the bar"
+    assert (err.sum() / ref.abs().sum()).item() <= MEAN_REL
+
+
+def test_decode_empty_and_tiny_sequences_in_one_batch(dev):
+    """Lengths 0, 1, 31, 32, 33 and a long one side by side: empty sequences give zeros and lse = -inf, and the balanced
+    chunk plan (more chunks than blocks for most of these) must still route every partial."""
+    case = O.make_decode_case(6, 128, 1, 1, seed=8)
+    big = O.make_decode_case(1, 128, 3000, 3000, seed=9)
+    lens = [0, 1, 31, 32, 33, 3000]
+    pages = sum((l + 127) // 128 for l in lens) + 1
+    g = torch.Generator().manual_seed(10)
+    case["nope"] = torch.randn(pages, 128, 512, generator=g).bfloat16()
+    case["rope"] = torch.randn(pages, 128, 64, generator=g).bfloat16()
+    bt = torch.zeros(6, (3000 + 127) // 128, dtype=torch.int32)
+    perm = torch.randperm(pages, generator=g).tolist()
+    for b, l in enumerate(lens):
+        for j in range((l + 127) // 128):
+            bt[b, j] = perm.pop()
+    case["block_table"], case["seq_lens"] = bt, torch.tensor(lens, dtype=torch.int32)
+    ref, ref_lse = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], bt, case["seq_lens"],
+                                     case["scale"], return_lse=True)
+    for splits in (1, 3):
+        got, lse = _run(case, dev, splits, with_lse=True)
+        assert (got[0].float() == 0).all() and torch.isinf(lse[0]).all() and (lse[0] < 0).all()
+        attn_close(got[1:], ref[1:], MAX_ABS, MEAN_REL)
+        assert torch.allclose(lse[1:].cpu(), ref_lse[1:], atol=2e-2, rtol=0)
+
+
 @pytest.mark.parametrize("q_len,heads", [(2, 128), (3, 16), (2, 40)])
 def test_decode_mtp_right_down_causal(dev, q_len, heads):
     """q_len > 1: token i of a request sees keys [0, L - q_len + i]."""
