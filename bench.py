@@ -75,8 +75,8 @@ def bench_dsa(K, dev, args):
     splits = args.splits or K.default_num_splits(B, 1, N, k)
     stages = [
         ("indexer", lambda: K.indexer_scores(q8, w, k8, ks, btd, lensd, logits, max_seq_len=max_len)),
-        ("topk", lambda: K.topk(logits, lensd, k, idx)),
-        ("build_rows", lambda: K.build_sparse_rows(idx, btd, lensd, 128, nblk, rows, counts)),
+        ("topk_with_rows", lambda: K.topk(logits, lensd, k, idx, block_table=btd, page_size=128, num_pages=nblk, rows=rows,
+                                          counts=counts)),
         ("sparse_decode", lambda: K.sparse_decode(qn, qr, nope, rope, rows, counts, 192 ** -0.5, out, num_splits=splits)),
     ]
 

@@ -163,6 +163,15 @@ int dsa_topk(const float* logits, int64_t logits_stride, const int32_t* seq_lens
              int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
              void* workspace /* may be NULL */, size_t workspace_bytes, mlahip_stream_t stream);
 
+/* dsa_topk and dsa_build_rows (below) in one pass: besides the positions every pick is translated through the block
+ * table into its flat cache row (page * page_size + offset) and counts[t] = picks of token t; what
+ * attention/backends/dsa.py:259-291 feeds to the sparse attention, without a second launch. */
+int dsa_topk_rows(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
+                  int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
+                  const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, int32_t page_size, int64_t num_pages,
+                  int32_t* rows, int64_t rows_stride, int32_t* counts, void* workspace /* may be NULL */,
+                  size_t workspace_bytes, mlahip_stream_t stream);
+
 /* ---- (a16) sparse MLA over the selected keys ----------------------------------------------------------
  * Replaces torch.ops.custom.npu_sparse_flash_attention, attention/backends/dsa.py:259-291 (sparse_block_size 1,
  * layout_kv "PA_BSND"): dsa_build_rows maps the [T,k] logical positions (-1 = unused,

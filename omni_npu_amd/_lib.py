@@ -39,6 +39,7 @@ SIGNATURES = {
     "dsa_quant_rows_fp8": (c_int32, [P, I64, I64, P, P, I64, I64, P, I64, I32, I64, P]),
     "dsa_topk_workspace_bytes": (SZ, [I32, I32, I64]),
     "dsa_topk": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, SZ, P]),
+    "dsa_topk_rows": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, I64, I32, I32, I64, P, I64, P, P, SZ, P]),
     "dsa_build_rows": (c_int32, [P, I64, P, I64, I32, P, P, I32, I32, I32, I32, I64, P, I64, P, P]),
     "dsa_sparse_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, I32, P, I64, P, I32, I32,
                                          F32, P, I64, I64, P, P, SZ, I32, P]),

@@ -711,6 +711,9 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
   const int rows = qlen * p.num_heads;
   if (row0 >= rows) continue;
 
+  // (everything that depends on b only is requested together: one memory round trip, not three)
+  const int id_first = p.seg_ids[2 * b], id_last = p.seg_ids[2 * b + 1];
+  const int mine = v2_work_units(p.seq_lens[b]);
   int tot_units = 0, before = 0;
   for (int i = lane; i < p.batch; i += 64) {
     const int c = v2_work_units(p.seq_lens[i]);
@@ -719,7 +722,6 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
   }
   tot_units = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot_units));
   before = __builtin_amdgcn_readfirstlane(wave_sum_i32(before));
-  const int mine = v2_work_units(p.seq_lens[b]);
   const int64_t G = p.num_chunks, T = tot_units;
   // does chunk c hold blocks of this sequence (units [before, before + mine), the first kSegCost of them start-up)?
   auto holds_blocks = [&](int64_t c) -> bool {
@@ -748,8 +750,8 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
     const bool dense_chunks = T >= G;
     int c, c_last;
     if (dense_chunks) {
-      c = p.seg_ids[2 * b] - b;
-      c_last = p.seg_ids[2 * b + 1] - b;
+      c = id_first - b;
+      c_last = id_last - b;
     } else {
       c = (int)((((int64_t)before + 1) * G - 1) / T);
       c_last = (int)((((int64_t)before + mine) * G - 1) / T);

@@ -65,7 +65,35 @@ struct TopkParams {
   const int32_t* seq_lens; const int32_t* qsl;
   int32_t batch, max_q_len, k;
   int32_t* out; int64_t o_st;
+  // optional (rows != NULL): also translate every pick into its flat cache row, and count the picks per token
+  const int32_t* block_table; int64_t bt_stride; int32_t max_blocks, page_size; int64_t num_pages;
+  int32_t* rows; int64_t r_st; int32_t* counts;
 };
+
+// Where pick number `at` of token t (request b) goes: its position into the index buffer and, if asked for, its flat
+// cache row (page * page_size + offset) into the row list that the sparse attention reads.
+struct TopkSink {
+  int32_t* out; int32_t* rows; const int32_t* bt; int32_t max_blocks, page_size; int64_t num_pages;
+  __device__ __forceinline__ void put(int at, int pos) const {
+    out[at] = pos;
+    if (rows) {
+      int pg = pos / page_size;
+      const int off = pos - pg * page_size;
+      pg = pg < max_blocks ? pg : max_blocks - 1;
+      int64_t blk = bt[pg];
+      blk = blk < 0 ? 0 : (blk >= num_pages ? num_pages - 1 : blk);
+      rows[at] = (int32_t)(blk * page_size + off);
+    }
+  }
+};
+__device__ __forceinline__ TopkSink topk_sink(const TopkParams& p, int b, int t) {
+  TopkSink s;
+  s.out = p.out + (int64_t)t * p.o_st;
+  s.rows = p.rows ? p.rows + (int64_t)t * p.r_st : nullptr;
+  s.bt = p.rows ? p.block_table + (int64_t)b * p.bt_stride : nullptr;
+  s.max_blocks = p.max_blocks; s.page_size = p.page_size; s.num_pages = p.num_pages;
+  return s;
+}
 
 constexpr int kCandCap = 8192;                             // boundary-bin keys that fit in LDS
 constexpr int kRankMax = 256;                              // up to here the threshold is found by ranking, not by radix passes
@@ -195,7 +223,7 @@ __device__ __forceinline__ void rank_threshold(const uint32_t* cand_u, const uin
 // Ordered output of the picks of [r_lo, r_hi) by one wavefront, 64 * kVec consecutive keys at a time with ballot prefix
 // sums; `o` = number of picks before r_lo.  A key is picked iff  u > prefix || (u == prefix && position <= pos_thresh).
 template <int kVec>
-__device__ __forceinline__ void ordered_write(const float* x, int32_t* out, int r_lo, int r_hi, int lane, int o, int k,
+__device__ __forceinline__ void ordered_write(const float* x, const TopkSink& out, int r_lo, int r_hi, int lane, int o, int k,
                                               uint32_t prefix, uint32_t pos_thresh) {
   const uint64_t below = lane == 0 ? 0ull : (~0ull >> (64 - lane));
   constexpr int kWDepth = 4;
@@ -228,7 +256,7 @@ __device__ __forceinline__ void ordered_write(const float* x, int32_t* out, int 
       int at = o + before;
 #pragma unroll
       for (int e = 0; e < kVec; e++)
-        if (tk[e]) { if (at < k) out[at] = i + e; at++; }
+        if (tk[e]) { if (at < k) out.put(at, i + e); at++; }
       o += total;
     }
   }
@@ -252,11 +280,14 @@ __global__ __launch_bounds__(kTopkThreads) void dsa_topk_kernel(const TopkParams
   int n = p.seq_lens[b] - qlen + ti + 1;                   // visible keys
   n = n < 0 ? 0 : n;
   const float* x = p.logits + (int64_t)t * p.l_st;
-  int32_t* out = p.out + (int64_t)t * p.o_st;
+  const TopkSink out = topk_sink(p, b, t);
   const int k = p.k;
+  if (p.counts && tid == 0) p.counts[t] = n < k ? n : k;
 
   if (n <= k) {                                            // everything is selected
-    for (int i = tid; i < k; i += kTopkThreads) out[i] = i < n ? i : -1;
+    for (int i = tid; i < k; i += kTopkThreads) {
+      if (i < n) out.put(i, i); else out.out[i] = -1;
+    }
     return;
   }
 
@@ -376,7 +407,7 @@ struct TopkMwParams {
   int64_t cand_cap;
 };
 
-struct TopkRow { const float* x; int32_t* out; int n, slot; bool live; };
+struct TopkRow { const float* x; int n, slot, b, t; bool live; };
 __device__ __forceinline__ TopkRow topk_row(const TopkParams& p, int slot) {
   TopkRow r;
   const int b = slot / p.max_q_len;
@@ -388,7 +419,8 @@ __device__ __forceinline__ TopkRow topk_row(const TopkParams& p, int slot) {
   int n = p.seq_lens[b] - qlen + ti + 1;                   // visible keys
   r.n = n < 0 ? 0 : n;
   r.x = p.logits + (int64_t)t * p.l_st;
-  r.out = p.out + (int64_t)t * p.o_st;
+  r.b = b;
+  r.t = t;
   r.slot = slot;
   return r;
 }
@@ -513,9 +545,13 @@ __global__ __launch_bounds__(kTopkThreads) void dsa_topk_write_kernel(const Topk
   const TopkRow r = topk_row(p.t, blockIdx.y);
   if (!r.live) return;
   const int n = r.n, k = p.t.k;
+  const TopkSink out = topk_sink(p.t, r.b, r.t);
+  if (p.t.counts && s == 0 && tid == 0) p.t.counts[r.t] = n < k ? n : k;
   if (n <= k) {                                            // everything is selected
     if (s == 0)
-      for (int i = tid; i < k; i += kTopkThreads) r.out[i] = i < n ? i : -1;
+      for (int i = tid; i < k; i += kTopkThreads) {
+        if (i < n) out.put(i, i); else out.out[i] = -1;
+      }
     return;
   }
   if (s * kSliceKeys >= n) return;
@@ -583,7 +619,7 @@ __global__ __launch_bounds__(kTopkThreads) void dsa_topk_write_kernel(const Topk
     int at = o + before;
 #pragma unroll
     for (int e = 0; e < 4; e++)
-      if (tk[e]) { if (at < k) r.out[at] = i + e; at++; }
+      if (tk[e]) { if (at < k) out.put(at, i + e); at++; }
     o += total;
   }
 }
@@ -661,16 +697,18 @@ extern "C" size_t dsa_topk_workspace_bytes(int32_t batch, int32_t max_q_len, int
   return tokens * ((size_t)kMaxSlices * kBins * 4 + 8 + 16 + (size_t)kMaxSlices * kMwWaves * 4 + (size_t)logits_stride * 8);
 }
 
-// workspace may be NULL: then one workgroup per token does all the work (no scratch memory at all).
-extern "C" int dsa_topk(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
-                        int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
-                        void* workspace, size_t workspace_bytes, hipStream_t stream) {
+static int topk_impl(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
+                     int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
+                     const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, int32_t page_size, int64_t num_pages,
+                     int32_t* rows, int64_t rows_stride, int32_t* counts, void* workspace, size_t workspace_bytes,
+                     hipStream_t stream) {
   MLA_REQUIRE(logits && seq_lens && out_indices, MLA_ERR_NULL, "dsa_topk: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && k >= 1 && out_stride >= k, MLA_ERR_SHAPE,
               "dsa_topk: batch=%d max_q_len=%d k=%d out_stride=%lld", batch, max_q_len, k, (long long)out_stride);
   MLA_REQUIRE(logits_stride < (1ll << 22), MLA_ERR_SHAPE, "dsa_topk: at most 2^22 keys per row");
   if (batch == 0) return MLA_OK;
-  TopkParams p{logits, logits_stride, seq_lens, query_start_loc, batch, max_q_len, k, out_indices, out_stride};
+  TopkParams p{logits, logits_stride, seq_lens, query_start_loc, batch, max_q_len, k, out_indices, out_stride,
+               block_table, bt_stride, max_blocks, page_size, num_pages, rows, rows_stride, counts};
   // rows that start on 16-byte boundaries are read four keys per load
   const bool vec = ((uintptr_t)logits % 16 == 0) && (logits_stride % 4 == 0);
   const int64_t tokens = (int64_t)batch * max_q_len;
@@ -704,6 +742,29 @@ extern "C" int dsa_topk(const float* logits, int64_t logits_stride, const int32_
     hipLaunchKernelGGL(dsa_topk_write_kernel<1>, grid, dim3(kTopkThreads), 0, stream, m);
   }
   return check_launch("dsa_topk (hist / gather / write)");
+}
+
+// workspace may be NULL: then one workgroup per token does all the work (no scratch memory at all).
+extern "C" int dsa_topk(const float* logits, int64_t logits_stride, const int32_t* seq_lens, const int32_t* query_start_loc,
+                        int32_t batch, int32_t max_q_len, int32_t k, int32_t* out_indices, int64_t out_stride,
+                        void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  return topk_impl(logits, logits_stride, seq_lens, query_start_loc, batch, max_q_len, k, out_indices, out_stride, nullptr, 0,
+                   1, 1, 1, nullptr, 0, nullptr, workspace, workspace_bytes, stream);
+}
+
+// dsa_topk and dsa_build_rows in one: besides the positions (the reference's index buffer) every pick is translated
+// through the block table into its flat cache row, and counts[t] = number of picks of token t.
+extern "C" int dsa_topk_rows(const float* logits, int64_t logits_stride, const int32_t* seq_lens,
+                             const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t k,
+                             int32_t* out_indices, int64_t out_stride, const int32_t* block_table, int64_t bt_stride,
+                             int32_t max_blocks, int32_t page_size, int64_t num_pages, int32_t* rows, int64_t rows_stride,
+                             int32_t* counts, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+  MLA_REQUIRE(block_table && rows && counts, MLA_ERR_NULL, "dsa_topk_rows: null pointer argument");
+  MLA_REQUIRE(page_size >= 1 && num_pages >= 1 && max_blocks >= 1 && rows_stride >= k && num_pages * page_size < (1ll << 31),
+              MLA_ERR_SHAPE, "dsa_topk_rows: page_size=%d max_blocks=%d rows_stride=%lld", page_size, max_blocks,
+              (long long)rows_stride);
+  return topk_impl(logits, logits_stride, seq_lens, query_start_loc, batch, max_q_len, k, out_indices, out_stride, block_table,
+                   bt_stride, max_blocks, page_size, num_pages, rows, rows_stride, counts, workspace, workspace_bytes, stream);
 }
 
 extern "C" int dsa_build_rows(const int32_t* indices, int64_t indices_stride, const int32_t* block_table, int64_t bt_stride,

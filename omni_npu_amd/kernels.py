@@ -295,10 +295,13 @@ def indexer_scores(q8: torch.Tensor, weights: torch.Tensor, k8_cache: torch.Tens
 
 def topk(logits: torch.Tensor, seq_lens: torch.Tensor, k: int, out: torch.Tensor, q_len: int = 1,
          query_start_loc: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-         single_workgroup: bool = False) -> torch.Tensor:
+         single_workgroup: bool = False, block_table: Optional[torch.Tensor] = None, page_size: int = PAGE,
+         num_pages: int = 0, rows: Optional[torch.Tensor] = None, counts: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Positions of the k largest logits among each token's visible keys, ties to the lower position, ascending
     position order, -1 padding; out int32 [T,k] or [T,1,k] (patch_dsv32_indexer.py:133-146).
-    single_workgroup=True runs the variant that needs no scratch memory (one workgroup per token)."""
+    single_workgroup=True runs the variant that needs no scratch memory (one workgroup per token).
+    With block_table / num_pages / rows [T,k] / counts [T] the same launch also fills the flat cache rows and the pick
+    counts that build_sparse_rows would produce from `out`."""
     _need_cuda(logits, seq_lens, out)
     lib = _lib.load()
     o2 = out.reshape(out.shape[0], -1) if out.dim() == 3 else out
@@ -312,8 +315,20 @@ def topk(logits: torch.Tensor, seq_lens: torch.Tensor, k: int, out: torch.Tensor
         need = lib.dsa_topk_workspace_bytes(b, q_len, logits.stride(0))
         ws = workspace if workspace is not None else _workspace(logits.device, need, tag="topk")
         ws_ptr, ws_bytes = ws.data_ptr(), ws.numel() * ws.element_size()
-    rc = lib.dsa_topk(logits.data_ptr(), logits.stride(0), seq_lens.data_ptr(),
-                      query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, k, o2.data_ptr(),
+    qsl = query_start_loc.data_ptr() if query_start_loc is not None else None
+    if rows is not None:
+        _need_cuda(block_table, rows, counts)
+        if block_table is None or counts is None or rows.dtype != torch.int32 or rows.dim() != 2 or rows.shape[1] < k or \
+                rows.stride(-1) != 1 or counts.dtype != torch.int32 or not counts.is_contiguous() or \
+                block_table.dtype != torch.int32 or num_pages < 1:
+            raise TypeError("topk: rows int32 [T,>=k], counts int32 [T], int32 block_table and num_pages go together")
+        rc = lib.dsa_topk_rows(logits.data_ptr(), logits.stride(0), seq_lens.data_ptr(), qsl, b, q_len, k, o2.data_ptr(),
+                               o2.stride(0), block_table.data_ptr(), block_table.stride(0), block_table.shape[1], page_size,
+                               num_pages, rows.data_ptr(), rows.stride(0), counts.data_ptr(), ws_ptr, ws_bytes,
+                               _stream(logits))
+        _lib.check(rc, "dsa_topk_rows")
+        return out
+    rc = lib.dsa_topk(logits.data_ptr(), logits.stride(0), seq_lens.data_ptr(), qsl, b, q_len, k, o2.data_ptr(),
                       o2.stride(0), ws_ptr, ws_bytes, _stream(logits))
     _lib.check(rc, "dsa_topk")
     return out

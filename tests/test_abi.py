@@ -20,7 +20,7 @@ def test_header_declares_the_path():
     syms = declared_symbols()
     for must in ("mla_cache_write_bf16", "mla_cache_write_fp8", "mla_decode_bf16", "mla_splitkv_reduce",
                  "mla_decode_workspace_bytes", "mla_gather_paged", "mla_merge_states", "dsa_indexer_scores_fp8",
-                 "dsa_topk", "dsa_topk_workspace_bytes", "dsa_sparse_decode_bf16", "mlahip_version", "mlahip_last_error_string"):
+                 "dsa_topk", "dsa_topk_rows", "dsa_topk_workspace_bytes", "dsa_sparse_decode_bf16", "mlahip_version", "mlahip_last_error_string"):
         assert must in syms
 
 

@@ -94,6 +94,39 @@ def test_topk_bit_exact_sets_and_ties(dev, n, k, single_workgroup):
         assert (got[r, len(g_valid):] == -1).all()
 
 
+@pytest.mark.parametrize("single_workgroup", [False, True], ids=["multi-workgroup", "single-workgroup"])
+def test_topk_rows_equals_topk_then_build_rows(dev, single_workgroup):
+    """The fused launch writes the same positions, the same flat cache rows and the same counts as dsa_topk followed
+    by dsa_build_rows (bit-exact integer work)."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(11)
+    lens = torch.tensor([20000, 150, 9000, 2048, 2049], dtype=torch.int32)
+    k, page = 2048, 128
+    nblk_seq = (lens + page - 1) // page
+    nblk = int(nblk_seq.sum())
+    perm = torch.randperm(nblk, generator=g).to(torch.int32)
+    bt = torch.zeros(len(lens), int(nblk_seq.max()), dtype=torch.int32)
+    o = 0
+    for b in range(len(lens)):
+        n = int(nblk_seq[b])
+        bt[b, :n] = perm[o:o + n]
+        o += n
+    x = torch.randn(len(lens), 20000, generator=g).to(dev)
+    btd, lensd = bt.to(dev), lens.to(dev)
+    idx_a = torch.full((len(lens), k), -5, dtype=torch.int32, device=dev)
+    rows_a = torch.full((len(lens), k), -5, dtype=torch.int32, device=dev)
+    cnt_a = torch.full((len(lens),), -5, dtype=torch.int32, device=dev)
+    K.topk(x, lensd, k, idx_a, single_workgroup=single_workgroup)
+    K.build_sparse_rows(idx_a, btd, lensd, page, nblk, rows_a, cnt_a)
+    idx_b, rows_b, cnt_b = torch.full_like(idx_a, -6), torch.full_like(rows_a, -6), torch.full_like(cnt_a, -6)
+    K.topk(x, lensd, k, idx_b, single_workgroup=single_workgroup, block_table=btd, page_size=page, num_pages=nblk,
+           rows=rows_b, counts=cnt_b)
+    assert torch.equal(idx_a, idx_b) and torch.equal(cnt_a, cnt_b)
+    for b in range(len(lens)):
+        c = int(cnt_a[b])
+        assert c == min(int(lens[b]), k) and torch.equal(rows_a[b, :c], rows_b[b, :c])
+
+
 def test_topk_on_indexer_logits_then_sparse_decode(dev):
     """Whole DSA decode chain at small scale: logits -> top-k (set equals the oracle's on the SAME logits) ->
     rows -> sparse MLA equals the oracle's sparse attention on that index set."""
