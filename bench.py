@@ -189,6 +189,85 @@ def bench_prefill(K, dev, args):
     }
 
 
+def bench_fp8(K, dev, args):
+    """configs[4]: fp8-e4m3 block-scaled latent cache, batch 256, contexts uniform[16384, 32768], 128 heads, q_len 2
+    (MTP pair), page 128; a step = fp8 cache write of the 512 new tokens + decode, replayed as a captured HIP graph."""
+    g = torch.Generator().manual_seed(args.seed)
+    B, N, QL = 256, 128, 2
+    lens = torch.randint(16384, 32769, (B,), generator=g).to(torch.int32)
+    nblk_seq = (lens + 127) // 128
+    nblk = int(nblk_seq.sum())
+    perm = torch.randperm(nblk, generator=g).to(torch.int32)
+    bt = torch.zeros(B, int(nblk_seq.max()), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        n = int(nblk_seq[b])
+        bt[b, :n] = perm[o:o + n]
+        o += n
+    cache = torch.empty(nblk, 128, K.FP8_ROW_BYTES, dtype=torch.uint8, device=dev)
+    # fill the cache on the GPU through the product's own quantising write, 64 pages at a time
+    for p0 in range(0, nblk, 64):
+        p1 = min(nblk, p0 + 64)
+        rows = (p1 - p0) * 128
+        K.cache_write_fp8(torch.randn(rows, 512, device=dev).bfloat16(), torch.randn(rows, 64, device=dev).bfloat16(),
+                          torch.arange(p0 * 128, p1 * 128, dtype=torch.int64, device=dev), cache)
+    T = B * QL
+    qn = torch.randn(T, N, 512, device=dev).bfloat16()
+    qr = torch.randn(T, N, 64, device=dev).bfloat16()
+    new_c = torch.randn(T, 512, device=dev).bfloat16()
+    new_r = torch.randn(T, 64, device=dev).bfloat16()
+    slots = torch.empty(T, dtype=torch.int64)
+    for b in range(B):
+        for j in range(QL):
+            pos = int(lens[b]) - QL + j
+            slots[b * QL + j] = int(bt[b, pos // 128]) * 128 + pos % 128
+    slots, btd, lensd = slots.to(dev), bt.to(dev), lens.to(dev)
+    out = torch.empty(T, N, 512, dtype=torch.bfloat16, device=dev)
+    splits = args.splits or K.default_num_splits(B, QL, N, int(lens.max()))
+
+    def step():
+        K.cache_write_fp8(new_c, new_r, slots, cache)
+        K.decode_fp8(qn, qr, cache, btd, lensd, 192 ** -0.5, out, q_len=QL, num_splits=splits)
+
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+
+    def ev_time(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(e) * 1e3 / n
+
+    n = max(3, min(args.steps, 10))
+    t_graph, t_eager = ev_time(graph.replay, n), ev_time(step, n)
+    sum_l = int(lens.sum())
+    flops = sum_l * N * QL * 2 * (576 + 512)
+    bytes_ = sum_l * K.FP8_ROW_BYTES + T * N * (576 + 512) * 2
+    best = min(t_graph, t_eager)
+    return {
+        "metric": "MLA decode us/layer, fp8-e4m3 block-scaled cache (B=256, ctx 16k-32k, 128 heads, q_len 2)",
+        "value": round(t_graph, 1), "unit": "us/layer", "n_gpus": 1, "steps": n, "warmup": 3, "higher_is_better": False,
+        "dtype": "bf16 MFMA over fp8 storage (dequantised on chip)", "data": "synthetic",
+        "config": {"workload": "configs[4]: fp8 cache, high-batch MTP decode", "batch": B, "heads": N, "q_len": QL,
+                   "seq_lens": "uniform[16384,32768]", "sum_seq_len": sum_l, "kv_splits": splits, "seed": args.seed},
+        "step_us": {"hip_graph_replay": round(t_graph, 1), "eager_launches": round(t_eager, 1)},
+        "roofline": {"kernel": "mla_decode_bf16_kernel<fp8>", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "algorithmic_flops": flops, "algorithmic_bytes": bytes_,
+                     "hbm_gbs": round(bytes_ / (best * 1e-6) / 1e9, 1)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -208,8 +287,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill"],
-                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -233,6 +312,9 @@ def main():
         return
     if args.workload == "prefill":
         print(json.dumps(bench_prefill(K, dev, args)))
+        return
+    if args.workload == "fp8":
+        print(json.dumps(bench_fp8(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len
