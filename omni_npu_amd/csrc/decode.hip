@@ -550,7 +550,7 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
     attr_set = true;
   }
   dim3 grid(num_splits, batch, (r_max + kRowsPerWg - 1) / kRowsPerWg);
-  if (!fp8 && !use_first_generation()) {
+  if (!use_first_generation()) {
     DecodeV2Params v;
     v.q_nope = p.q_nope; v.qn_st = p.qn_st; v.qn_sh = p.qn_sh; v.q_rope = p.q_rope; v.qr_st = p.qr_st; v.qr_sh = p.qr_sh;
     v.nope = p.nope; v.nope_sp = p.nope_sp; v.nope_sr = p.nope_sr; v.rope = p.rope; v.rope_sp = p.rope_sp; v.rope_sr = p.rope_sr;
@@ -560,7 +560,10 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
     v.corr_scale = p.lse_part + rows; v.corr_row = (const __bf16**)(p.lse_part + 2 * rows);
     v.seg_ids = (int32_t*)(p.lse_part + 4 * rows);
     v.sparse_rows = p.sparse_rows; v.sparse_stride = p.sparse_stride; v.page_size = p.page_size;
-    return launch_decode_v2(v, sparse_rows != nullptr, dim3((unsigned)(batch * num_splits), 1, grid.z), stream);
+    v.cache8 = fp8 ? (const uint8_t*)nope_cache : nullptr; v.c8_sp = nope_page_stride;
+    const dim3 grid2((unsigned)(batch * num_splits), 1, grid.z);
+    if (fp8) return launch_decode_v2_fp8(v, grid2, stream);
+    return launch_decode_v2(v, sparse_rows != nullptr, grid2, stream);
   }
   if (fp8) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeFp8>, grid, dim3(256), kFp8LdsB, stream, p);
   else if (sparse_rows) hipLaunchKernelGGL(mla_decode_bf16_kernel<kModeSparse>, grid, dim3(256), kDecodeLdsB, stream, p);
@@ -690,7 +693,8 @@ extern "C" int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t q
                              block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
                              scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, true, stream);
   if (rc != MLA_OK) return rc;
-  // the fp8 kernel writes its partials in [sequence][split] order: no sequence lengths, no chunk arithmetic
-  return mla_splitkv_reduce(workspace, workspace_bytes, nullptr, query_start_loc, batch, max_q_len, num_heads, num_splits,
-                            out, out_stride_t, out_stride_h, lse_out, stream);
+  // the first-generation kernel writes its partials in [sequence][split] order (no sequence lengths, no chunk arithmetic),
+  // the current one in the balanced chunk order of the bf16 path
+  return mla_splitkv_reduce(workspace, workspace_bytes, use_first_generation() ? nullptr : seq_lens, query_start_loc, batch,
+                            max_q_len, num_heads, num_splits, out, out_stride_t, out_stride_h, lse_out, stream);
 }

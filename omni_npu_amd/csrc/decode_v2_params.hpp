@@ -21,6 +21,7 @@ struct DecodeV2Params {
   const __bf16** corr_row;       // [chunks + B, R_max]: that key's latent vector in the cache
   int32_t* seg_ids;              // [B][2]: partial number of the sequence's first / last segment
   const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
+  const uint8_t* cache8; int64_t c8_sp;   // fp8 kernel: block-scaled cache, page stride in bytes (rows are 656 bytes apart)
 };
 
 struct ChunkReduceParams {
@@ -35,5 +36,7 @@ int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream);
 
 // Launches mla_decode_v2_kernel<sparse> on `stream`; returns 0 or a negative error code.
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
+// Launches mla_decode_v2_fp8_kernel (decode_v2_fp8.hip) over p.cache8.
+int launch_decode_v2_fp8(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
 
 }  // namespace mlahip
