@@ -268,6 +268,93 @@ def bench_fp8(K, dev, args):
     }
 
 
+def bench_prologue(K, dev, args):
+    """The step in front of the path: fused RMSNorm + rotary embedding + cache write of T new tokens and the rotary embedding
+    of their 128 query heads, at decode size (T = 64: latency) and at prefill-chunk size (T = 8192: bandwidth)."""
+    import time
+    from oracle import mla_oracle as O
+    g = torch.Generator().manual_seed(args.seed)
+    N = 128
+    out = {}
+    cpu = None
+    for T in (64, 8192):
+        kv = torch.randn(T, 576, generator=g).bfloat16()
+        gamma = (1 + 0.1 * torch.randn(512, generator=g)).bfloat16()
+        pos = torch.randint(0, 32768, (T,), generator=g)
+        cos, sin = O.rope_tables(pos)
+        nblk = T // 128 + 64
+        slots = torch.randperm(nblk * 128, generator=g)[:T]
+        q = torch.randn(T, N, 192, generator=g).bfloat16()
+        d = [x.to(dev) for x in (kv, gamma, cos, sin, slots, q)]
+        nope = torch.zeros(nblk, 128, 512, dtype=torch.bfloat16, device=dev)
+        rope = torch.zeros(nblk, 128, 64, dtype=torch.bfloat16, device=dev)
+        q_out = torch.empty(T, N, 64, dtype=torch.bfloat16, device=dev)
+
+        def fused():
+            K.kv_rmsnorm_rope_cache(d[0], d[1], d[2], d[3], d[4], nope, rope, eps=1e-6)
+
+        def qrope():
+            K.interleave_rope(d[5][..., 128:], d[2], d[3], out=q_out)
+
+        def ev_time(fn, n, reps=10):
+            # `reps` launches per replay of a captured graph: a launch loop from Python would measure the host (tens of
+            # microseconds a call), not these kernels
+            fn()
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                fn()
+                with torch.cuda.graph(graph, stream=side):
+                    for _ in range(reps):
+                        fn()
+            torch.cuda.synchronize()
+            for _ in range(2):
+                graph.replay()
+            torch.cuda.synchronize()
+            a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(n):
+                graph.replay()
+            e.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(e) * 1e3 / (n * reps)
+
+        t_f, t_q = ev_time(fused, args.steps), ev_time(qrope, args.steps)
+        kv_bytes = T * (1152 + 2 * 128 + 8 + 1152) + 1024           # kv in, cos + sin rows, slot, cache rows out, gamma
+        q_bytes = T * N * 128 * 2 + T * 2 * 128
+        out[T] = {"fused_kv_us": round(t_f, 2), "q_rope_us": round(t_q, 2), "fused_kv_gbs": round(kv_bytes / t_f / 1e3, 1),
+                  "q_rope_gbs": round(q_bytes / t_q / 1e3, 1), "kv_bytes": kv_bytes, "q_bytes": q_bytes}
+        if T == 8192:
+            nope_c, rope_c = torch.zeros(nblk, 128, 512).bfloat16(), torch.zeros(nblk, 128, 64).bfloat16()
+            ts = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                O.kv_rmsnorm_rope_cache(kv, gamma, cos, sin, slots, nope_c, rope_c, 1e-6)
+                O.interleave_rope(q[..., 128:], cos, sin)
+                ts.append(time.perf_counter() - t0)
+            cpu = sorted(ts)[1]
+            got = nope.cpu().view(-1, 512)[slots]
+            bits = (got.view(torch.int16).int() - nope_c.view(-1, 512)[slots].view(torch.int16).int()).abs().max().item()
+    big = out[8192]
+    step_us = big["fused_kv_us"] + big["q_rope_us"]
+    tot_bytes = big["kv_bytes"] + big["q_bytes"]
+    return {
+        "metric": "fused RMSNorm + rotary embedding + cache write, plus query rotary embedding, us (T = 8192 tokens, 128 heads)",
+        "value": round(step_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "bf16 (fp32 arithmetic)", "data": "synthetic",
+        "config": {"workload": "step before the attention path (next row 1)", "tokens": [64, 8192], "heads": N, "seed": args.seed},
+        "sizes": {str(k): v for k, v in out.items()},
+        "roofline": {"kernel": "kv_rmsnorm_rope_cache_kernel<false> + interleave_rope_kernel", "bound": "hbm",
+                     "achieved": round(tot_bytes / step_us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(tot_bytes / step_us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "algorithmic_bytes": tot_bytes},
+        "cpu_baseline": {"value": round(cpu * 1e6, 1), "unit": "us", "cores": torch.get_num_threads(),
+                         "kind": "port", "sample": "oracle (torch float64) on the same 8192 tokens, median of 3",
+                         "gpu_vs_oracle_max_ulp": int(bits)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -287,8 +374,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8"],
-                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -315,6 +402,9 @@ def main():
         return
     if args.workload == "fp8":
         print(json.dumps(bench_fp8(K, dev, args)))
+        return
+    if args.workload == "prologue":
+        print(json.dumps(bench_prologue(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len

@@ -54,6 +54,43 @@ int mla_cache_write_fp8(const void* kv_c, int64_t kv_c_stride, const void* k_pe,
                         const int64_t* slot_mapping, int32_t num_tokens, void* cache, int64_t page_stride_bytes,
                         int64_t row_stride_bytes, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
 
+/* ---- the step in front of the path, fused (next row 1) ----------------------------------------------
+ * Replaces torch_npu.npu_kv_rmsnorm_rope_cache as called at v1/layers/attention/npu_mla.py:196-206, 296-309 and
+ * v1/layers/attention/npu_dsa.py:410-424, 517-527: RMSNorm(kv_a [T,512], gamma, eps) and the rotary embedding of
+ * k_pe [T,64] written straight into the paged cache rows named by slot_mapping (negative / out-of-range slots are
+ * skipped), plus, when the pointers are not NULL, the normalised latent and the rotated rope key as plain tensors
+ * (is_output_kv=True).  kv_a and k_pe are usually the two halves of one [T,576] tensor (k_pe = kv_a + 512).
+ * Arithmetic (fp32, one rounding to bf16): y = x * rsqrt(mean(x^2) + eps) * gamma;
+ * x1 = k_pe[0::2], x2 = k_pe[1::2], o1 = x1*cos - x2*sin, o2 = x2*cos + x1*sin with pair i reading table entry
+ * i*cos_step of the token's cos / sin row (rows cs_stride elements apart): cos_step 1 for the reference's cat(c, c)
+ * rows (layers/rotary_embedding/rotary_embedding_torch_npu.py:170-173), 2 for rows that repeat every entry.
+ * interleaved_out = 0 stores cat(o1, o2) (the reference's result, rotary_embedding_torch_npu.py:146-163);
+ * 1 stores the pairs back in place (GPT-J layout, tests/integration/attention/test_npu_mla_math.py:125-144). */
+int mla_kv_rmsnorm_rope_cache(const void* kv_a, int64_t kv_a_stride, const void* k_pe, int64_t k_pe_stride,
+                              const void* gamma /* bf16 [512] */, const void* cos, const void* sin, int64_t cs_stride,
+                              int32_t cos_step, int32_t interleaved_out, const int64_t* slot_mapping, int32_t num_tokens,
+                              float eps, void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride,
+                              void* rope_cache, int64_t rope_page_stride, int64_t rope_row_stride, int32_t page_size,
+                              int64_t num_pages, void* kv_a_out /* may be NULL */, int64_t kv_a_out_stride,
+                              void* k_pe_out /* may be NULL */, int64_t k_pe_out_stride, mlahip_stream_t stream);
+
+/* Same, into the fp8-e4m3 block-scaled cache of mla_cache_write_fp8 (the bf16-rounded normalised row is quantised,
+ * so the bytes equal mla_cache_write_fp8 applied to the outputs of the bf16 variant). */
+int mla_kv_rmsnorm_rope_cache_fp8(const void* kv_a, int64_t kv_a_stride, const void* k_pe, int64_t k_pe_stride,
+                                  const void* gamma, const void* cos, const void* sin, int64_t cs_stride,
+                                  int32_t cos_step, int32_t interleaved_out, const int64_t* slot_mapping,
+                                  int32_t num_tokens, float eps, void* cache, int64_t page_stride_bytes,
+                                  int64_t row_stride_bytes, int32_t page_size, int64_t num_pages, void* kv_a_out,
+                                  int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride,
+                                  mlahip_stream_t stream);
+
+/* Replaces torch_npu.npu_interleave_rope (npu_mla.py:210, 316; npu_dsa.py:407, 528) for the query's rope part:
+ * x [T, N, 64] through its strides -> out [T, N, 64], same rotation and table conventions as above.  In place
+ * (out == x) only with interleaved_out = 1. */
+int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_stride_h, int64_t num_tokens, int32_t num_heads,
+                        const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, int32_t interleaved_out,
+                        void* out, int64_t out_stride_t, int64_t out_stride_h, mlahip_stream_t stream);
+
 /* ---- (a8, a14) absorbed-MLA paged decode ----------------------------------------------------------
  * Replaces the decode call of torch.ops.npu.npu_fused_infer_attention_score, attention/backends/mla.py:781-804
  * (input_layout "TND_NTD", block_size 128, sparse_mode 3): sequence b owns query tokens

@@ -22,6 +22,11 @@ SIGNATURES = {
     "mla_cache_write_bf16": (c_int32, [P, I64, P, I64, P, I32, P, I64, I64, P, I64, I64, I32, I64, P]),
     "mla_scatter_rows": (c_int32, [P, I64, I32, P, I32, P, I64, I64, I32, I64, P]),
     "mla_cache_write_fp8": (c_int32, [P, I64, P, I64, P, I32, P, I64, I64, I32, I64, P]),
+    "mla_kv_rmsnorm_rope_cache": (c_int32, [P, I64, P, I64, P, P, P, I64, I32, I32, P, I32, F32, P, I64, I64, P, I64, I64,
+                                            I32, I64, P, I64, P, I64, P]),
+    "mla_kv_rmsnorm_rope_cache_fp8": (c_int32, [P, I64, P, I64, P, P, P, I64, I32, I32, P, I32, F32, P, I64, I64, I32, I64,
+                                                P, I64, P, I64, P]),
+    "mla_interleave_rope": (c_int32, [P, I64, I64, I64, I32, P, P, I64, I32, I32, P, I64, I64, P]),
     "mla_decode_fp8": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32, I32, I32, F32, P, I64,
                                  I64, P, P, SZ, I32, P]),
     "mla_gather_paged": (c_int32, [P, I64, I64, P, I64, I64, I64, I32, P, I64, I64, P, I64, I32, P, P, I32, I64, P]),

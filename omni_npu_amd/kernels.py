@@ -102,6 +102,86 @@ def cache_write_fp8(kv_c: torch.Tensor, k_pe: torch.Tensor, slot_mapping: torch.
     _lib.check(rc, "mla_cache_write_fp8")
 
 
+def _table_step(cos: torch.Tensor, sin: torch.Tensor, t: int, table: str):
+    """cos / sin rows [T, W] (singleton dims dropped) and the entry step of pair i: 'half' = the reference's cat(c, c)
+    rows or plain [T,32] rows (entry i), 'repeat' = rows that repeat every entry (entry 2i)."""
+    cos, sin = cos.reshape(cos.shape[0], -1), sin.reshape(sin.shape[0], -1)
+    step = {"half": 1, "repeat": 2}[table]
+    if cos.shape != sin.shape or cos.shape[0] < t or cos.shape[1] < 31 * step + 1 or cos.stride(-1) != 1 or sin.stride(-1) != 1 \
+            or cos.stride(0) != sin.stride(0) or cos.dtype != torch.bfloat16 or sin.dtype != torch.bfloat16:
+        raise ValueError(f"cos / sin must be bf16 [T, >= {31 * step + 1}] rows with equal strides, got {tuple(cos.shape)}")
+    return cos, sin, step
+
+
+def kv_rmsnorm_rope_cache(kv: torch.Tensor, gamma: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                          slot_mapping: torch.Tensor, nope_cache: torch.Tensor, rope_cache: Optional[torch.Tensor],
+                          eps: float = 1e-6, table: str = "half", interleaved_out: bool = False,
+                          kv_a_out: Optional[torch.Tensor] = None, k_pe_out: Optional[torch.Tensor] = None) -> None:
+    """RMSNorm(kv[:, :512]) * gamma and the rotary embedding of kv[:, 512:] written into the paged cache rows
+    ``slot_mapping`` names, in one launch (reference: torch_npu.npu_kv_rmsnorm_rope_cache,
+    src/omni_npu/v1/layers/attention/npu_mla.py:196-206).  ``rope_cache=None`` selects the fp8 cache
+    (``nope_cache`` = uint8 [num_blocks, page, 656])."""
+    _need_cuda(kv, gamma, cos, sin, slot_mapping, nope_cache)
+    lib = _lib.load()
+    kv = kv.reshape(kv.shape[0], -1)
+    if kv.shape[-1] != D_NOPE + D_ROPE or kv.dtype != torch.bfloat16 or kv.stride(-1) != 1:
+        raise ValueError(f"kv must be bf16 [T, 576] with a contiguous last dim, got {kv.dtype} {tuple(kv.shape)}")
+    if gamma.shape != (D_NOPE,) or gamma.dtype != torch.bfloat16 or not gamma.is_contiguous():
+        raise ValueError("gamma must be a contiguous bf16 [512] vector")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.to(torch.int64).contiguous()
+    t = min(slot_mapping.numel(), kv.shape[0])
+    cos, sin, step = _table_step(cos, sin, t, table)
+    for o, w, name in ((kv_a_out, D_NOPE, "kv_a_out"), (k_pe_out, D_ROPE, "k_pe_out")):
+        if o is not None and (o.dim() != 2 or o.shape[0] < t or o.shape[1] != w or o.dtype != torch.bfloat16 or o.stride(-1) != 1
+                              or not o.is_cuda):
+            raise ValueError(f"{name} must be a bf16 GPU tensor [T, {w}]")
+    outs = (kv_a_out.data_ptr() if kv_a_out is not None else None, kv_a_out.stride(0) if kv_a_out is not None else 0,
+            k_pe_out.data_ptr() if k_pe_out is not None else None, k_pe_out.stride(0) if k_pe_out is not None else 0)
+    k_pe = kv[:, D_NOPE:]
+    if rope_cache is None:
+        c = nope_cache
+        if c.dtype != torch.uint8 or c.dim() != 3 or c.shape[-1] != FP8_ROW_BYTES or c.stride(-1) != 1:
+            raise ValueError(f"fp8 cache must be uint8 [num_blocks, page, {FP8_ROW_BYTES}], got {c.dtype} {tuple(c.shape)}")
+        rc = lib.mla_kv_rmsnorm_rope_cache_fp8(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
+                                               cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out),
+                                               slot_mapping.data_ptr(), t, float(eps), c.data_ptr(), c.stride(0), c.stride(1),
+                                               c.shape[1], c.shape[0], *outs, _stream(kv))
+        _lib.check(rc, "mla_kv_rmsnorm_rope_cache_fp8")
+        return
+    _need_cuda(rope_cache)
+    nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
+    if nope.dtype != torch.bfloat16 or rope.dtype != torch.bfloat16 or nope.shape[:2] != rope.shape[:2]:
+        raise ValueError("nope / rope caches must be bf16 and agree on [num_blocks, page]")
+    rc = lib.mla_kv_rmsnorm_rope_cache(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
+                                       cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out),
+                                       slot_mapping.data_ptr(), t, float(eps), nope.data_ptr(), nope.stride(0), nope.stride(1),
+                                       rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[1], nope.shape[0], *outs,
+                                       _stream(kv))
+    _lib.check(rc, "mla_kv_rmsnorm_rope_cache")
+
+
+def interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, out: Optional[torch.Tensor] = None,
+                    table: str = "half", interleaved_out: bool = False) -> torch.Tensor:
+    """Rotary embedding of x [T, N, 64] (pairs (2i, 2i+1)), result cat(o1, o2) like the reference's
+    torch_npu.npu_interleave_rope (src/omni_npu/v1/layers/attention/npu_mla.py:210) or, with ``interleaved_out``, pairs in
+    place.  Returns ``out`` (a new tensor unless given)."""
+    _need_cuda(x, cos, sin)
+    lib = _lib.load()
+    if x.dim() != 3 or x.shape[-1] != D_ROPE or x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+        raise ValueError(f"x must be bf16 [T, N, 64] with a contiguous last dim, got {x.dtype} {tuple(x.shape)}")
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if out.shape != x.shape or out.dtype != x.dtype or out.stride(-1) != 1 or not out.is_cuda:
+        raise ValueError("out must match x")
+    cos, sin, step = _table_step(cos, sin, x.shape[0], table)
+    rc = lib.mla_interleave_rope(x.data_ptr(), x.stride(0), x.stride(1), x.shape[0], x.shape[1], cos.data_ptr(), sin.data_ptr(),
+                                 cos.stride(0), step, int(interleaved_out), out.data_ptr(), out.stride(0), out.stride(1),
+                                 _stream(x))
+    _lib.check(rc, "mla_interleave_rope")
+    return out
+
+
 def gather_paged(nope_cache: torch.Tensor, rope_cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor,
                  cu_seq_lens: torch.Tensor, batch_size: int, seq_starts: Optional[torch.Tensor] = None,
                  total_rows: Optional[int] = None) -> None:

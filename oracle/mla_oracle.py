@@ -35,6 +35,15 @@ Pinning status (what checks each function beyond re-typing its formula lives in
                                   against the mathematics: float64 brute force, the selection invariant
                                   (every kept score >= every dropped score, lowest index on ties), and
                                   "k >= L  ==> sparse == dense decode".
+* ``rms_norm``, ``interleave_rope``,
+  ``kv_rmsnorm_rope_cache``       restate the reference's own torch formulation of the fused vendor op
+                                  (layers/rotary_embedding/rotary_embedding_torch_npu.py:146-173 for the
+                                  rotation and its cat(c, c) tables; the kv_a_layernorm + npu_interleave_rope
+                                  branch of v1/layers/attention/npu_dsa.py:405-408).  The vendor op itself is
+                                  closed: PARITY UNPINNED against it.  Pinned against the mathematics:
+                                  torch.nn.functional.rms_norm, a float64 loop, rotation invariants (pair norms,
+                                  position 0 = de-interleave only, q.k depends on the position difference only)
+                                  and agreement of the two output layouts up to the fixed permutation.
 * ``fp8 quantise / dequantise``   PARITY UNPINNED against the reference (it has no fp8 KV format,
                                   attention/ops.py:11-12 ignores its scale); pinned by the round-trip error
                                   bound of e4m3 (relative 2^-4 per element, exact for representable values).
@@ -268,6 +277,64 @@ def chunked_prefill(q, kv_c_suffix, k_pe_suffix, w_kv_b, nope_cache, rope_cache,
     if ctx_out is not None:
         out, _ = merge_attn_states(ctx_out, ctx_lse.unsqueeze(-1), out, lse.unsqueeze(-1))
     return out.reshape(t, -1)
+
+
+# --------------------------------------------------------------------------------------
+# the step in front of the path: RMSNorm + rotary embedding + cache write
+# --------------------------------------------------------------------------------------
+def rope_tables(positions: torch.Tensor, rotary_dim: int = D_ROPE, base: float = 10000.0, layout: str = "half",
+                dtype=torch.bfloat16):
+    """cos / sin rows for ``positions``: inv_freq = base^(-2i/d), angle = pos * inv_freq
+    (layers/rotary_embedding/deepseek_scaling_rope.py:51-87 without the YaRN blend).  layout "half" gives the rows
+    the reference hands to its fused ops, cat(c, c) (rotary_embedding_torch_npu.py:170-173); "repeat" repeats
+    every entry (c0, c0, c1, c1, ...), the layout tests/integration/attention/test_npu_mla_math.py:125-144 reads
+    with [..., ::2]."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))
+    ang = torch.outer(positions.float(), inv_freq)
+    c, s = ang.cos(), ang.sin()
+    if layout == "half":
+        return torch.cat((c, c), -1).to(dtype), torch.cat((s, s), -1).to(dtype)
+    return c.repeat_interleave(2, -1).to(dtype), s.repeat_interleave(2, -1).to(dtype)
+
+
+def rms_norm(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> torch.Tensor:
+    """y = x * rsqrt(mean(x^2) + eps) * gamma over the last dim, in float64, rounded once to x.dtype
+    (the kv_a_layernorm of v1/layers/attention/npu_dsa.py:405)."""
+    xd = x.double()
+    inv = torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + eps)
+    return (xd * inv * gamma.double()).to(x.dtype)
+
+
+def interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, table: str = "half",
+                    interleaved_out: bool = False) -> torch.Tensor:
+    """x [T, ..., D] with pairs (2i, 2i+1); cos / sin [T, W] rows.  x1 = x[..., 0::2], x2 = x[..., 1::2],
+    o1 = x1*cos - x2*sin, o2 = x2*cos + x1*sin, result cat(o1, o2)
+    (layers/rotary_embedding/rotary_embedding_torch_npu.py:146-163, non-neox branch).  ``interleaved_out`` puts
+    the pairs back in place instead.  float64, rounded once."""
+    d = x.shape[-1]
+    step = {"half": 1, "repeat": 2}[table]
+    c = cos.reshape(cos.shape[0], -1)[:, 0:(d // 2) * step:step].double()
+    s = sin.reshape(sin.shape[0], -1)[:, 0:(d // 2) * step:step].double()
+    while c.dim() < x.dim():
+        c, s = c.unsqueeze(1), s.unsqueeze(1)
+    x1, x2 = x[..., 0::2].double(), x[..., 1::2].double()
+    o1, o2 = x1 * c - x2 * s, x2 * c + x1 * s
+    if interleaved_out:
+        return torch.stack((o1, o2), -1).reshape(x.shape).to(x.dtype)
+    return torch.cat((o1, o2), -1).to(x.dtype)
+
+
+def kv_rmsnorm_rope_cache(kv, gamma, cos, sin, slot_mapping, nope_cache, rope_cache, eps, table="half",
+                          interleaved_out=False):
+    """The fused vendor op torch_npu.npu_kv_rmsnorm_rope_cache (v1/layers/attention/npu_mla.py:196-206) as the
+    composition the reference itself uses when it does not fuse (npu_dsa.py:405-408 + the cache scatter of
+    attention/backends/mla.py:868-881).  Returns (k_pe_rotated, kv_a_normed); the caches are updated in place."""
+    kv = kv.reshape(kv.shape[0], -1)
+    kv_a = rms_norm(kv[:, :D_NOPE], gamma, eps)
+    k_pe = interleave_rope(kv[:, D_NOPE:], cos, sin, table, interleaved_out)
+    cache_write(nope_cache, slot_mapping, kv_a)
+    cache_write(rope_cache, slot_mapping, k_pe)
+    return k_pe, kv_a
 
 
 # --------------------------------------------------------------------------------------
