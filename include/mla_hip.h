@@ -123,8 +123,7 @@ int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_st
                           int32_t max_q_len, int32_t num_heads, float scale, void* workspace, size_t workspace_bytes,
                           int32_t num_splits, mlahip_stream_t stream);
 
-/* seq_lens: the array the split phase was given (partials in chunk order); NULL for the [sequence][split] order
- * that mla_decode_fp8 uses internally.  Output rows must be 16-byte aligned (strides multiples of 8 elements). */
+/* seq_lens: the array the split phase was given (the partials are in its chunk order; required).  Output rows must be 16-byte aligned (strides multiples of 8 elements). */
 int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* seq_lens,
                        const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
                        int32_t num_splits, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
