@@ -59,7 +59,8 @@ int mla_cache_write_fp8(const void* kv_c, int64_t kv_c_stride, const void* k_pe,
  * v1/layers/attention/npu_dsa.py:410-424, 517-527: RMSNorm(kv_a [T,512], gamma, eps) and the rotary embedding of
  * k_pe [T,64] written straight into the paged cache rows named by slot_mapping (negative / out-of-range slots are
  * skipped), plus, when the pointers are not NULL, the normalised latent and the rotated rope key as plain tensors
- * (is_output_kv=True).  kv_a and k_pe are usually the two halves of one [T,576] tensor (k_pe = kv_a + 512).
+ * (is_output_kv=True); slot_mapping = NULL skips the cache altogether (both plain outputs are then required).
+ * kv_a and k_pe are usually the two halves of one [T,576] tensor (k_pe = kv_a + 512).
  * Arithmetic (fp32, one rounding to bf16): y = x * rsqrt(mean(x^2) + eps) * gamma;
  * x1 = k_pe[0::2], x2 = k_pe[1::2], o1 = x1*cos - x2*sin, o2 = x2*cos + x1*sin with pair i reading table entry
  * i*cos_step of the token's cos / sin row (rows cs_stride elements apart): cos_step 1 for the reference's cat(c, c)

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void kv_rmsnorm_rope_cache_kernel(NormRopePara
   const int lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= p.num_tokens) return;
-  const int64_t slot = p.slots[t];
+  const int64_t slot = p.slots ? p.slots[t] : -1;
   const bool store = slot >= 0 && slot < p.num_pages * p.page_size;
   if (!store && !p.kv_a_out && !p.k_pe_out) return;
   const int64_t pg = store ? slot / p.page_size : 0;
@@ -174,20 +174,21 @@ static int norm_rope_impl(bool fp8, const void* kv_a, int64_t kv_a_stride, const
                           int64_t rope_sr_b, int32_t page_size, int64_t num_pages, void* kv_a_out,
                           int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride, hipStream_t stream) {
   const char* who = fp8 ? "mla_kv_rmsnorm_rope_cache_fp8" : "mla_kv_rmsnorm_rope_cache";
-  MLA_REQUIRE(kv_a && k_pe && gamma && slot_mapping && nope_cache && (fp8 || rope_cache), MLA_ERR_NULL,
-              "%s: null pointer argument", who);
+  // without a slot mapping nothing is cached: the normalised latent and the rotated key only go to the plain outputs
+  MLA_REQUIRE(kv_a && k_pe && gamma && (slot_mapping ? (nope_cache && (fp8 || rope_cache)) : (kv_a_out && k_pe_out)),
+              MLA_ERR_NULL, "%s: null pointer argument", who);
   if (int rc = check_tables(who, cos, sin, cs_stride, cos_step)) return rc;
-  MLA_REQUIRE(num_tokens >= 0 && page_size >= 1 && num_pages >= 1 && eps >= 0.f, MLA_ERR_SHAPE,
+  MLA_REQUIRE(num_tokens >= 0 && (!slot_mapping || (page_size >= 1 && num_pages >= 1)) && eps >= 0.f, MLA_ERR_SHAPE,
               "%s: num_tokens=%d page_size=%d num_pages=%lld eps=%g", who, num_tokens, page_size, (long long)num_pages,
               (double)eps);
   MLA_REQUIRE(kv_a_stride % 8 == 0 && k_pe_stride % 8 == 0 && (uintptr_t)kv_a % 16 == 0 && (uintptr_t)k_pe % 16 == 0 &&
-                  (uintptr_t)gamma % 16 == 0 && nope_sp_b % 16 == 0 && nope_sr_b % 16 == 0 &&
-                  (uintptr_t)nope_cache % 16 == 0 &&
-                  (fp8 || (rope_sp_b % 16 == 0 && rope_sr_b % 16 == 0 && (uintptr_t)rope_cache % 16 == 0)) &&
+                  (uintptr_t)gamma % 16 == 0 &&
+                  (!slot_mapping || (nope_sp_b % 16 == 0 && nope_sr_b % 16 == 0 && (uintptr_t)nope_cache % 16 == 0 &&
+                                     (fp8 || (rope_sp_b % 16 == 0 && rope_sr_b % 16 == 0 && (uintptr_t)rope_cache % 16 == 0)))) &&
                   (!kv_a_out || (kv_a_out_stride % 8 == 0 && (uintptr_t)kv_a_out % 16 == 0)) &&
                   (!k_pe_out || (k_pe_out_stride % 8 == 0 && (uintptr_t)k_pe_out % 16 == 0)),
               MLA_ERR_SHAPE, "%s: rows must be 16-byte aligned", who);
-  MLA_REQUIRE(!fp8 || nope_sr_b >= kF8RowB, MLA_ERR_SHAPE, "%s: fp8 cache rows are 656 bytes", who);
+  MLA_REQUIRE(!fp8 || !slot_mapping || nope_sr_b >= kF8RowB, MLA_ERR_SHAPE, "%s: fp8 cache rows are 656 bytes", who);
   if (num_tokens == 0) return MLA_OK;
   NormRopeParams p;
   p.kv_a = (const __bf16*)kv_a; p.kv_a_stride = kv_a_stride; p.k_pe = (const __bf16*)k_pe; p.k_pe_stride = k_pe_stride;

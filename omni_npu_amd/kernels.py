@@ -114,13 +114,14 @@ def _table_step(cos: torch.Tensor, sin: torch.Tensor, t: int, table: str):
 
 
 def kv_rmsnorm_rope_cache(kv: torch.Tensor, gamma: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
-                          slot_mapping: torch.Tensor, nope_cache: torch.Tensor, rope_cache: Optional[torch.Tensor],
+                          slot_mapping: Optional[torch.Tensor], nope_cache: Optional[torch.Tensor],
+                          rope_cache: Optional[torch.Tensor],
                           eps: float = 1e-6, table: str = "half", interleaved_out: bool = False,
                           kv_a_out: Optional[torch.Tensor] = None, k_pe_out: Optional[torch.Tensor] = None) -> None:
     """RMSNorm(kv[:, :512]) * gamma and the rotary embedding of kv[:, 512:] written into the paged cache rows
     ``slot_mapping`` names, in one launch (reference: torch_npu.npu_kv_rmsnorm_rope_cache,
     src/omni_npu/v1/layers/attention/npu_mla.py:196-206).  ``rope_cache=None`` selects the fp8 cache
-    (``nope_cache`` = uint8 [num_blocks, page, 656])."""
+    (``nope_cache`` = uint8 [num_blocks, page, 656]); ``slot_mapping=None`` caches nothing and only fills ``kv_a_out`` / ``k_pe_out``."""
     _need_cuda(kv, gamma, cos, sin, slot_mapping, nope_cache)
     lib = _lib.load()
     kv = kv.reshape(kv.shape[0], -1)
@@ -128,9 +129,9 @@ def kv_rmsnorm_rope_cache(kv: torch.Tensor, gamma: torch.Tensor, cos: torch.Tens
         raise ValueError(f"kv must be bf16 [T, 576] with a contiguous last dim, got {kv.dtype} {tuple(kv.shape)}")
     if gamma.shape != (D_NOPE,) or gamma.dtype != torch.bfloat16 or not gamma.is_contiguous():
         raise ValueError("gamma must be a contiguous bf16 [512] vector")
-    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+    if slot_mapping is not None and (slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous()):
         slot_mapping = slot_mapping.to(torch.int64).contiguous()
-    t = min(slot_mapping.numel(), kv.shape[0])
+    t = min(slot_mapping.numel(), kv.shape[0]) if slot_mapping is not None else kv.shape[0]
     cos, sin, step = _table_step(cos, sin, t, table)
     for o, w, name in ((kv_a_out, D_NOPE, "kv_a_out"), (k_pe_out, D_ROPE, "k_pe_out")):
         if o is not None and (o.dim() != 2 or o.shape[0] < t or o.shape[1] != w or o.dtype != torch.bfloat16 or o.stride(-1) != 1
@@ -139,6 +140,14 @@ def kv_rmsnorm_rope_cache(kv: torch.Tensor, gamma: torch.Tensor, cos: torch.Tens
     outs = (kv_a_out.data_ptr() if kv_a_out is not None else None, kv_a_out.stride(0) if kv_a_out is not None else 0,
             k_pe_out.data_ptr() if k_pe_out is not None else None, k_pe_out.stride(0) if k_pe_out is not None else 0)
     k_pe = kv[:, D_NOPE:]
+    if slot_mapping is None:
+        if kv_a_out is None or k_pe_out is None:
+            raise ValueError("without a slot mapping both kv_a_out and k_pe_out are required")
+        rc = lib.mla_kv_rmsnorm_rope_cache(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
+                                           cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out), None, t,
+                                           float(eps), None, 0, 0, None, 0, 0, 1, 1, *outs, _stream(kv))
+        _lib.check(rc, "mla_kv_rmsnorm_rope_cache")
+        return
     if rope_cache is None:
         c = nope_cache
         if c.dtype != torch.uint8 or c.dim() != 3 or c.shape[-1] != FP8_ROW_BYTES or c.stride(-1) != 1:
