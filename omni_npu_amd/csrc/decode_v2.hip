@@ -107,7 +107,16 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h32 = lane & 31;
   const int half = lane >> 5;
-  const int chunk = blockIdx.x, grp = blockIdx.z;
+  // The row groups of one chunk (more than 128 query rows: several tokens per sequence) stream the same cache rows.
+  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has its own L2, so they are renumbered to
+  // sit on one XCD, next to each other in its queue: they run at the same time and share the rows in that L2.
+  int chunk = blockIdx.x, grp = blockIdx.z;
+  if (gridDim.z > 1 && (gridDim.x & 7) == 0) {
+    const int lin = blockIdx.x + gridDim.x * blockIdx.z;
+    const int j = lin >> 3;
+    grp = j % gridDim.z;
+    chunk = (j / gridDim.z) * 8 + (lin & 7);
+  }
   const int r_max = p.max_q_len * p.num_heads;
   if (grp * 128 >= r_max) return;
   const uint32_t lds0 = lds_addr_of(lds);

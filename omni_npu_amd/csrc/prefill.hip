@@ -74,7 +74,20 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h32 = lane & 31, half = lane >> 5;
-  const int qb = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+  // Workgroups go to the eight XCDs round-robin in launch order (x fastest), and each XCD has its own L2.  All query
+  // blocks of one (sequence, head) stream the same keys and values, so they are renumbered to sit on ONE XCD, next to each
+  // other in its queue: they then run at the same time and all but the first find the K / V tiles in that L2.
+  int qb = blockIdx.x, head = blockIdx.y, b = blockIdx.z;
+  {
+    const int nqb = gridDim.x, npairs = gridDim.y * gridDim.z;
+    if ((npairs & 7) == 0) {
+      const int lin = blockIdx.x + nqb * (blockIdx.y + gridDim.y * blockIdx.z);
+      const int j = lin >> 3, pair = (j / nqb) * 8 + (lin & 7);
+      qb = j % nqb;
+      head = pair % gridDim.y;
+      b = pair / gridDim.y;
+    }
+  }
   const int q0 = p.cu_q[b], sq = p.cu_q[b + 1] - q0;
   const int k0 = p.cu_k[b], sk = p.cu_k[b + 1] - k0;
   if (qb * kPfRows >= sq) return;
