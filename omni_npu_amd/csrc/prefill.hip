@@ -69,6 +69,40 @@ __device__ __forceinline__ void pf_issue_tile(const PrefillParams& p, int64_t k0
   }
 }
 
+// Per-lane source offsets of a FULL tile (all 64 keys exist), relative to the tile's first key: the copies then need one
+// uniform base per tensor and no per-lane address arithmetic.
+struct PfLaneOffsets { uint32_t kn[4], v[4], kp[2]; };
+__device__ __forceinline__ PfLaneOffsets pf_lane_offsets(const PrefillParams& p, int wave, int lane) {
+  PfLaneOffsets o;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = (wave * 4 + i) * 4 + (lane >> 4);
+    const int c = (lane & 15) ^ pf_swz16(r & 15);
+    o.kn[i] = (uint32_t)(r * p.kn_st * 2 + c * 16);
+    o.v[i] = (uint32_t)(r * p.v_st * 2 + c * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = (wave * 2 + i) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ pf_swz8(r & 15);
+    o.kp[i] = (uint32_t)(r * p.kp_st * 2 + c * 16);
+  }
+  return o;
+}
+__device__ __forceinline__ void pf_issue_full_tile(const PrefillParams& p, const PfLaneOffsets& o, int64_t k0, int head,
+                                                   uint32_t buf, int wave) {
+  const char* kn = (const char*)(p.k_nope + k0 * p.kn_st + (int64_t)head * p.kn_sh);
+  const char* vv = (const char*)(p.v + k0 * p.v_st + (int64_t)head * p.v_sh);
+  const char* kp = (const char*)(p.k_pe + k0 * p.kp_st);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    dma16_sv(kn, o.kn[i], buf + (wave * 4 + i) * 1024);
+    dma16_sv(vv, o.v[i], buf + kPfKnB + kPfKrB + (wave * 4 + i) * 1024);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; i++) dma16_sv(kp, o.kp[i], buf + kPfKnB + (wave * 2 + i) * 1024);
+}
+
 __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
@@ -97,6 +131,10 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
   const int shift = sk - sq;                                  // right-down alignment of the causal mask
   int limit = p.causal ? row + shift + 1 : sk;                // visible keys of this row
   limit = !row_ok ? 0 : (limit < 0 ? 0 : (limit > sk ? sk : limit));
+  int wave_min_limit = limit;                                 // fewest keys any row of this wave can see
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) { const int other = __shfl_xor(wave_min_limit, o, 64); wave_min_limit = other < wave_min_limit ? other : wave_min_limit; }
+  wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
   // keys any row of this workgroup can see
   int wg_limit = sk;
   if (p.causal) {
@@ -118,7 +156,14 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
   if (tiles > 0) {
     const uint32_t lds0 = lds_addr_of(lds);
     const int64_t klast = (int64_t)k0 + sk - 1;
-    pf_issue_tile(p, k0, klast, head, lds0, wave, lane);
+    const PfLaneOffsets lane_off = pf_lane_offsets(p, wave, lane);
+    const bool fast_ok = (uint64_t)p.kn_st * 128 < (1u << 31) && (uint64_t)p.v_st * 128 < (1u << 31) && (uint64_t)p.kp_st * 128 < (1u << 31);
+    auto issue = [&](int tile, uint32_t buf) {
+      const int64_t first = (int64_t)k0 + (int64_t)tile * kPfTile;
+      if (fast_ok && first + kPfTile - 1 <= klast) pf_issue_full_tile(p, lane_off, first, head, buf, wave);
+      else pf_issue_tile(p, first, klast, head, buf, wave, lane);
+    };
+    issue(0, lds0);
 
     bf16x8 qf[12];
     {
@@ -153,7 +198,7 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
     for (int tile = 0; tile < tiles; tile++) {
       const char* buf = lds + (tile & 1) * kPfBufB;
       if (tile + 1 < tiles) {
-        pf_issue_tile(p, (int64_t)k0 + (tile + 1) * kPfTile, klast, head, lds0 + ((tile + 1) & 1) * kPfBufB, wave, lane);
+        issue(tile + 1, lds0 + ((tile + 1) & 1) * kPfBufB);
         MLA_WAIT_VMCNT(10);
       } else {
         MLA_WAIT_VMCNT(0);
@@ -176,22 +221,30 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 128 + roff[kk]);
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[8 + kk], s, 0, 0, 0);
         }
-        const int key_lane0 = key_base + tb * 32 + 4 * half;
-        float mx = -INFINITY;
+        // Only blocks that some row of this wave cannot see in full pay for the mask (causal diagonal, end of the keys,
+        // rows past the end of the sequence); everywhere else the scores go straight to the maximum.  The scale is
+        // folded into the exponent's multiply-add (scale > 0, so the maximum of the raw scores is the raw maximum).
+        if (key_base + tb * 32 + 32 > wave_min_limit) {
+          const int key_lane0 = key_base + tb * 32 + 4 * half;
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int key = key_lane0 + 8 * (r >> 2) + (r & 3);
-          s[r] = key < limit ? s[r] * p.scale_log2 : -INFINITY;
-          mx = fmaxf(mx, s[r]);
+          for (int r = 0; r < 16; r++) {
+            const int key = key_lane0 + 8 * (r >> 2) + (r & 3);
+            s[r] = key < limit ? s[r] : -INFINITY;
+          }
         }
-        mx = fmaxf(mx, xor32(mx));
+        float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+        for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, s[r]), s[r + 1]);
+        mx = fmaxf(mx, s[15]);
+        mx = fmaxf(mx, xor32(mx)) * p.scale_log2;
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = fast_exp2(m_run - m_safe);
+        const float neg = -m_safe;
         float psum = 0.f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          s[r] = fast_exp2(s[r] - m_safe);
+          s[r] = fast_exp2(__builtin_fmaf(s[r], p.scale_log2, neg));
           psum += s[r];
         }
         l_run = l_run * alpha + psum;
@@ -260,6 +313,7 @@ extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64
   MLA_REQUIRE(batch >= 0 && num_heads >= 1 && max_q_len >= 0 && batch <= 65535 && num_heads <= 65535, MLA_ERR_SHAPE,
               "mla_prefill_varlen: batch=%d num_heads=%d max_q_len=%d", batch, num_heads, max_q_len);
   MLA_REQUIRE(out_dtype == 0 || out_dtype == 1, MLA_ERR_UNSUPPORTED, "mla_prefill_varlen: out dtype code %d", out_dtype);
+  MLA_REQUIRE(scale > 0.f, MLA_ERR_UNSUPPORTED, "mla_prefill_varlen: the softmax scale must be positive (got %g)", (double)scale);
   MLA_REQUIRE(qn_stride_t % 8 == 0 && qn_stride_h % 8 == 0 && qp_stride_t % 8 == 0 && qp_stride_h % 8 == 0 &&
                   kn_stride_t % 8 == 0 && kn_stride_h % 8 == 0 && kp_stride_t % 8 == 0 && v_stride_t % 8 == 0 &&
                   v_stride_h % 8 == 0 && out_stride_t % 4 == 0 && out_stride_h % 4 == 0 && (uintptr_t)q_nope % 16 == 0 &&
