@@ -349,7 +349,7 @@ def bench_prologue(K, dev, args):
         "metric": "fused RMSNorm + rotary embedding + cache write, plus query rotary embedding, us (T = 8192 tokens, 128 heads)",
         "value": round(step_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "higher_is_better": False, "dtype": "bf16 (fp32 arithmetic)", "data": "synthetic",
-        "config": {"workload": "step before the attention path (next row 1)", "tokens": [64, 8192], "heads": N, "seed": args.seed},
+        "config": {"workload": "step before the attention path: fused norm + rotary + cache write", "tokens": [64, 8192], "heads": N, "seed": args.seed},
         "sizes": {str(k): v for k, v in out.items()},
         "roofline": {"kernel": "kv_rmsnorm_rope_cache_kernel<false> + interleave_rope_kernel", "bound": "hbm",
                      "achieved": round(tot_bytes / step_us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

@@ -28,7 +28,7 @@ typedef struct ihipStream_t* mlahip_stream_t;
 int mlahip_version(void);
 const char* mlahip_last_error_string(void);
 
-/* ---- (a6) latent-KV cache write ------------------------------------------------------------------
+/* ---- latent-KV cache write ------------------------------------------------------------------
  * Replaces torch_npu.npu_scatter_nd_update_ in store_kv, attention/backends/mla.py:868-881 and
  * attention/backends/dsa.py:359-362:  cache.flatten(0,1)[slot[t]] = src[t]; slot = page * page_size + offset;
  * negative slots (padding) and slots past the cache are skipped. */
@@ -54,7 +54,7 @@ int mla_cache_write_fp8(const void* kv_c, int64_t kv_c_stride, const void* k_pe,
                         const int64_t* slot_mapping, int32_t num_tokens, void* cache, int64_t page_stride_bytes,
                         int64_t row_stride_bytes, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
 
-/* ---- the step in front of the path, fused (next row 1) ----------------------------------------------
+/* ---- the step in front of the path, fused ----------------------------------------------
  * Replaces torch_npu.npu_kv_rmsnorm_rope_cache as called at v1/layers/attention/npu_mla.py:196-206, 296-309 and
  * v1/layers/attention/npu_dsa.py:410-424, 517-527: RMSNorm(kv_a [T,512], gamma, eps) and the rotary embedding of
  * k_pe [T,64] written straight into the paged cache rows named by slot_mapping (negative / out-of-range slots are
@@ -92,7 +92,7 @@ int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_stride_h, i
                         const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, int32_t interleaved_out,
                         void* out, int64_t out_stride_t, int64_t out_stride_h, mlahip_stream_t stream);
 
-/* ---- (a8, a14) absorbed-MLA paged decode ----------------------------------------------------------
+/* ---- absorbed-MLA paged decode ----------------------------------------------------------
  * Replaces the decode call of torch.ops.npu.npu_fused_infer_attention_score, attention/backends/mla.py:781-804
  * (input_layout "TND_NTD", block_size 128, sparse_mode 3): sequence b owns query tokens
  * [b*max_q_len, (b+1)*max_q_len) or [qsl[b], qsl[b+1]); token i of its s tokens sees keys [0, L_b - s + i].
@@ -140,7 +140,7 @@ int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h,
                    int32_t num_heads, float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
                    void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
 
-/* ---- (a12, a13) chunked-context helpers -------------------------------------------------------------
+/* ---- chunked-context helpers -------------------------------------------------------------
  * mla_gather_paged replaces ops.gather_and_maybe_dequant_cache (attention/ops.py:5-41, which never dequantises):
  * dst[cu[i] + j] = cat(nope[row], rope[row]) for position seq_starts[i] + j, j < cu[i+1]-cu[i].
  * mla_merge_states replaces ops.merge_attn_states (attention/ops.py:44-106): +inf lse reads as -inf, both sides
@@ -156,7 +156,7 @@ int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_str
                      int32_t in_dtype, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
                      float* out_lse /* may be NULL */, int32_t tokens, int32_t heads, int32_t dim, mlahip_stream_t stream);
 
-/* ---- (a10, a11) non-absorbed varlen attention for prefill -------------------------------------------
+/* ---- non-absorbed varlen attention for prefill -------------------------------------------
  * Replaces the prefill calls of npu_fused_infer_attention_score, attention/backends/mla.py:574-590 (suffix:
  * right-down causal, sparse_mode 3) and :415-431 (context chunk: no mask, softmax_lse_flag): q_nope [T,N,128],
  * q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64] shared by all heads (mla.py:579 repeats it), v [Tk,N,128];
@@ -169,7 +169,7 @@ int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_strid
                        int32_t max_q_len, int32_t causal, float scale, void* out, int64_t out_stride_t,
                        int64_t out_stride_h, int32_t out_dtype, float* lse_out, mlahip_stream_t stream);
 
-/* ---- (a15) DSA lightning indexer --------------------------------------------------------------------
+/* ---- DSA lightning indexer --------------------------------------------------------------------
  * Replaces torch.ops.custom.npu_lightning_indexer, v1/layers/attention/npu_dsa.py:92-103 and
  * vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:133-146, in two steps:
  * dsa_indexer_scores_fp8: logits[t,s] = k_scale[s] * sum_h w[t,h] (* q_scale[t,h]) * relu(q8[t,h,:] . k8[s,:])
@@ -209,7 +209,7 @@ int dsa_topk_rows(const float* logits, int64_t logits_stride, const int32_t* seq
                   int32_t* rows, int64_t rows_stride, int32_t* counts, void* workspace /* may be NULL */,
                   size_t workspace_bytes, mlahip_stream_t stream);
 
-/* ---- (a16) sparse MLA over the selected keys ----------------------------------------------------------
+/* ---- sparse MLA over the selected keys ----------------------------------------------------------
  * Replaces torch.ops.custom.npu_sparse_flash_attention, attention/backends/dsa.py:259-291 (sparse_block_size 1,
  * layout_kv "PA_BSND"): dsa_build_rows maps the [T,k] logical positions (-1 = unused,
  * v1/layers/attention/npu_dsa.py:553-555) through the block table to flat cache rows, compacted, with a count per

@@ -138,7 +138,7 @@ def test_decode_invariants():
 
 
 def test_absorbed_decode_equals_non_absorbed_attention():
-    """Ties decode (a8) to prefill (a10): absorb -> latent attention -> v-up-proj  ==  attention on the
+    """Ties decode to prefill: absorb -> latent attention -> v-up-proj  ==  attention on the
     up-projected keys/values (weight layout of tests/integration/attention/test_npu_mla_math.py:302-313)."""
     g = torch.Generator().manual_seed(7)
     n, p, v, L = 4, 128, 128, 37
