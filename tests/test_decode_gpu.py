@@ -125,6 +125,20 @@ def test_decode_empty_and_tiny_sequences_in_one_batch(dev):
         assert torch.allclose(lse[1:].cpu(), ref_lse[1:], atol=2e-2, rtol=0)
 
 
+def test_decode_row_groups_renumbered_onto_one_xcd(dev):
+    """256 query rows per sequence (two row groups) and a chunk count that is a multiple of eight: the kernel renumbers
+    its workgroups so that the groups of a chunk share an XCD; results must not change."""
+    case = O.make_decode_case(4, 128, 200, 900, seed=13, q_len=2)
+    ref = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"])
+    for splits in (2, 4):                                     # 8 and 16 chunks
+        got, _ = _run(case, dev, num_splits=splits)
+        attn_close(got, ref, MAX_ABS, MEAN_REL)
+    got3, _ = _run(case, dev, num_splits=3)                   # 12 chunks: launch order kept
+    got2, _ = _run(case, dev, num_splits=2)
+    assert (got3.float() - got2.float()).abs().max().item() <= 8e-3
+
+
 @pytest.mark.parametrize("q_len,heads", [(2, 128), (3, 16), (2, 40)])
 def test_decode_mtp_right_down_causal(dev, q_len, heads):
     """q_len > 1: token i of a request sees keys [0, L - q_len + i]."""

@@ -30,6 +30,8 @@ def _case(seed, q_lens, k_lens, n):
     (False, [16, 48, 7], [32, 100, 64], 4),          # context chunk: no mask, more keys than queries
     (True, [40, 70], [100, 70], 2),                  # right-down alignment: more keys than queries
     (False, [5, 9], [0, 33], 2),                     # an empty key range: zeros and lse = -inf
+    (True, [300, 129, 64], [300, 200, 64], 8),       # 24 (sequence, head) pairs: the XCD-aware renumbering is active
+    (False, [130, 260], [500, 70], 16),              # the same without a mask
 ])
 def test_prefill_varlen_matches_oracle(dev, causal, q_lens, k_lens, n):
     from omni_npu_amd import kernels as K
