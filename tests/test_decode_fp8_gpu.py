@@ -103,3 +103,35 @@ def test_decode_step_replayed_from_a_hip_graph(dev):
         c["rope"] = rope
         ref = O.absorbed_decode(q1, c["q_rope"], deq, rope, c["block_table"], new_lens, c["scale"])
         attn_close(got, ref, FP8_MAX_ABS, FP8_MEAN_REL)
+
+
+def test_decode_fp8_large_shape_properties(dev):
+    """Batch 32, MTP pairs, contexts of 8k-16k over the fp8 cache (the benchmark's shape at an eighth of its batch): a sample of
+    sequences against the oracle, invariance under the split count, and bit-identical results after moving every physical
+    page (the block tables rewritten to match)."""
+    from omni_npu_amd import kernels as K
+    batch, heads, q_len = 32, 128, 2
+    c = O.make_decode_case(batch, heads, 8192, 16384, seed=17, q_len=q_len)
+    q8, sc = O.fp8_quant_block(c["nope"].float())
+    cache = _fill_cache(c, dev)
+    qn, qr, bt, lens = c["q_nope"].to(dev), c["q_rope"].to(dev), c["block_table"].to(dev), c["seq_lens"].to(dev)
+
+    def run(cache_, bt_, splits):
+        out = torch.empty(batch * q_len, heads, 512, dtype=torch.bfloat16, device=dev)
+        K.decode_fp8(qn, qr, cache_, bt_, lens, c["scale"], out, q_len=q_len, num_splits=splits)
+        torch.cuda.synchronize()
+        return out
+
+    got8, got5 = run(cache, bt, 8), run(cache, bt, 5)         # 256 chunks (row groups renumbered) and 160
+    assert (got8.float() - got5.float()).abs().max().item() <= 8e-3
+    deq = O.fp8_dequant_block(q8, sc)
+    for b in (0, 13, 31):
+        ref = O.absorbed_decode(c["q_nope"][b * q_len:(b + 1) * q_len], c["q_rope"][b * q_len:(b + 1) * q_len], deq,
+                                c["rope"], c["block_table"][b:b + 1], c["seq_lens"][b:b + 1], c["scale"])
+        attn_close(got8[b * q_len:(b + 1) * q_len], ref, FP8_MAX_ABS, FP8_MEAN_REL)
+    nblk = cache.shape[0]
+    perm = torch.randperm(nblk, generator=torch.Generator().manual_seed(2))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(nblk)
+    got_perm = run(cache[perm.to(dev)].contiguous(), inv[c["block_table"].long()].to(torch.int32).to(dev), 8)
+    assert torch.equal(got_perm, got8)
