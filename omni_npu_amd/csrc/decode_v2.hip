@@ -703,15 +703,20 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
 // N-way merge of the partials of the query rows (src/omni_npu/attention/ops.py:109-141), for the chunk layout written
 // by mla_decode_v2_kernel.  The partials of sequence b are those of the chunks that hold blocks of it, numbered
 // chunk + b.  A wavefront merges kRedRows consecutive rows of one sequence (lane l owns columns 8l..8l+7): it derives
-// the chunk list once, then asks for everything it needs of up to kRedParts partials of all its rows before it uses
-// any of it - the kernel is a chain of dependent memory round trips, and this keeps the chain at two.
-constexpr int kRedRows = 2;
+// the chunk list once, fetches the per-row records of up to kRedParts partials with scalar loads, then asks for the
+// partials and the latent vectors of the flagged dominant keys together before it uses any of them - the kernel is a
+// chain of dependent memory round trips, and this keeps the vector part of the chain at one.  (One row per wave keeps it
+// at four waves per SIMD; the gathers of the dominant keys' vectors are a third of its time.)
+constexpr int kRedRows = 1;
 constexpr int kRedParts = 6;
 __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
   const int lane = threadIdx.x & 63;
   const int r_max = p.max_q_len * p.num_heads;
   const int groups = (r_max + kRedRows - 1) / kRedRows;     // row groups per sequence
-  for (int64_t gw = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6); gw < (int64_t)p.batch * groups; gw += (int64_t)gridDim.x * 4) {
+  // (the wave number is made a scalar: everything derived from it, the addresses of the per-row records included, then
+  // lives in scalar registers and is fetched with scalar loads)
+  for (int64_t gw = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6); gw < (int64_t)p.batch * groups;
+       gw += (int64_t)gridDim.x * 4) {
   const int b = (int)(gw / groups);
   const int row0 = (int)(gw - (int64_t)b * groups) * kRedRows;
   int q0, qlen;
@@ -774,8 +779,11 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
         part[q] = c <= c_last ? (int64_t)(c + b) * r_max + row0 : -1;
         if (c <= c_last) { np++; c++; }
       }
+      // The per-row records (log-sum-exp, correction factor, address of the dominant key's latent vector) are uniform:
+      // scalar loads.  Once they are here the partials AND the latent vectors of the flagged segments are asked for
+      // together, so that the whole pass costs one vector-memory round trip.
       float lse[kRedRows][kRedParts], cs[kRedRows][kRedParts];
-      h8 v[kRedRows][kRedParts];
+      const __bf16* cp[kRedRows][kRedParts];
 #pragma unroll
       for (int q = 0; q < kRedParts; q++)
 #pragma unroll
@@ -784,7 +792,19 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
           const int64_t pr = on ? part[q] + j : 0;
           lse[j][q] = on ? p.lse_part[pr] : -INFINITY;
           cs[j][q] = on ? p.corr_scale[pr] : 0.f;
+          cp[j][q] = p.corr_row[pr];
+          if (lse[j][q] == INFINITY || lse[j][q] == -INFINITY) cs[j][q] = 0.f;
+        }
+      h8 v[kRedRows][kRedParts];
+      bf16x8 kv[kRedRows][kRedParts];
+#pragma unroll
+      for (int q = 0; q < kRedParts; q++)
+#pragma unroll
+        for (int j = 0; j < kRedRows; j++) {
+          const bool on = q < np && row0 + j < rows;
+          const int64_t pr = on ? part[q] + j : 0;
           v[j][q] = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
+          if (cs[j][q] != 0.f) kv[j][q] = *(const bf16x8*)(cp[j][q] + lane * 8);
         }
 #pragma unroll
       for (int q = 0; q < kRedParts; q++)
@@ -800,9 +820,8 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
           for (int e = 0; e < 8; e++) a[j][e] = a[j][e] * so + (float)v[j][q][e] * w;
           // the split kernel rounded this segment's dominant probability to bf16: put the difference back
           if (cs[j][q] != 0.f) {
-            const bf16x8 kv = *(const bf16x8*)(p.corr_row[part[q] + j] + lane * 8);
 #pragma unroll
-            for (int e = 0; e < 8; e++) a[j][e] += (float)kv[e] * (w * cs[j][q]);
+            for (int e = 0; e < 8; e++) a[j][e] += (float)kv[j][q][e] * (w * cs[j][q]);
           }
         }
     }
