@@ -411,11 +411,13 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   // (positive) values through an unsigned maximum, so no compare-and-select chain and no branch is needed.  Two values
   // closer than 2^-18 relative may swap places, which only matters to a correction that is itself a rounding error.
   auto argmax_pack = [&](const f32x16& s) -> uint32_t {
-    // (plain assembly without side effects: the optimiser mangles the equivalent C++ reduction)
-    const uint32_t keep = ~31u;
+    // The tagging is left to the compiler on purpose: the probabilities come out of v_exp_f32, and a vector-ALU
+    // instruction that reads the result of a transcendental one needs a wait state in between, which the compiler only
+    // inserts in front of instructions it can see into (not in front of inline assembly).  The maximum chain is plain
+    // assembly without side effects (the optimiser mangles the equivalent C++ reduction); it only reads tagged values.
     uint32_t u[16];
 #pragma unroll
-    for (int r = 0; r < 16; r++) asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(u[r]) : "v"(s[r]), "s"(keep), "n"(r));
+    for (int r = 0; r < 16; r++) u[r] = (__float_as_uint(s[r]) & ~31u) | (uint32_t)r;
     uint32_t pk = u[0];
 #pragma unroll
     for (int r = 1; r < 15; r += 2) asm("v_max3_u32 %0, %1, %2, %3" : "=v"(pk) : "v"(pk), "v"(u[r]), "v"(u[r + 1]));

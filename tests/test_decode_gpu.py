@@ -43,6 +43,64 @@ def test_decode_config1_plumbing(dev, num_splits):
     assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
 
 
+@pytest.mark.parametrize("heads,num_splits", [(16, 1), (16, 3), (128, 2)])
+def test_decode_dominant_key_records_name_the_right_cache_row(dev, heads, num_splits):
+    """The split phase leaves, per partial row, the cache row of the chunk's most probable key when that key carries more
+    than 1/16 of the chunk's weight (the merge phase takes the bf16 rounding of that probability out again).  A record
+    that names another key of the same 32-key block still passes the attention tolerance most of the time, so the
+    records are checked directly: every recorded row must be the most probable key of its head within its 32-key block
+    (chunks are cut at multiples of 32 keys, so blocks are 32-aligned within the sequence), and keys with more than 1/8 of their whole
+    row's weight must be recorded."""
+    from omni_npu_amd import kernels as K
+    from omni_npu_amd import _lib
+    case = O.make_decode_case(4, heads, 128, 1024, seed=0)
+    b, n = 4, heads
+    nope = case["nope"].to(dev)
+    ws = torch.zeros(_lib.load().mla_decode_workspace_bytes(b, 1, n, num_splits), dtype=torch.uint8, device=dev)
+    out = torch.empty(b, n, 512, dtype=torch.bfloat16, device=dev)
+    K.decode(case["q_nope"].to(dev), case["q_rope"].to(dev), nope, case["rope"].to(dev), case["block_table"].to(dev),
+             case["seq_lens"].to(dev), case["scale"], out, q_len=1, num_splits=num_splits, workspace=ws)
+    torch.cuda.synchronize()
+    rows = b * (num_splits + 1) * n                      # partial rows: fp16 outputs, then lse, scale, row address
+    w = ws.cpu()
+    off = rows * 512 * 2 + rows * 4
+    corr_scale = w[off:off + rows * 4].view(torch.float32)
+    corr_row = w[off + rows * 4:off + rows * 12].view(torch.int64)
+    row_bytes = nope.stride(-2) * 2
+    recorded = {}                                        # (cache slot, head) of every record
+    for i in torch.nonzero(corr_scale).flatten().tolist():
+        delta = int(corr_row[i]) - nope.data_ptr()
+        assert delta % row_bytes == 0 and 0 <= delta // row_bytes < nope.shape[0] * nope.shape[1]
+        recorded[(delta // row_bytes, i % n)] = i
+    assert len(recorded) >= 8                            # the case has peaked rows; an empty set would test nothing
+    checked = expected = found = 0
+    for s in range(b):
+        L = int(case["seq_lens"][s])
+        slots = O.slots_for(case["block_table"], s, 0, L)
+        kn = case["nope"].view(-1, 512)[slots].float()
+        kr = case["rope"].view(-1, 64)[slots].float()
+        sc = (case["q_nope"][s].float() @ kn.T + case["q_rope"][s].float() @ kr.T) * case["scale"]
+        p = torch.softmax(sc, -1)
+        pos_of = {int(v): t for t, v in enumerate(slots.tolist())}
+        for (slot, h), i in recorded.items():
+            if slot not in pos_of:
+                continue
+            t = pos_of[slot]
+            blk = p[h, (t // 32) * 32:min(L, (t // 32) * 32 + 32)]
+            assert p[h, t] >= blk.max() * (1 - 1e-4), (s, h, t, int(blk.argmax()) + (t // 32) * 32)
+            checked += 1
+        top = p.argmax(-1)
+        for h in range(n):
+            if p[h, top[h]] > 1 / 8:
+                expected += 1
+                found += (int(slots[top[h]]), h) in recorded
+    assert checked == len(recorded)                      # every record points into one of the four sequences
+    # A dominant key in the first 32-key block of its chunk has probability exactly 1 against that block's reference
+    # maximum, which bf16 holds exactly: its correction is zero and reads as "no record".  That is about one block in
+    # ten here; anything beyond that would be records getting lost.
+    assert expected >= 8 and found >= 0.8 * expected, (found, expected)
+
+
 @pytest.mark.parametrize("lens", [(1, 1), (1, 70), (63, 65), (127, 129), (200, 300)])
 def test_decode_ragged_edges(dev, lens):
     """Sequence lengths around tile (64) and page (128) boundaries, 128 heads, head-major output."""
