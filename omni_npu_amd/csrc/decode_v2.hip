@@ -709,16 +709,25 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
 // partials and the latent vectors of the flagged dominant keys together before it uses any of them - the kernel is a
 // chain of dependent memory round trips, and this keeps the vector part of the chain at one.  (One row per wave keeps it
 // at four waves per SIMD; the gathers of the dominant keys' vectors are a third of its time.)
+// With many partials per sequence (few sequences, long contexts: up to 257 partials of one row) a single wavefront would
+// walk them in dozens of dependent round trips, so the kWide form gives a row to a whole workgroup: wavefront w merges
+// every fourth partial, sixteen per pass, and the four running states are merged through LDS at the end.
 constexpr int kRedRows = 1;
-constexpr int kRedParts = 6;
+constexpr int kRedPartsNarrow = 6, kRedPartsWide = 16;
+template <bool kWide>
 __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
+  constexpr int kRedParts = kWide ? kRedPartsWide : kRedPartsNarrow;
+  __shared__ float comb_ml[kWide ? 8 : 1];                  // wide: running maximum and sum of wavefronts 0..3
+  __shared__ float comb_a[kWide ? 4 * 64 * 8 : 1];          //       and their unnormalised rows
   const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int r_max = p.max_q_len * p.num_heads;
   const int groups = (r_max + kRedRows - 1) / kRedRows;     // row groups per sequence
   // (the wave number is made a scalar: everything derived from it, the addresses of the per-row records included, then
   // lives in scalar registers and is fetched with scalar loads)
-  for (int64_t gw = (int64_t)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6); gw < (int64_t)p.batch * groups;
-       gw += (int64_t)gridDim.x * 4) {
+  const int64_t gw_first = kWide ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+  const int64_t gw_step = kWide ? (int64_t)gridDim.x : (int64_t)gridDim.x * 4;
+  for (int64_t gw = gw_first; gw < (int64_t)p.batch * groups; gw += gw_step) {
   const int b = (int)(gw / groups);
   const int row0 = (int)(gw - (int64_t)b * groups) * kRedRows;
   int q0, qlen;
@@ -772,6 +781,13 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
       c = (int)((((int64_t)before + 1) * G - 1) / T);
       c_last = (int)((((int64_t)before + mine) * G - 1) / T);
     }
+    // wide: wavefront w takes the chunks c + w, c + w + 4, ...; where chunks have to be tested one by one (tiny
+    // workloads, a handful of partials) wavefront 0 takes them all
+    int c_step = 1;
+    if constexpr (kWide) {
+      if (dense_chunks) { c += wave; c_step = 4; }
+      else if (wave != 0) c = c_last + 1;
+    }
     while (c <= c_last) {
       int64_t part[kRedParts];                               // partial numbers of this pass (uniform), -1 = none
       int np = 0;
@@ -779,11 +795,25 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
       for (int q = 0; q < kRedParts; q++) {
         while (c <= c_last && !dense_chunks && !holds_blocks(c)) c++;     // wrote nothing for this sequence
         part[q] = c <= c_last ? (int64_t)(c + b) * r_max + row0 : -1;
-        if (c <= c_last) { np++; c++; }
+        if (c <= c_last) { np++; c += c_step; }
       }
       // The per-row records (log-sum-exp, correction factor, address of the dominant key's latent vector) are uniform:
-      // scalar loads.  Once they are here the partials AND the latent vectors of the flagged segments are asked for
-      // together, so that the whole pass costs one vector-memory round trip.
+      // scalar loads.  One-wavefront form: once they are here the partials AND the latent vectors of the flagged segments
+      // are asked for together, so that the whole pass costs one vector-memory round trip (measured: asking for the
+      // partials first costs it registers and 4 us).  Wide form: the partials are asked for first, their addresses
+      // need nothing but the chunk list, and the records travel at the same time.
+      h8 v[kRedRows][kRedParts];
+      auto ask_partials = [&] {
+#pragma unroll
+        for (int q = 0; q < kRedParts; q++)
+#pragma unroll
+          for (int j = 0; j < kRedRows; j++) {
+            const bool on = q < np && row0 + j < rows;
+            const int64_t pr = on ? part[q] + j : 0;
+            v[j][q] = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
+          }
+      };
+      if constexpr (kWide) ask_partials();
       float lse[kRedRows][kRedParts], cs[kRedRows][kRedParts];
       const __bf16* cp[kRedRows][kRedParts];
 #pragma unroll
@@ -797,17 +827,13 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
           cp[j][q] = p.corr_row[pr];
           if (lse[j][q] == INFINITY || lse[j][q] == -INFINITY) cs[j][q] = 0.f;
         }
-      h8 v[kRedRows][kRedParts];
+      if constexpr (!kWide) ask_partials();
       bf16x8 kv[kRedRows][kRedParts];
 #pragma unroll
       for (int q = 0; q < kRedParts; q++)
 #pragma unroll
-        for (int j = 0; j < kRedRows; j++) {
-          const bool on = q < np && row0 + j < rows;
-          const int64_t pr = on ? part[q] + j : 0;
-          v[j][q] = *(const h8*)(p.o_part + pr * kDNope + lane * 8);
+        for (int j = 0; j < kRedRows; j++)
           if (cs[j][q] != 0.f) kv[j][q] = *(const bf16x8*)(cp[j][q] + lane * 8);
-        }
 #pragma unroll
       for (int q = 0; q < kRedParts; q++)
 #pragma unroll
@@ -827,6 +853,33 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
           }
         }
     }
+  }
+  if constexpr (kWide) {
+    static_assert(!kWide || kRedRows == 1, "the exchange below holds one row per wavefront");
+    if (lane == 0) { comb_ml[wave * 2] = m[0]; comb_ml[wave * 2 + 1] = tot[0]; }
+#pragma unroll
+    for (int e = 0; e < 8; e++) comb_a[(wave * 8 + e) * 64 + lane] = a[0][e];
+    __syncthreads();
+    if (wave == 0) {
+      float mm = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < 4; w++) mm = fmaxf(mm, comb_ml[w * 2]);
+      float tt = 0.f, aa[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        const float mw = comb_ml[w * 2];
+        const float f = mw == -INFINITY ? 0.f : __expf(mw - mm);          // a wavefront without partials weighs nothing
+        tt += comb_ml[w * 2 + 1] * f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) aa[e] += comb_a[(w * 8 + e) * 64 + lane] * f;
+      }
+      m[0] = mm;
+      tot[0] = tt;
+#pragma unroll
+      for (int e = 0; e < 8; e++) a[0][e] = aa[e];
+    }
+    __syncthreads();                                          // the exchange area is reused by the next row
+    if (wave != 0) continue;
   }
 #pragma unroll
   for (int j = 0; j < kRedRows; j++) {
@@ -848,11 +901,17 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
 
 int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
-  const int64_t waves = (int64_t)p.batch * ((r_max + kRedRows - 1) / kRedRows);
-  int64_t wgs = (waves + 3) / 4;
-  static const int64_t cap = getenv("MLA_REDUCE_WGS") ? atoll(getenv("MLA_REDUCE_WGS")) : (1ll << 30);
-  if (wgs > cap) wgs = cap;
-  hipLaunchKernelGGL(mla_chunk_reduce_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  const int64_t row_groups = (int64_t)p.batch * ((r_max + kRedRows - 1) / kRedRows);
+  // a sequence has about num_chunks / batch + 1 partials; past two passes of the one-wavefront form the wide form wins
+  // (as long as all rows' workgroups are resident at once: two per CU at its register use)
+  const bool wide = p.batch > 0 && p.num_chunks / p.batch + 1 > 2 * kRedPartsNarrow && row_groups <= 512;
+  if (wide) {
+    const int64_t wgs = row_groups < (1ll << 30) ? row_groups : (1ll << 30);
+    hipLaunchKernelGGL(mla_chunk_reduce_kernel<true>, dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  } else {
+    const int64_t wgs = (row_groups + 3) / 4;
+    hipLaunchKernelGGL(mla_chunk_reduce_kernel<false>, dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  }
   return check_launch("mla_chunk_reduce_kernel");
 }
 

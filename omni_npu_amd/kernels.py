@@ -259,9 +259,10 @@ def _workspace(dev: torch.device, nbytes: int, tag: str = "decode") -> torch.Ten
 def default_num_splits(batch: int, max_q_len: int, num_heads: int, max_seq_len: int, num_cus: int = 256) -> int:
     """Static split count (a function of shapes only, so a captured graph stays valid)."""
     groups = batch * math.ceil(max_q_len * num_heads / 128)
-    tiles = max(1, math.ceil(max_seq_len / 64))
+    # a chunk should hold at least eight 32-key blocks: that is what starting a segment costs
+    by_length = max(1, math.ceil(max_seq_len / 256))
     want = max(1, math.ceil(num_cus / max(groups, 1)))
-    return int(max(1, min(want, tiles, 64)))
+    return int(max(1, min(want, by_length, 256)))
 
 
 def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,

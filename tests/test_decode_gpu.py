@@ -111,6 +111,21 @@ def test_decode_ragged_edges(dev, lens):
     attn_close(got.transpose(0, 1), ref, MAX_ABS, MEAN_REL)
 
 
+@pytest.mark.parametrize("batch,heads,q_len,lo,hi,splits", [(1, 128, 1, 9000, 9000, 200), (2, 16, 2, 3000, 7000, 40),
+                                                            (1, 128, 1, 20000, 20000, None), (3, 128, 1, 50, 400, 24),
+                                                            (2, 128, 2, 1, 5000, 13)])
+def test_decode_many_partials_per_sequence(dev, batch, heads, q_len, lo, hi, splits):
+    """Few sequences and long contexts: dozens to hundreds of partials per row, merged by a workgroup per row (four
+    wavefronts, every fourth partial each); the fourth case has more chunks than work units, so some chunks are empty
+    and the partial list is found by testing chunk by chunk."""
+    case = O.make_decode_case(batch, heads, lo, hi, seed=21 + batch, q_len=q_len)
+    ref, ref_lse = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                                     case["seq_lens"], case["scale"], return_lse=True)
+    got, lse = _run(case, dev, splits, with_lse=True)
+    attn_close(got, ref, MAX_ABS, MEAN_REL)
+    assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
+
+
 def test_decode_single_key_returns_the_row(dev):
     """L = 1: softmax over one key is 1, the output is that latent row exactly (in bf16)."""
     case = O.make_decode_case(3, 128, 1, 1, seed=5)
