@@ -273,3 +273,54 @@ def test_decode_headline_shape_properties(dev):
     c2["block_table"] = inv[case["block_table"].long()].to(torch.int32)
     got_perm, _ = _run(c2, dev, num_splits=8)
     assert torch.equal(got_perm, got8)
+
+
+def test_decode_step_with_many_partials_replayed_from_a_hip_graph(dev):
+    """Cache write + decode of two long sequences (dozens of chunks each, merged by a workgroup per row) captured once and
+    replayed with new lengths, slots, queries and rows written into the same device buffers; eager work runs between the
+    replays, every replay must equal the eager step bit for bit, and the eager step must match the oracle."""
+    from omni_npu_amd import kernels as K
+    batch, heads = 2, 128
+    c = O.make_decode_case(batch, heads, 5000, 9000, seed=77)
+    qn, qr = c["q_nope"].to(dev), c["q_rope"].to(dev)
+    nope, rope = c["nope"].to(dev), c["rope"].to(dev)
+    new_c, new_r = c["new_c"].to(dev), c["new_r"].to(dev)
+    lens, slots, bt = c["seq_lens"].to(dev), c["slot_mapping"].to(dev), c["block_table"].to(dev)
+    out = torch.empty(batch, heads, 512, dtype=torch.bfloat16, device=dev)
+    max_len = bt.shape[1] * 128
+    splits = K.default_num_splits(batch, 1, heads, max_len)
+    assert splits + 1 > 12                                    # enough partials per row for the workgroup-per-row merge
+    ws = torch.empty(K._lib.load().mla_decode_workspace_bytes(batch, 1, heads, splits), dtype=torch.uint8, device=dev)
+
+    def step():
+        K.cache_write(new_c, new_r, slots, nope, rope)
+        K.decode(qn, qr, nope, rope, bt, lens, c["scale"], out, num_splits=splits, workspace=ws, max_seq_len=max_len)
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    ref_nope, ref_rope = c["nope"].clone(), c["rope"].clone()
+    O.cache_write(ref_nope, c["slot_mapping"], c["new_c"])   # the warm-up step wrote the case's own new rows
+    O.cache_write(ref_rope, c["slot_mapping"], c["new_r"])
+    for trial in range(3):
+        g = torch.Generator().manual_seed(200 + trial)
+        new_lens = (c["seq_lens"] - torch.randint(0, 3000, (batch,), generator=g).to(torch.int32)).clamp_min(1)
+        sl = torch.cat([O.slots_for(c["block_table"], b, int(new_lens[b]) - 1, int(new_lens[b])) for b in range(batch)])
+        q1 = torch.randn(batch, heads, 512, generator=g).bfloat16()
+        r1 = torch.randn(batch, 512, generator=g).bfloat16()
+        lens.copy_(new_lens.to(dev)); slots.copy_(sl.to(dev)); qn.copy_(q1.to(dev)); new_c.copy_(r1.to(dev))
+        before_n, before_r = nope.clone(), rope.clone()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        nope.copy_(before_n); rope.copy_(before_r)
+        out.zero_()
+        step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, out), f"replay {trial} differs from the eager step"
+        O.cache_write(ref_nope, sl, r1)
+        O.cache_write(ref_rope, sl, c["new_r"])
+        ref = O.absorbed_decode(q1, c["q_rope"], ref_nope, ref_rope, c["block_table"], new_lens, c["scale"])
+        attn_close(got, ref, MAX_ABS, MEAN_REL)
