@@ -107,15 +107,17 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int h32 = lane & 31;
   const int half = lane >> 5;
-  // The row groups of one chunk (more than 128 query rows: several tokens per sequence) stream the same cache rows.
-  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has its own L2, so they are renumbered to
-  // sit on one XCD, next to each other in its queue: they run at the same time and share the rows in that L2.
+  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has its own L2.  Two families of workgroups
+  // read the same bytes and are renumbered to sit on one XCD: the row groups of one chunk (more than 128 query rows:
+  // several tokens per sequence) stream the same cache rows, next to each other in the XCD's queue so that they run at
+  // the same time; and consecutive chunks belong to the same sequence and load the same queries, so every XCD takes a
+  // contiguous eighth of the chunks (the query rows then come from memory once per sequence, not once per chunk).
   int chunk = blockIdx.x, grp = blockIdx.z;
-  if (gridDim.z > 1 && (gridDim.x & 7) == 0) {
-    const int lin = blockIdx.x + gridDim.x * blockIdx.z;
-    const int j = lin >> 3;
+  if ((gridDim.x & 7) == 0) {
+    const int lin = blockIdx.x + gridDim.x * blockIdx.z;    // launch order
+    const int j = lin >> 3;                                  // j-th workgroup of XCD lin & 7
     grp = j % gridDim.z;
-    chunk = (j / gridDim.z) * 8 + (lin & 7);
+    chunk = (lin & 7) * (gridDim.x >> 3) + j / gridDim.z;
   }
   const int r_max = p.max_q_len * p.num_heads;
   if (grp * 128 >= r_max) return;
