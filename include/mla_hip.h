@@ -130,9 +130,23 @@ int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int3
                        int32_t num_splits, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
                        mlahip_stream_t stream);
 
+/* mla_splitkv_reduce with the value up-projection of attention/backends/mla.py:309-315 (_v_up_proj; DSA:
+ * dsa.py:233-240) fused in: out[t, n, v] = sum_c o[t, n, c] * w_uv[n, c, v] for the num_tokens query tokens, o being
+ * the merged (bf16-rounded) attention result that mla_splitkv_reduce would have written.  w_uv is the reference's
+ * W_UV, bf16 [N, 512, 128] through (w_stride_n, w_stride_k) in elements, last dim contiguous; `out` is addressed as
+ * [T, N, 128] through its strides (the reference's [T, N*128] output is out_stride_t = N*128, out_stride_h = 128).
+ * Replaces four launches of the reference's sequence (merge, batched GEMM, transpose, copy into the output). */
+int mla_splitkv_reduce_vup(const void* workspace, size_t workspace_bytes, const int32_t* seq_lens,
+                           const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                           int32_t num_splits, int32_t num_tokens, const void* w_uv, int64_t w_stride_n,
+                           int64_t w_stride_k, void* out, int64_t out_stride_t, int64_t out_stride_h,
+                           mlahip_stream_t stream);
+
 /* Same decode over the fp8-e4m3 block-scaled cache written by mla_cache_write_fp8 (row stride exactly 656 bytes,
  * page size 128).  Tiles are dequantised to bf16 on chip and take the bf16 MFMA path ("dequantise, then attend").
- * No reference counterpart: attention/backends/mla.py:791-792 passes antiquant_mode=0, antiquant_scale=None. */
+ * No reference counterpart: attention/backends/mla.py:791-792 passes antiquant_mode=0, antiquant_scale=None.
+ * out == NULL runs the split phase only: the partials stay in the workspace for mla_splitkv_reduce or
+ * mla_splitkv_reduce_vup (same seq_lens / query_start_loc / batch / max_q_len / num_heads / num_splits). */
 int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope, int64_t qr_stride_t,
                    int64_t qr_stride_h, const void* cache, int64_t page_stride_bytes, int64_t row_stride_bytes,
                    int64_t num_pages, const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
@@ -213,7 +227,9 @@ int dsa_topk_rows(const float* logits, int64_t logits_stride, const int32_t* seq
  * Replaces torch.ops.custom.npu_sparse_flash_attention, attention/backends/dsa.py:259-291 (sparse_block_size 1,
  * layout_kv "PA_BSND"): dsa_build_rows maps the [T,k] logical positions (-1 = unused,
  * v1/layers/attention/npu_dsa.py:553-555) through the block table to flat cache rows, compacted, with a count per
- * token; dsa_sparse_decode_bf16 runs the absorbed-MLA kernel over those rows (cache pages must be contiguous). */
+ * token; dsa_sparse_decode_bf16 runs the absorbed-MLA kernel over those rows (cache pages must be contiguous).
+ * out == NULL runs its split phase only; the merge is then mla_splitkv_reduce or mla_splitkv_reduce_vup with
+ * seq_lens = counts, query_start_loc = NULL, batch = num_tokens, max_q_len = 1. */
 int dsa_build_rows(const int32_t* indices, int64_t indices_stride, const int32_t* block_table, int64_t bt_stride,
                    int32_t max_blocks, const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
                    int32_t max_q_len, int32_t k, int32_t page_size, int64_t num_pages, int32_t* rows,

@@ -35,6 +35,7 @@ SIGNATURES = {
     "mla_decode_bf16_split": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                         I32, I32, F32, P, SZ, I32, P]),
     "mla_splitkv_reduce": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, P, I64, I64, P, P]),
+    "mla_splitkv_reduce_vup": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, I32, P, I64, I64, P, I64, I64, P]),
     "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                   I32, I32, F32, P, I64, I64, P, P, SZ, I32, P]),
     "mla_prefill_varlen": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, P, I64, I64, P, P, I32, I32, I32, I32,

@@ -219,8 +219,18 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         ql_nope = torch.bmm(q_nope.transpose(0, 1), self.W_UK_T).transpose(0, 1)
         return ql_nope, q_pe
 
-    def _apply_sparse_attention(self, q_nope, q_pe, kv_cache, meta, lens, q_len, qsl, topk_indices) -> torch.Tensor:
-        """Absorbed MLA over the indexer's positions (reference dsa.py:259-291); token-major [T,N,512]."""
+    def _fusable_w_uv(self, out: torch.Tensor) -> bool:
+        """The fused merge + up-projection kernel takes bf16 W_UV [N,512,128] with contiguous rows and writes rows of 128."""
+        w = self.W_UV
+        return (w.dtype == torch.bfloat16 and w.dim() == 3 and w.shape[1:] == (512, 128) and w.stride(2) == 1
+                and w.stride(0) % 8 == 0 and w.stride(1) % 8 == 0 and w.data_ptr() % 16 == 0
+                and out.dtype == torch.bfloat16 and out.stride(-1) == 1 and out.stride(0) % 4 == 0 and out.data_ptr() % 8 == 0)
+
+    def _apply_sparse_attention(self, q_nope, q_pe, kv_cache, meta, lens, q_len, qsl, topk_indices,
+                                proj_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """Absorbed MLA over the indexer's positions (reference dsa.py:259-291); token-major [T,N,512].  With
+        ``proj_out`` ([T, N*V]) the value up-projection (dsa.py:233-240) is fused into the merge of the partials and
+        nothing is returned."""
         bs = q_nope.shape[0]
         k = topk_indices.shape[-1]
         nope, rope = kv_cache[0], kv_cache[1]
@@ -228,6 +238,9 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         counts = torch.empty(bs, dtype=torch.int32, device=q_nope.device)
         K.build_sparse_rows(topk_indices.reshape(bs, k), meta.block_table, lens, nope.shape[1], nope.shape[0], rows, counts,
                             q_len=q_len, query_start_loc=qsl)
+        if proj_out is not None:
+            K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, proj_out, w_uv=self.W_UV)
+            return None
         out = torch.empty(bs, self.num_heads, self.kv_lora_rank, dtype=q_nope.dtype, device=q_nope.device)
         K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, out)
         return out
@@ -266,15 +279,19 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
             p = attn_metadata.prefill
             assert p is not None
             q_nope, q_pe = self._absorb_prolog(q[ndt:])
+            fused = output[ndt:] if self._fusable_w_uv(output[ndt:]) else None
             attn_out = self._apply_sparse_attention(q_nope, q_pe, kv_cache, p, p.kv_lens, p.max_query_len,
                                                     p.query_start_loc.to(torch.int32).contiguous(),
-                                                    topk[ndt:num_actual_toks])
-            self._v_up_proj(attn_out, out=output[ndt:])
+                                                    topk[ndt:num_actual_toks], proj_out=fused)
+            if fused is None:
+                self._v_up_proj(attn_out, out=output[ndt:])
         if has_decode:
             d = attn_metadata.decode
             assert d is not None
             q_nope, q_pe = self._absorb_prolog(q[:ndt])
+            fused = output[:ndt] if self._fusable_w_uv(output[:ndt]) else None
             attn_out = self._apply_sparse_attention(q_nope, q_pe, kv_cache, d, d.seq_lens, d.q_len, d.query_start_loc,
-                                                    topk[:ndt])
-            self._v_up_proj(attn_out, out=output[:ndt])
+                                                    topk[:ndt], proj_out=fused)
+            if fused is None:
+                self._v_up_proj(attn_out, out=output[:ndt])
         return output_padded

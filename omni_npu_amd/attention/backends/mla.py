@@ -241,13 +241,31 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         return output.to(torch.bfloat16).flatten(start_dim=-2)
 
     # ---- decode ----
-    def _forward_decode(self, decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer=None) -> torch.Tensor:
-        """Absorbed paged decode; returns the head-major [N, T, 512] tensor of the reference (mla.py:781-804)."""
+    def _fusable_w_uv(self, out: torch.Tensor) -> bool:
+        """The fused merge + up-projection kernel takes bf16 W_UV [N,512,128] with contiguous rows and writes rows of 128."""
+        w = self.W_UV
+        return (w.dtype == torch.bfloat16 and w.dim() == 3 and w.shape[1:] == (512, 128) and w.stride(2) == 1
+                and w.stride(0) % 8 == 0 and w.stride(1) % 8 == 0 and w.data_ptr() % 16 == 0
+                and out.dtype == torch.bfloat16 and out.stride(-1) == 1 and out.stride(0) % 4 == 0 and out.data_ptr() % 8 == 0)
+
+    def _forward_decode(self, decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer=None,
+                        proj_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """Absorbed paged decode; returns the head-major [N, T, 512] tensor of the reference (mla.py:781-804).  With
+        ``proj_out`` ([T, N*V]) the value up-projection (mla.py:309-315) is fused into the merge of the split-KV
+        partials: the result goes straight into ``proj_out`` and nothing is returned."""
         d = attn_metadata.decode
         assert d is not None
         t = decode_ql_nope.shape[0]
-        o = torch.empty(self.num_heads, t, self.kv_lora_rank, dtype=decode_ql_nope.dtype, device=decode_ql_nope.device)
         kw = dict(q_len=d.q_len, query_start_loc=d.query_start_loc, max_seq_len=d.block_table.shape[1] * K.PAGE)
+        if proj_out is not None:
+            if self.fp8_cache:
+                K.decode_fp8(decode_ql_nope, decode_q_pe, kv_cache[0], d.block_table, d.seq_lens, self.scale, proj_out,
+                             w_uv=self.W_UV, **kw)
+            else:
+                K.decode(decode_ql_nope, decode_q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens, self.scale,
+                         proj_out, w_uv=self.W_UV, **kw)
+            return None
+        o = torch.empty(self.num_heads, t, self.kv_lora_rank, dtype=decode_ql_nope.dtype, device=decode_ql_nope.device)
         if self.fp8_cache:
             K.decode_fp8(decode_ql_nope, decode_q_pe, kv_cache[0], d.block_table, d.seq_lens, self.scale,
                          o.transpose(0, 1), **kw)
@@ -305,7 +323,11 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             decode_q_nope, decode_q_pe = decode_q.split([self.qk_nope_head_dim, self.qk_rope_head_dim], dim=-1)
             # (B, N, P) -> (N, B, P) x (N, P, L) -> (N, B, L) -> (B, N, L) view
             decode_ql_nope = torch.bmm(decode_q_nope.transpose(0, 1), self.W_UK_T).transpose(0, 1)
-            attn_out = self._forward_decode(decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer)
-            out_proj = self._v_up_proj(attn_out)
-            output[:out_proj.shape[0]].copy_(out_proj)
+            ndt = decode_ql_nope.shape[0]
+            if self._fusable_w_uv(output[:ndt]):
+                self._forward_decode(decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer, proj_out=output[:ndt])
+            else:
+                attn_out = self._forward_decode(decode_ql_nope, decode_q_pe, kv_cache, attn_metadata, layer)
+                out_proj = self._v_up_proj(attn_out)
+                output[:out_proj.shape[0]].copy_(out_proj)
         return output_padded

@@ -161,7 +161,7 @@ extern "C" int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, i
                                       const int32_t* counts, int32_t num_tokens, int32_t num_heads, float scale, void* out,
                                       int64_t out_stride_t, int64_t out_stride_h, float* lse_out, void* workspace,
                                       size_t workspace_bytes, int32_t num_splits, hipStream_t stream) {
-  MLA_REQUIRE(sparse_rows && counts && out, MLA_ERR_NULL, "dsa_sparse_decode_bf16: null pointer argument");
+  MLA_REQUIRE(sparse_rows && counts, MLA_ERR_NULL, "dsa_sparse_decode_bf16: null pointer argument");
   MLA_REQUIRE(sparse_stride >= 1 && page_size >= 1, MLA_ERR_SHAPE, "dsa_sparse_decode_bf16: sparse_stride=%lld page_size=%d",
               (long long)sparse_stride, page_size);
   MLA_REQUIRE(nope_page_stride == (int64_t)page_size * nope_row_stride && rope_page_stride == (int64_t)page_size * rope_row_stride,
@@ -170,7 +170,7 @@ extern "C" int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, i
                              nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
                              nullptr, 0, 0, counts, nullptr, num_tokens, 1, num_heads, scale, workspace, workspace_bytes,
                              num_splits, sparse_rows, sparse_stride, page_size, false, stream);
-  if (rc != MLA_OK) return rc;
+  if (rc != MLA_OK || !out) return rc;                      // out == NULL: split phase only, the partials stay in the workspace
   return mla_splitkv_reduce(workspace, workspace_bytes, counts, nullptr, num_tokens, 1, num_heads, num_splits, out,
                             out_stride_t, out_stride_h, lse_out, stream);
 }
@@ -186,7 +186,7 @@ extern "C" int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t q
                               int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
                               int64_t out_stride_h, float* lse_out, void* workspace, size_t workspace_bytes,
                               int32_t num_splits, hipStream_t stream) {
-  MLA_REQUIRE(cache && out && block_table, MLA_ERR_NULL, "mla_decode_fp8: null pointer argument");
+  MLA_REQUIRE(cache && block_table, MLA_ERR_NULL, "mla_decode_fp8: null pointer argument");
   MLA_REQUIRE(row_stride_bytes == kFp8RowB && page_stride_bytes >= (int64_t)kPage * kFp8RowB && page_stride_bytes % 16 == 0,
               MLA_ERR_UNSUPPORTED, "mla_decode_fp8: rows must be exactly 656 bytes apart, pages 128 rows (got %lld / %lld)",
               (long long)row_stride_bytes, (long long)page_stride_bytes);
@@ -195,7 +195,7 @@ extern "C" int mla_decode_fp8(const void* q_nope, int64_t qn_stride_t, int64_t q
                              kFp8RowB + 8 /* unused in fp8 mode */, cache, page_stride_bytes, kFp8RowB + 8, num_pages,
                              block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
                              scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, true, stream);
-  if (rc != MLA_OK) return rc;
+  if (rc != MLA_OK || !out) return rc;                      // out == NULL: split phase only, the partials stay in the workspace
   // partials come in the balanced chunk order of the bf16 path: the same merge
   return mla_splitkv_reduce(workspace, workspace_bytes, seq_lens, query_start_loc, batch,
                             max_q_len, num_heads, num_splits, out, out_stride_t, out_stride_h, lse_out, stream);

@@ -74,6 +74,7 @@ __device__ __forceinline__ float half_sum(float v) {
 __device__ __forceinline__ int v2_num_blocks(int len) { return len > 0 ? (len + kBlk - 1) / kBlk : 0; }
 constexpr int kSegCost = 8;                                // start-up cost of a segment, in blocks (about 19 us / 2.3 us)
 __device__ __forceinline__ int v2_work_units(int len) { return len > 0 ? (len + kBlk - 1) / kBlk + kSegCost : 0; }
+static_assert(kBlk == kPlanBlk && kSegCost == kPlanSegCost, "the merge kernels recompute the chunk plan with these constants");
 __device__ __forceinline__ int wave_sum_i32(int v) {
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);

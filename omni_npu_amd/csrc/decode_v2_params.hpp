@@ -34,6 +34,16 @@ struct ChunkReduceParams {
 };
 int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream);
 
+// The chunk plan of the split kernels, as the merge kernels recompute it: work is counted in blocks of kPlanBlk keys,
+// and every non-empty sequence costs kPlanSegCost more units of start-up.
+constexpr int kPlanBlk = 32;
+constexpr int kPlanSegCost = 8;
+__device__ __forceinline__ int plan_work_units(int len) { return len > 0 ? (len + kPlanBlk - 1) / kPlanBlk + kPlanSegCost : 0; }
+
+// Merge of the partials fused with the value up-projection (reduce_vup.hip): out[t, n*128 + v] = merged o[t,n,:] . W_UV[n,:,v]
+int launch_reduce_vup(const ChunkReduceParams& r, const void* w_uv, int64_t w_stride_n, int64_t w_stride_k,
+                      int32_t num_tokens, hipStream_t stream);
+
 // Launches mla_decode_v2_kernel<sparse> on `stream`; returns 0 or a negative error code.
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
 // Launches mla_decode_v2_fp8_kernel (decode_v2_fp8.hip) over p.cache8.

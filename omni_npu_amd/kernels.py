@@ -265,27 +265,33 @@ def default_num_splits(batch: int, max_q_len: int, num_heads: int, max_seq_len: 
     return int(max(1, min(want, by_length, 256)))
 
 
-def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
-           block_table: torch.Tensor, seq_lens: torch.Tensor, scale: float, out: torch.Tensor,
-           q_len: int = 1, query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
-           num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
-           workspace: Optional[torch.Tensor] = None, phase: str = "both") -> torch.Tensor:
-    """Absorbed-MLA paged decode (reference: FIA decode call, src/omni_npu/attention/backends/mla.py:781-804).
+def _vup_out(out: torch.Tensor, w_uv: torch.Tensor, t: int, n: int) -> torch.Tensor:
+    """The [T,N,128] view of the output of a decode with the value up-projection fused in, after checking w_uv."""
+    _need_cuda(w_uv)
+    if w_uv.dtype != torch.bfloat16 or w_uv.shape != (n, D_NOPE, 128) or w_uv.stride(2) != 1:
+        raise TypeError(f"w_uv must be bf16 [{n},512,128] with contiguous rows, got {tuple(w_uv.shape)}")
+    o3 = out.view(t, n, 128) if out.dim() == 2 else out
+    if o3.shape != (t, n, 128) or o3.dtype != torch.bfloat16 or o3.stride(-1) != 1:
+        raise ValueError(f"with w_uv the output must be bf16 [T, N*128] or [T,N,128], got {tuple(out.shape)}")
+    return o3
 
-    q_nope [T,N,512], q_rope [T,N,64] (any token/head strides), caches [nblk,128,512] / [nblk,128,64],
-    block_table int32 [B,maxblk], seq_lens int32 [B] on the device, ``out`` a bf16 tensor viewed as
-    [T,N,512] through its strides: pass ``o.transpose(0,1)`` of an [N,T,512] buffer for the reference's
-    head-major result.  Sequence b owns query tokens [b*q_len, (b+1)*q_len) unless query_start_loc
-    (int32 [B+1], device) says otherwise; token i of a request sees keys [0, L - s + i].
-    ``phase`` = "both" | "split" | "reduce" runs the split-KV kernel, the reduction, or both (one C call).
-    """
+
+def _reduce_vup(lib, ws_args, seq_lens, qsl, b, q_len, n, num_splits, t, w_uv, o3, st) -> None:
+    rc = lib.mla_splitkv_reduce_vup(*ws_args, seq_lens.data_ptr(), qsl, b, q_len, n, num_splits, t, w_uv.data_ptr(),
+                                    w_uv.stride(0), w_uv.stride(1), o3.data_ptr(), o3.stride(0), o3.stride(1), st)
+    _lib.check(rc, "mla_splitkv_reduce_vup")
+
+
+def _decode_args(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out, out_width, q_len,
+                 query_start_loc, lse_out, num_splits, max_seq_len, workspace):
+    """Checks shared by decode() and decode_vup(); returns what the C calls need."""
     _need_cuda(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, out)
     lib = _lib.load()
     nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
     t, n, _ = q_nope.shape
     b = seq_lens.numel()
-    if q_nope.shape != (t, n, D_NOPE) or q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, D_NOPE):
-        raise ValueError(f"decode: q_nope {tuple(q_nope.shape)} q_rope {tuple(q_rope.shape)} out {tuple(out.shape)}")
+    if q_nope.shape != (t, n, D_NOPE) or q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, out_width):
+        raise ValueError(f"decode: q_nope {tuple(q_nope.shape)} q_rope {tuple(q_rope.shape)} out {tuple(out.shape)} (want [T,N,{out_width}])")
     for x in (q_nope, q_rope, out, nope, rope):
         if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
             raise TypeError("decode: bf16 tensors with a contiguous last dim only")
@@ -317,6 +323,43 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
     ws_args = (ws.data_ptr(), ws.numel() * ws.element_size())
     lse_p = lse_out.data_ptr() if lse_out is not None else None
     st = _stream(q_nope)
+    return lib, front, ws_args, lse_p, st, qsl, seq_lens, b, n, num_splits
+
+
+def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
+           block_table: torch.Tensor, seq_lens: torch.Tensor, scale: float, out: torch.Tensor,
+           q_len: int = 1, query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
+           num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
+           workspace: Optional[torch.Tensor] = None, phase: str = "both",
+           w_uv: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Absorbed-MLA paged decode (reference: FIA decode call, src/omni_npu/attention/backends/mla.py:781-804).
+
+    q_nope [T,N,512], q_rope [T,N,64] (any token/head strides), caches [nblk,128,512] / [nblk,128,64],
+    block_table int32 [B,maxblk], seq_lens int32 [B] on the device, ``out`` a bf16 tensor viewed as
+    [T,N,512] through its strides: pass ``o.transpose(0,1)`` of an [N,T,512] buffer for the reference's
+    head-major result.  Sequence b owns query tokens [b*q_len, (b+1)*q_len) unless query_start_loc
+    (int32 [B+1], device) says otherwise; token i of a request sees keys [0, L - s + i].
+    ``phase`` = "both" | "split" | "reduce" runs the split-KV kernel, the reduction, or both (one C call).
+    With ``w_uv`` (bf16 [N,512,128], the reference's W_UV) the value up-projection of mla.py:309-315 is fused into the
+    reduction: ``out`` is then [T, N*128] (or a [T,N,128] view) and holds o[t,n,:] @ w_uv[n]; no lse_out.
+    """
+    if w_uv is not None:
+        if lse_out is not None or phase == "split":
+            raise ValueError("decode: w_uv goes with the reduction and without lse_out")
+        t, n, _ = q_nope.shape
+        o3 = _vup_out(out, w_uv, t, n)
+        lib, front, ws_args, _, st, qsl, seq_lens, b, n, num_splits = _decode_args(
+            q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, o3, 128, q_len, query_start_loc, None,
+            num_splits, max_seq_len, workspace)
+        if phase == "both":
+            _lib.check(lib.mla_decode_bf16_split(*front, *ws_args, num_splits, st), "mla_decode_bf16_split")
+        elif phase != "reduce":
+            raise ValueError(f"decode: unknown phase {phase!r}")
+        _reduce_vup(lib, ws_args, seq_lens, qsl, b, q_len, n, num_splits, t, w_uv, o3, st)
+        return out
+    lib, front, ws_args, lse_p, st, qsl, seq_lens, b, n, num_splits = _decode_args(
+        q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out, D_NOPE, q_len, query_start_loc, lse_out,
+        num_splits, max_seq_len, workspace)
     if phase == "both":
         rc = lib.mla_decode_bf16(*front, out.data_ptr(), out.stride(0), out.stride(1), lse_p, *ws_args, num_splits, st)
         _lib.check(rc, "mla_decode_bf16")
@@ -445,14 +488,20 @@ def build_sparse_rows(indices: torch.Tensor, block_table: torch.Tensor, seq_lens
 def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
                   rows: torch.Tensor, counts: torch.Tensor, scale: float, out: torch.Tensor,
                   lse_out: Optional[torch.Tensor] = None, num_splits: Optional[int] = None,
-                  workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Absorbed MLA of token t over cache rows rows[t, :counts[t]] (reference: npu_sparse_flash_attention call,
-    src/omni_npu/attention/backends/dsa.py:259-291).  out bf16 viewed as [T,N,512]."""
+    src/omni_npu/attention/backends/dsa.py:259-291).  out bf16 viewed as [T,N,512]; with ``w_uv`` (bf16 [N,512,128])
+    the value up-projection of dsa.py:233-240 is fused into the merge and out is [T, N*128] / [T,N,128]."""
     _need_cuda(q_nope, q_rope, nope_cache, rope_cache, rows, counts, out)
     lib = _lib.load()
     nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
     t, n, _ = q_nope.shape
-    if q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, D_NOPE) or rows.shape[0] < t or counts.numel() < t:
+    o3 = None
+    if w_uv is not None:
+        if lse_out is not None:
+            raise ValueError("sparse_decode: w_uv goes without lse_out")
+        o3 = _vup_out(out, w_uv, t, n)
+    if q_rope.shape != (t, n, D_ROPE) or (o3 is None and out.shape != (t, n, D_NOPE)) or rows.shape[0] < t or counts.numel() < t:
         raise ValueError("sparse_decode: shape mismatch")
     for x in (q_nope, q_rope, out, nope, rope):
         if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
@@ -466,10 +515,14 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
     rc = lib.dsa_sparse_decode_bf16(
         q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
         nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[0],
-        nope.shape[1], rows.data_ptr(), rows.stride(0), counts.data_ptr(), t, n, float(scale), out.data_ptr(),
-        out.stride(0), out.stride(1), lse_out.data_ptr() if lse_out is not None else None, ws.data_ptr(),
+        nope.shape[1], rows.data_ptr(), rows.stride(0), counts.data_ptr(), t, n, float(scale),
+        out.data_ptr() if o3 is None else None, out.stride(0) if o3 is None else 0, out.stride(1) if o3 is None else 0,
+        lse_out.data_ptr() if lse_out is not None else None, ws.data_ptr(),
         ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
     _lib.check(rc, "dsa_sparse_decode_bf16")
+    if o3 is not None:
+        _reduce_vup(lib, (ws.data_ptr(), ws.numel() * ws.element_size()), counts, None, t, 1, n, num_splits, t, w_uv, o3,
+                    _stream(q_nope))
     return out
 
 
@@ -511,15 +564,21 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
                seq_lens: torch.Tensor, scale: float, out: torch.Tensor, q_len: int = 1,
                query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
                num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
-               workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Absorbed-MLA paged decode over the fp8 block-scaled cache (uint8 [num_blocks, 128, 656], see cache_write_fp8)."""
+               workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Absorbed-MLA paged decode over the fp8 block-scaled cache (uint8 [num_blocks, 128, 656], see cache_write_fp8).
+    With ``w_uv`` (bf16 [N,512,128]) the value up-projection is fused into the merge: out is [T, N*128] / [T,N,128]."""
     _need_cuda(q_nope, q_rope, cache, block_table, seq_lens, out)
     lib = _lib.load()
     t, n, _ = q_nope.shape
     b = seq_lens.numel()
+    o3 = None
+    if w_uv is not None:
+        if lse_out is not None:
+            raise ValueError("decode_fp8: w_uv goes without lse_out")
+        o3 = _vup_out(out, w_uv, t, n)
     if cache.dtype != torch.uint8 or cache.dim() != 3 or cache.shape[1:] != (PAGE, FP8_ROW_BYTES) or cache.stride(-1) != 1:
         raise ValueError(f"decode_fp8: cache must be uint8 [num_blocks, {PAGE}, {FP8_ROW_BYTES}]")
-    if q_nope.shape != (t, n, D_NOPE) or q_rope.shape != (t, n, D_ROPE) or out.shape != (t, n, D_NOPE):
+    if q_nope.shape != (t, n, D_NOPE) or q_rope.shape != (t, n, D_ROPE) or (o3 is None and out.shape != (t, n, D_NOPE)):
         raise ValueError("decode_fp8: q_nope [T,N,512], q_rope [T,N,64], out [T,N,512]")
     for x in (q_nope, q_rope, out):
         if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
@@ -538,10 +597,17 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
                             q_rope.stride(1), cache.data_ptr(), cache.stride(0), cache.stride(1), cache.shape[0],
                             block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
                             query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, n, float(scale),
-                            out.data_ptr(), out.stride(0), out.stride(1),
+                            out.data_ptr() if o3 is None else None, out.stride(0) if o3 is None else 0,
+                            out.stride(1) if o3 is None else 0,
                             lse_out.data_ptr() if lse_out is not None else None, ws.data_ptr(),
                             ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
     _lib.check(rc, "mla_decode_fp8")
+    if o3 is not None:
+        if not seq_lens.is_contiguous():
+            seq_lens = seq_lens.contiguous()
+        _reduce_vup(lib, (ws.data_ptr(), ws.numel() * ws.element_size()), seq_lens,
+                    query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, n, num_splits, t, w_uv, o3,
+                    _stream(q_nope))
     return out
 
 
