@@ -361,6 +361,85 @@ def bench_prologue(K, dev, args):
     }
 
 
+def bench_epilogue(K, dev, args):
+    """The step behind the split kernel: merge of the split-KV partials + value up-projection into the layer's [T, N*128]
+    output, on the headline shape (B=64, 128 heads, contexts 4k-8k, 4 chunks per sequence).  Fused (one launch) beside the
+    reference's sequence (merge, batched GEMM, transpose, copy), each timed as HIP-graph replays of the part after the
+    split kernel (the split kernel runs once, outside the timed region: its partials stay in the workspace)."""
+    import time
+    from oracle import mla_oracle as O
+    B, N = 64, 128
+    case = build_workload(args.seed, B, N, 4096, 8192, 1)
+    g = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in case.items()}
+    gen = torch.Generator().manual_seed(args.seed + 1)
+    w_cpu = (torch.randn(N, 512, 128, generator=gen) * 0.02).bfloat16()
+    w = w_cpu.to(dev)
+    splits = args.splits or K.default_num_splits(B, 1, N, int(case["seq_lens"].max()))
+    ws = torch.zeros(K._lib.load().mla_decode_workspace_bytes(B, 1, N, splits), dtype=torch.uint8, device=dev)
+    o = torch.empty(N, B, 512, dtype=torch.bfloat16, device=dev)
+    out_f = torch.empty(B, N * 128, dtype=torch.bfloat16, device=dev)
+    out_u = torch.empty_like(out_f)
+    dargs = (g["q_nope"], g["q_rope"], g["nope"], g["rope"], g["block_table"], g["seq_lens"], case["scale"])
+    K.decode(*dargs, o.transpose(0, 1), num_splits=splits, workspace=ws, phase="split")
+    torch.cuda.synchronize()
+
+    def fused():
+        K.decode(*dargs, out_f, num_splits=splits, workspace=ws, phase="reduce", w_uv=w)
+
+    def unfused():
+        K.decode(*dargs, o.transpose(0, 1), num_splits=splits, workspace=ws, phase="reduce")
+        out_u.copy_(torch.bmm(o, w).transpose(0, 1).contiguous().view(-1, N * 128))
+
+    def ev_time(fn, n, reps=10):
+        fn()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            fn()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(reps):
+                    fn()
+        torch.cuda.synchronize()
+        for _ in range(2):
+            graph.replay()
+        torch.cuda.synchronize()
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(e) * 1e3 / (n * reps)
+
+    t_f, t_u = ev_time(fused, args.steps), ev_time(unfused, args.steps)
+    segments = B * (splits + 1)                               # upper bound of the partials the merge reads
+    alg_bytes = segments * N * 1040 + N * 512 * 128 * 2 + B * N * 128 * 2
+    # oracle chain on the host: attention of a sample of sequences, then the up-projection of all
+    sample = 8
+    t0 = time.perf_counter()
+    ref_o = O.absorbed_decode(case["q_nope"][:sample], case["q_rope"][:sample], case["nope"], case["rope"],
+                              case["block_table"][:sample], case["seq_lens"][:sample], case["scale"])
+    ref = torch.bmm(ref_o.transpose(0, 1), w_cpu.float()).transpose(0, 1).reshape(sample, N * 128)
+    cpu_s = time.perf_counter() - t0
+    err = (out_f[:sample].float().cpu() - ref).abs().max().item()
+    same = (out_f.float() - out_u.float()).abs().max().item()
+    return {
+        "metric": "merge of the split-KV partials + value up-projection, us/layer (B=64, 128 heads, 4 chunks per sequence)",
+        "value": round(t_f, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "step behind the split kernel: merge + W_UV up-projection into [T, N*128]", "batch": B, "heads": N,
+                   "kv_splits": splits, "seed": args.seed},
+        "unfused_us": round(t_u, 2), "fused_vs_unfused_max_abs": same,
+        "roofline": {"kernel": "mla_reduce_vup_kernel", "bound": "hbm", "achieved": round(alg_bytes / t_f / 1e3, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_bytes / t_f / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": alg_bytes},
+        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", "cores": torch.get_num_threads(),
+                         "kind": "port", "sample": f"oracle attention (torch fp32) of {sample} of {B} sequences + up-projection, scaled by sequence count",
+                         "gpu_vs_oracle_max_abs": err},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -380,8 +459,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue"],
-                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -411,6 +490,9 @@ def main():
         return
     if args.workload == "prologue":
         print(json.dumps(bench_prologue(K, dev, args)))
+        return
+    if args.workload == "epilogue":
+        print(json.dumps(bench_epilogue(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len

@@ -25,6 +25,7 @@ constexpr int kVupOB = kVupTok * kDNope * 2;    // 16384: merged rows of one pas
 constexpr int kVupFlagOff = kVupWB + kVupOB;    // one int per token of the pass: its row is valid
 constexpr int kVupLdsB = kVupFlagOff + 64;
 constexpr int kVupParts = 6;                    // partials of a row asked for together
+constexpr int kVupAhead = 4;                    // GEMM steps whose operands are requested ahead (at most 4: the wait ladder)
 
 __device__ __forceinline__ int vup_wave_sum(int v) {
 #pragma unroll
@@ -208,13 +209,35 @@ __global__ __launch_bounds__(1024) void mla_reduce_vup_kernel(const ReduceVupPar
       f32x16 acc;
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[r] = 0.f;
-#pragma unroll 8
-      for (int kk = 0; kk < 32; kk++) {
-        const bf16x4 wl = lds_read_tr16(lds + kk * 4096 + a_off);
-        const bf16x4 wh = lds_read_tr16(lds + kk * 4096 + 2048 + a_off);
-        const bf16x8 wa = __builtin_shufflevector(wl, wh, 0, 1, 2, 3, 4, 5, 6, 7);
-        const bf16x8 ob = *(const bf16x8*)(lds + (b_off ^ (uint32_t)(kk << 5)));
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa, ob, acc, 0, 0, 0);
+      // Operands are read with hand-placed LDS instructions kVupAhead steps ahead of the MFMA that consumes them and
+      // explicit waits (three reads per step, returned in order): left to itself the compiler reads, waits and
+      // multiplies one step at a time and pays the LDS latency 32 times.
+      {
+        const uint32_t a_lo = lds0 + a_off, a_hi = a_lo + 16 * 4096;     // the offset field holds 16 steps of 4 KiB
+        const uint32_t b_ad = lds0 + b_off;
+        constexpr int D = kVupAhead;
+        bf16x4 wl[D], wh[D];
+        bf16x8 ob[D];
+#define VUP_READ(slot, kk)                                                                                             \
+        do {                                                                                                           \
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(wl[slot]) : "v"((kk) < 16 ? a_lo : a_hi), "i"(((kk) & 15) * 4096)); \
+          asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(wh[slot]) : "v"((kk) < 16 ? a_lo : a_hi), "i"(((kk) & 15) * 4096 + 2048)); \
+          asm volatile("ds_read_b128 %0, %1" : "=v"(ob[slot]) : "v"(b_ad ^ (uint32_t)((kk) << 5)));                      \
+        } while (0)
+#pragma unroll
+        for (int i = 0; i < D; i++) VUP_READ(i, i);
+#pragma unroll
+        for (int kk = 0; kk < 32; kk++) {
+          const int younger = (31 - kk) < (D - 1) ? (31 - kk) : (D - 1);      // steps asked for after step kk
+          if (younger >= 3) asm volatile("s_waitcnt lgkmcnt(9)" : "+v"(wl[kk % D]), "+v"(wh[kk % D]), "+v"(ob[kk % D]));
+          else if (younger == 2) asm volatile("s_waitcnt lgkmcnt(6)" : "+v"(wl[kk % D]), "+v"(wh[kk % D]), "+v"(ob[kk % D]));
+          else if (younger == 1) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(wl[kk % D]), "+v"(wh[kk % D]), "+v"(ob[kk % D]));
+          else asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(wl[kk % D]), "+v"(wh[kk % D]), "+v"(ob[kk % D]));
+          const bf16x8 wa = __builtin_shufflevector(wl[kk % D], wh[kk % D], 0, 1, 2, 3, 4, 5, 6, 7);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa, ob[kk % D], acc, 0, 0, 0);
+          if (kk + D < 32) VUP_READ(kk % D, kk + D);
+        }
+#undef VUP_READ
       }
       const int tt = (tb * pp.passes + pass) * kVupTok + tr;
       const bool ok = h32 < kVupTok && *(const int*)(lds + kVupFlagOff + tr * 4) != 0;

@@ -71,7 +71,10 @@ def test_fused_up_projection_strided_output_and_varlen_queries(dev):
     from omni_npu_amd import kernels as K
     batch, heads, q_len = 3, 128, 2
     c = O.make_decode_case(batch, heads, 100, 500, seed=9, q_len=q_len)
-    w = _w_uv(heads, seed=1)
+    # W_UV as the reference derives it: a transposed view [N, 512, 128] of a [512, N, 128] tensor (row stride N * 128)
+    g = torch.Generator().manual_seed(1)
+    w = (torch.randn(512, heads, 128, generator=g) * 0.02).bfloat16().to(dev).transpose(0, 1)
+    assert not w.is_contiguous()
     qsl = torch.tensor([0, 2, 3, 5], dtype=torch.int32)        # request 1 has one token only
     keep = torch.tensor([0, 1, 2, 4, 5])
     qn, qr = c["q_nope"][keep].contiguous(), c["q_rope"][keep].contiguous()
@@ -79,11 +82,11 @@ def test_fused_up_projection_strided_output_and_varlen_queries(dev):
     buf = torch.full((t + 3, heads * 128 + 64), 7.0, dtype=torch.bfloat16, device=dev)
     out = buf[:t, 64:]
     K.decode(qn.to(dev), qr.to(dev), c["nope"].to(dev), c["rope"].to(dev), c["block_table"].to(dev), c["seq_lens"].to(dev),
-             c["scale"], out.view(t, heads, 128), q_len=q_len, query_start_loc=qsl.to(dev), num_splits=2, w_uv=w.to(dev))
+             c["scale"], out.view(t, heads, 128), q_len=q_len, query_start_loc=qsl.to(dev), num_splits=2, w_uv=w)
     o = torch.empty(t, heads, 512, dtype=torch.bfloat16, device=dev)
     K.decode(qn.to(dev), qr.to(dev), c["nope"].to(dev), c["rope"].to(dev), c["block_table"].to(dev), c["seq_lens"].to(dev),
              c["scale"], o, q_len=q_len, query_start_loc=qsl.to(dev), num_splits=2)
-    unfused = torch.bmm(o.transpose(0, 1).float(), w.to(dev).float()).transpose(0, 1).reshape(t, heads * 128)
+    unfused = torch.bmm(o.transpose(0, 1).float(), w.float()).transpose(0, 1).reshape(t, heads * 128)
     torch.cuda.synchronize()
     assert (out.float() - unfused).abs().max().item() <= unfused.abs().max().item() * 2 ** -7
     assert (buf[t:] == 7.0).all() and (buf[:, :64] == 7.0).all()
