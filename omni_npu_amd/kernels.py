@@ -276,7 +276,20 @@ def _vup_out(out: torch.Tensor, w_uv: torch.Tensor, t: int, n: int) -> torch.Ten
     return o3
 
 
+# The fused merge + up-projection gives a row to ONE wavefront (six partials per round trip).  Past this many partials per
+# sequence (few sequences with long contexts) the separate merge, which puts a workgroup on every row, followed by the
+# library GEMM is faster.
+VUP_MAX_SPLITS = 11
+
+
 def _reduce_vup(lib, ws_args, seq_lens, qsl, b, q_len, n, num_splits, t, w_uv, o3, st) -> None:
+    if num_splits > VUP_MAX_SPLITS:
+        o = torch.empty(n, t, D_NOPE, dtype=torch.bfloat16, device=o3.device)
+        rc = lib.mla_splitkv_reduce(*ws_args, seq_lens.data_ptr(), qsl, b, q_len, n, num_splits, o.data_ptr(), o.stride(1),
+                                    o.stride(0), None, st)
+        _lib.check(rc, "mla_splitkv_reduce")
+        o3.copy_(torch.bmm(o, w_uv).transpose(0, 1))
+        return
     rc = lib.mla_splitkv_reduce_vup(*ws_args, seq_lens.data_ptr(), qsl, b, q_len, n, num_splits, t, w_uv.data_ptr(),
                                     w_uv.stride(0), w_uv.stride(1), o3.data_ptr(), o3.stride(0), o3.stride(1), st)
     _lib.check(rc, "mla_splitkv_reduce_vup")
