@@ -919,16 +919,9 @@ int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
 }
 
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)mla_decode_v2_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kV2LdsB);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void*)mla_decode_v2_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, kV2LdsB);
-    if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_decode_bf16: cannot reserve %d bytes of LDS: %s", kV2LdsB,
-                                     hipGetErrorString(e));
-    attr_set = true;
-  }
+  const int rc = sparse ? ensure_dynamic_lds((const void*)mla_decode_v2_kernel<true>, kV2LdsB, "dsa_sparse_decode_bf16")
+                        : ensure_dynamic_lds((const void*)mla_decode_v2_kernel<false>, kV2LdsB, "mla_decode_bf16");
+  if (rc != MLA_OK) return rc;
   if (sparse) hipLaunchKernelGGL(mla_decode_v2_kernel<true>, grid, dim3(256), kV2LdsB, stream, p);
   else hipLaunchKernelGGL(mla_decode_v2_kernel<false>, grid, dim3(256), kV2LdsB, stream, p);
   return check_launch("mla_decode_v2_kernel");

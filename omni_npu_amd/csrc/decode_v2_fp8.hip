@@ -624,14 +624,8 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV
 }  // namespace f8v2
 
 int launch_decode_v2_fp8(const DecodeV2Params& p, dim3 grid, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)f8v2::mla_decode_v2_fp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       f8v2::kV2LdsB);
-    if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_decode_fp8: cannot reserve %d bytes of LDS: %s", f8v2::kV2LdsB,
-                                     hipGetErrorString(e));
-    attr_set = true;
-  }
+  const int rc = ensure_dynamic_lds((const void*)f8v2::mla_decode_v2_fp8_kernel, f8v2::kV2LdsB, "mla_decode_fp8");
+  if (rc != MLA_OK) return rc;
   hipLaunchKernelGGL(f8v2::mla_decode_v2_fp8_kernel, grid, dim3(256), f8v2::kV2LdsB, stream, p);
   return check_launch("mla_decode_v2_fp8_kernel");
 }

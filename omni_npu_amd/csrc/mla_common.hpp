@@ -20,6 +20,8 @@ enum : int {
 };
 int fail(int code, const char* fmt, ...);
 int check_launch(const char* what);
+// raises the dynamic-LDS limit of `kernel` to `bytes` on the current device (once per kernel and device)
+int ensure_dynamic_lds(const void* kernel, int bytes, const char* what);
 
 #define MLA_REQUIRE(cond, code, ...)                 \
   do {                                               \

@@ -331,14 +331,8 @@ extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64
   p.scale_log2 = scale * kLog2e;
   p.out = out; p.o_st = out_stride_t; p.o_sh = out_stride_h; p.out_fp32 = out_dtype;
   p.lse = lse_out;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)mla_prefill_varlen_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       kPfLdsB);
-    if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_prefill_varlen: cannot reserve %d bytes of LDS: %s", kPfLdsB,
-                                     hipGetErrorString(e));
-    attr_set = true;
-  }
+  const int rc = ensure_dynamic_lds((const void*)mla_prefill_varlen_kernel, kPfLdsB, "mla_prefill_varlen");
+  if (rc != MLA_OK) return rc;
   dim3 grid((max_q_len + kPfRows - 1) / kPfRows, num_heads, batch);
   hipLaunchKernelGGL(mla_prefill_varlen_kernel, grid, dim3(256), kPfLdsB, stream, p);
   return check_launch("mla_prefill_varlen_kernel");

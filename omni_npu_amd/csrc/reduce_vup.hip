@@ -258,14 +258,8 @@ __global__ __launch_bounds__(1024) void mla_reduce_vup_kernel(const ReduceVupPar
 
 int launch_reduce_vup(const ChunkReduceParams& r, const void* w_uv, int64_t w_stride_n, int64_t w_stride_k,
                       int32_t num_tokens, hipStream_t stream) {
-  static bool attr_set = false;
-  if (!attr_set) {
-    const hipError_t e = hipFuncSetAttribute((const void*)mla_reduce_vup_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             kVupLdsB);
-    if (e != hipSuccess) return fail(MLA_ERR_LAUNCH, "mla_splitkv_reduce_vup: cannot reserve %d bytes of LDS: %s", kVupLdsB,
-                                     hipGetErrorString(e));
-    attr_set = true;
-  }
+  const int rc = ensure_dynamic_lds((const void*)mla_reduce_vup_kernel, kVupLdsB, "mla_splitkv_reduce_vup");
+  if (rc != MLA_OK) return rc;
   ReduceVupParams pp;
   pp.r = r;
   pp.w_uv = (const __bf16*)w_uv; pp.w_sn = w_stride_n; pp.w_sk = w_stride_k;
