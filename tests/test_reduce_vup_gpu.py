@@ -22,7 +22,7 @@ def _w_uv(n, seed):
 @pytest.mark.parametrize("batch,heads,q_len,lo,hi,splits", [(4, 16, 1, 128, 1024, 2), (64, 128, 1, 100, 700, 4),
                                                             (5, 128, 2, 1, 600, 3), (19, 40, 1, 50, 400, None),
                                                             (2, 128, 1, 3000, 6000, 11), (3, 128, 1, 50, 300, 9),
-                                                            (2, 128, 1, 3000, 6000, 40)])
+                                                            (2, 128, 1, 3000, 6000, 40), (150, 128, 2, 2, 200, 1)])
 def test_fused_merge_and_up_projection(dev, batch, heads, q_len, lo, hi, splits):
     """Up to 11 chunks per sequence the fused kernel runs (rows of 7..12 partials take two rounds; the case with more
     chunks than work units has empty chunks); the last case takes the route for many partials per row (separate merge
