@@ -267,3 +267,20 @@ def test_graph_wrapper_pass_through_and_pad_list():
     assert w2.extra == 7
     with pytest.raises(AttributeError):
         w2.missing
+
+
+def test_default_split_count_is_a_function_of_shapes_only():
+    """About one chunk per compute unit, never fewer than eight 32-key blocks per chunk, at most 256 chunks per sequence;
+    shapes of the benchmark configurations keep the counts they were measured with."""
+    from omni_npu_amd import kernels as K
+    assert K.default_num_splits(64, 1, 128, 8192) == 4            # headline: 256 chunks
+    assert K.default_num_splits(32, 1, 128, 2048) == 8            # sparse decode over top-2048
+    assert K.default_num_splits(256, 2, 128, 32768) == 1          # fp8 configuration: two row groups per sequence already
+    assert K.default_num_splits(1, 1, 128, 131072) == 256         # one long sequence fills the device
+    assert K.default_num_splits(1, 1, 128, 1000) == 4             # ... but a chunk keeps eight blocks
+    assert K.default_num_splits(1, 1, 16, 1) == 1
+    assert K.default_num_splits(4, 3, 128, 65536) == 22           # 4 x 3 row groups: ceil(256 / 12)
+    for b in (1, 3, 64, 1000):
+        for l in (1, 255, 256, 257, 10 ** 6):
+            s = K.default_num_splits(b, 1, 128, l)
+            assert 1 <= s <= 256 and (s == 1 or l / s >= 128)
