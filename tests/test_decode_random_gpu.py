@@ -1,0 +1,78 @@
+"""Seeded sweep over shapes of the paged decode: batch, heads (multiples of 8 up to 128), query tokens per request, ragged
+context lengths down to the number of query tokens, split counts from 1 to more chunks than there is work; bf16 cache,
+fp8 cache, row-list (sparse) form and the fused up-projection, each against the oracle at the tolerance of its own test
+file.  The cases are fixed by the seed, so a failure names its case."""
+import random
+
+import pytest
+import torch
+
+from oracle import mla_oracle as O
+from tests.conftest import attn_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _cases(n, seed):
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        q_len = rng.choice([1, 1, 1, 2, 2, 3, 4])
+        heads = rng.choice([8, 16, 40, 64, 128, 128])
+        batch = rng.randint(1, 9)
+        lo = rng.choice([q_len, q_len, 31, 32, 33, 127, 128, 129, 500])
+        hi = lo + rng.choice([0, 1, 40, 300, 1400])
+        splits = rng.choice([None, 1, 2, 3, 5, 13, 40])
+        out.append((i, batch, heads, q_len, lo, hi, splits))
+    return out
+
+
+@pytest.mark.parametrize("i,batch,heads,q_len,lo,hi,splits", _cases(64, seed=2024))
+def test_decode_random_shapes(dev, i, batch, heads, q_len, lo, hi, splits):
+    from omni_npu_amd import kernels as K
+    c = O.make_decode_case(batch, heads, lo, hi, seed=1000 + i, q_len=q_len)
+    t = batch * q_len
+    ref, ref_lse = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"],
+                                     c["scale"], return_lse=True)
+    args = [c[k].to(dev) for k in ("q_nope", "q_rope", "nope", "rope", "block_table", "seq_lens")]
+    out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty(t, heads, dtype=torch.float32, device=dev)
+    K.decode(*args, c["scale"], out, q_len=q_len, num_splits=splits, lse_out=lse)
+    attn_close(out, ref, 2e-2, 2e-3)
+    assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
+
+    if i % 2 == 0:                                            # the same case through the fused up-projection
+        g = torch.Generator().manual_seed(i)
+        w = (torch.randn(heads, 512, 128, generator=g) * 0.02).bfloat16()
+        out_v = torch.full((t, heads * 128), float("nan"), dtype=torch.bfloat16, device=dev)
+        K.decode(*args, c["scale"], out_v, q_len=q_len, num_splits=splits, w_uv=w.to(dev))
+        ref_v = torch.bmm(ref.transpose(0, 1), w.float()).transpose(0, 1).reshape(t, heads * 128)
+        attn_close(out_v, ref_v, 2e-2 * 0.45, 2e-3 * 1.5)
+
+    if i % 3 == 0:                                            # ... and over the fp8 cache
+        q8, sc = O.fp8_quant_block(c["nope"].float())
+        deq = O.fp8_dequant_block(q8, sc)
+        cache = torch.zeros(c["nope"].shape[0], 128, 656, dtype=torch.uint8, device=dev)
+        K.cache_write_fp8(args[2].view(-1, 512), args[3].view(-1, 64),
+                          torch.arange(cache.shape[0] * 128, dtype=torch.int64, device=dev), cache)
+        out8 = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+        K.decode_fp8(args[0], args[1], cache, args[4], args[5], c["scale"], out8, q_len=q_len, num_splits=splits)
+        ref8 = O.absorbed_decode(c["q_nope"], c["q_rope"], deq, c["rope"], c["block_table"], c["seq_lens"], c["scale"])
+        attn_close(out8, ref8, 6e-2, 6e-3)
+
+    if q_len == 1 and i % 2 == 1:                             # ... and with every other key named by a row list
+        k = max(1, (hi + 1) // 2)
+        idx = torch.full((batch, k), -1, dtype=torch.int32)
+        rows = torch.zeros(batch, k, dtype=torch.int32)
+        counts = torch.zeros(batch, dtype=torch.int32)
+        for b in range(batch):
+            L = int(c["seq_lens"][b])
+            pos = torch.arange(0, L, 2)[:k]
+            idx[b, :pos.numel()] = pos.to(torch.int32)
+            rows[b, :pos.numel()] = O.slots_for(c["block_table"], b, 0, L)[pos].to(torch.int32)
+            counts[b] = pos.numel()
+        out_s = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+        K.sparse_decode(args[0], args[1], args[2], args[3], rows.to(dev), counts.to(dev), c["scale"], out_s,
+                        num_splits=splits)
+        ref_s = O.sparse_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], idx, c["scale"])
+        attn_close(out_s, ref_s, 2e-2, 2e-3)
