@@ -549,7 +549,7 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
     _need_cuda(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, out, lse_out)
     lib = _lib.load()
     t, n, p = q_nope.shape
-    k_pe = k_pe.reshape(k_pe.shape[0], -1)
+    k_pe = k_pe.reshape(k_pe.shape[0], 64)
     if p != 128 or q_pe.shape != (t, n, 64) or k_nope.shape[1:] != (n, 128) or v.shape != k_nope.shape or \
             k_pe.shape != (k_nope.shape[0], 64) or out.shape != (t, n, 128):
         raise ValueError("prefill_varlen: shapes must be q_nope [T,N,128], q_pe [T,N,64], k_nope/v [Tk,N,128], k_pe [Tk,64]")
@@ -563,6 +563,13 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
         raise TypeError("prefill_varlen: cu_q / cu_k must be contiguous int32 [B+1]")
     if lse_out is not None and (lse_out.dtype != torch.float32 or lse_out.numel() != t * n or not lse_out.is_contiguous()):
         raise TypeError("prefill_varlen: lse_out must be contiguous fp32 [T,N]")
+    if k_nope.shape[0] == 0 or t == 0:
+        # no keys at all (a context chunk in which every sequence is empty): zeros and lse = -inf, as the kernel gives for
+        # an empty key range; empty tensors have no address to hand to the library
+        out.zero_()
+        if lse_out is not None:
+            lse_out.fill_(float("-inf"))
+        return out
     rc = lib.mla_prefill_varlen(q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_pe.data_ptr(), q_pe.stride(0),
                                 q_pe.stride(1), k_nope.data_ptr(), k_nope.stride(0), k_nope.stride(1), k_pe.data_ptr(),
                                 k_pe.stride(0), v.data_ptr(), v.stride(0), v.stride(1), cu_q.data_ptr(), cu_k.data_ptr(),

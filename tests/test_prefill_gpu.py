@@ -104,3 +104,42 @@ def test_chunked_context_flow_gather_attend_merge(dev):
     K.merge_states(ctx_out, ctx_lse, out_s, lse_s, merged)
     # the reference's bar for this flow is atol = rtol = 3e-2 (tests/integration/attention/test_mla_chunked_prefill.py:72-76)
     attn_close(merged.view(t, -1), ref, 3e-2, 6e-3)
+
+
+def _random_prefill_cases(n_cases, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    for i in range(n_cases):
+        b = rng.randint(1, 4)
+        n = rng.choice([1, 2, 8, 16])
+        causal = rng.random() < 0.6
+        q_lens = [rng.choice([1, 2, 31, 32, 33, 63, 64, 65, 127, 128, 129, 200, 257]) for _ in range(b)]
+        if causal:                                            # at least as many keys as queries (right-down alignment)
+            k_lens = [q + rng.choice([0, 0, 1, 63, 64, 65, 300]) for q in q_lens]
+        else:
+            k_lens = [rng.choice([0, 1, 31, 64, 65, 129, 500]) for _ in range(b)]
+        cases.append((i, causal, q_lens, k_lens, n))
+    return cases
+
+
+@pytest.mark.parametrize("i,causal,q_lens,k_lens,n", _random_prefill_cases(32, seed=7))
+def test_prefill_varlen_random_shapes(dev, i, causal, q_lens, k_lens, n):
+    """Seeded sweep over batch, heads, ragged query and key lengths around the 32 / 64 / 128 tile edges, with and
+    without the causal mask (empty key ranges included: zeros and lse = -inf)."""
+    from omni_npu_amd import kernels as K
+    q, kv, k_pe, cu_q, cu_k = _case(500 + i, q_lens, k_lens, n)
+    scale = 192 ** -0.5
+    ref, ref_lse = O.attention_varlen(q[..., :128], q[..., 128:], kv[..., :128], k_pe.view(-1, 64), kv[..., 128:], cu_q,
+                                      cu_k, scale, causal)
+    dq, dkv, dpe = q.to(dev), kv.to(dev), k_pe.to(dev)
+    out = torch.full((q.shape[0], n, 128), float("nan"), dtype=torch.float32, device=dev)
+    lse = torch.full((q.shape[0], n), float("nan"), dtype=torch.float32, device=dev)
+    K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
+                     torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
+                     max(q_lens), scale, causal, out, lse)
+    attn_close(out, ref, 2e-2, 2e-3)
+    got_lse = lse.cpu()
+    fin = torch.isfinite(ref_lse)
+    assert torch.equal(torch.isfinite(got_lse), fin)
+    assert torch.allclose(got_lse[fin], ref_lse[fin], atol=2e-2)
