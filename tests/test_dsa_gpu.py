@@ -183,3 +183,49 @@ def test_sparse_decode_with_padding_and_full_coverage(dev):
     dense = O.absorbed_decode(dc["q_nope"], dc["q_rope"], dc["nope"], dc["rope"], dc["block_table"], dc["seq_lens"],
                               dc["scale"])
     attn_close(out, dense, 2e-2, 2e-3)
+
+
+def _random_indexer_cases(n_cases, seed):
+    import random
+    rng = random.Random(seed)
+    out = []
+    for i in range(n_cases):
+        q_len = rng.choice([1, 1, 2, 3])
+        batch = rng.randint(1, 6)
+        lo = rng.choice([q_len, 31, 32, 33, 127, 128, 129, 1000])
+        hi = lo + rng.choice([0, 1, 100, 2500])
+        k = rng.choice([1, 7, 64, 300, 2048])
+        out.append((i, batch, lo, hi, q_len, k, rng.random() < 0.5))
+    return out
+
+
+@pytest.mark.parametrize("i,batch,lo,hi,q_len,k,single_workgroup", _random_indexer_cases(24, seed=99))
+def test_indexer_topk_rows_random_shapes(dev, i, batch, lo, hi, q_len, k, single_workgroup):
+    """Seeded sweep over the indexer chain: logits against the oracle, top-k sets (on the kernel's own logits) bit-exact
+    with ties to the lower position, and the fused row translation equal to positions mapped through the block table;
+    ragged lengths around the 32-key block and 128-token page edges, MTP queries, k from 1 to 2048."""
+    from omni_npu_amd import kernels as K
+    c = make_indexer_case(batch, lo, hi, seed=300 + i, q_len=q_len)
+    t = batch * q_len
+    max_len = int(c["seq_lens"].max())
+    nblk = c["k8"].shape[0]
+    logits = torch.full((t, K.indexer_logits_stride(max_len)), float("nan"), device=dev)
+    K.indexer_scores(c["q8"].to(dev), c["w"].to(dev), c["k8"].to(dev), c["k_scale"].to(dev), c["block_table"].to(dev),
+                     c["seq_lens"].to(dev), logits, q_len=q_len, q_scale=c["q_scale"].to(dev), max_seq_len=max_len)
+    idx = torch.full((t, k), -7, dtype=torch.int32, device=dev)
+    rows = torch.full((t, k), -7, dtype=torch.int32, device=dev)
+    counts = torch.full((t,), -7, dtype=torch.int32, device=dev)
+    K.topk(logits, c["seq_lens"].to(dev), k, idx, q_len=q_len, single_workgroup=single_workgroup,
+           block_table=c["block_table"].to(dev), page_size=128, num_pages=nblk, rows=rows, counts=counts)
+    lg, idx_c, rows_c, counts_c = logits.cpu(), idx.cpu(), rows.cpu(), counts.cpu()
+    for tt in range(t):
+        ref = oracle_logits(c, tt)
+        n = ref.numel()
+        assert (lg[tt, :n] - ref).abs().max().item() <= 1e-4 * ref.abs().max().item() + 1e-6
+        want = O.topk_stable(lg[tt], k, n)
+        got = [v for v in idx_c[tt].tolist() if v >= 0]
+        assert got == sorted(v for v in want.tolist() if v >= 0), (tt, n, k)
+        assert idx_c[tt, len(got):].eq(-1).all() and int(counts_c[tt]) == len(got) == min(n, k)
+        b = tt // q_len
+        pos = torch.tensor(got, dtype=torch.long)
+        assert torch.equal(rows_c[tt, :len(got)].long(), c["block_table"][b, pos // 128].long() * 128 + pos % 128)
