@@ -715,11 +715,13 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
 // With many partials per sequence (few sequences, long contexts: up to 257 partials of one row) a single wavefront would
 // walk them in dozens of dependent round trips, so the kWide form gives a row to a whole workgroup: wavefront w merges
 // every fourth partial, sixteen per pass, and the four running states are merged through LDS at the end.
-constexpr int kRedRows = 1;
-constexpr int kRedPartsNarrow = 6, kRedPartsWide = 16;
-template <bool kWide>
+// With one chunk per sequence (large batches) a row has one partial, or two where a chunk border falls inside its
+// sequence: the kFew form then gives a wavefront four rows of two partials, a quarter of the wavefronts and rounds.
+constexpr int kRedPartsNarrow = 6, kRedPartsWide = 16, kRedPartsFew = 2, kRedRowsFew = 4;
+template <bool kWide, bool kFew>
 __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
-  constexpr int kRedParts = kWide ? kRedPartsWide : kRedPartsNarrow;
+  constexpr int kRedParts = kWide ? kRedPartsWide : (kFew ? kRedPartsFew : kRedPartsNarrow);
+  constexpr int kRedRows = kFew ? kRedRowsFew : 1;
   __shared__ float comb_ml[kWide ? 8 : 1];                  // wide: running maximum and sum of wavefronts 0..3
   __shared__ float comb_a[kWide ? 4 * 64 * 8 : 1];          //       and their unnormalised rows
   const int lane = threadIdx.x & 63;
@@ -904,16 +906,22 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
 
 int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
-  const int64_t row_groups = (int64_t)p.batch * ((r_max + kRedRows - 1) / kRedRows);
-  // a sequence has about num_chunks / batch + 1 partials; past two passes of the one-wavefront form the wide form wins
-  // (as long as all rows' workgroups are resident at once: two per CU at its register use)
-  const bool wide = p.batch > 0 && p.num_chunks / p.batch + 1 > 2 * kRedPartsNarrow && row_groups <= 512;
+  const int64_t per_seq = p.batch > 0 ? p.num_chunks / p.batch + 1 : 0;     // about that many partials per sequence
+  // many partials: past two passes of the one-wavefront form the wide form wins, as long as all rows' workgroups are
+  // resident at once (two per CU at its register use)
+  const bool wide = per_seq > 2 * kRedPartsNarrow && (int64_t)p.batch * r_max <= 512;
+  // one or two partials and rows for more than one round of resident wavefronts: four rows per wavefront
+  const bool few = !wide && per_seq <= kRedPartsFew && (int64_t)p.batch * r_max > 16384;
   if (wide) {
+    const int64_t row_groups = (int64_t)p.batch * r_max;
     const int64_t wgs = row_groups < (1ll << 30) ? row_groups : (1ll << 30);
-    hipLaunchKernelGGL(mla_chunk_reduce_kernel<true>, dim3((unsigned)wgs), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL((mla_chunk_reduce_kernel<true, false>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  } else if (few) {
+    const int64_t row_groups = (int64_t)p.batch * ((r_max + kRedRowsFew - 1) / kRedRowsFew);
+    hipLaunchKernelGGL((mla_chunk_reduce_kernel<false, true>), dim3((unsigned)((row_groups + 3) / 4)), dim3(256), 0, stream, p);
   } else {
-    const int64_t wgs = (row_groups + 3) / 4;
-    hipLaunchKernelGGL(mla_chunk_reduce_kernel<false>, dim3((unsigned)wgs), dim3(256), 0, stream, p);
+    const int64_t row_groups = (int64_t)p.batch * r_max;
+    hipLaunchKernelGGL((mla_chunk_reduce_kernel<false, false>), dim3((unsigned)((row_groups + 3) / 4)), dim3(256), 0, stream, p);
   }
   return check_launch("mla_chunk_reduce_kernel");
 }

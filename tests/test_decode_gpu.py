@@ -126,6 +126,18 @@ def test_decode_many_partials_per_sequence(dev, batch, heads, q_len, lo, hi, spl
     assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
 
 
+@pytest.mark.parametrize("batch,heads,q_len,lo,hi", [(130, 128, 1, 1, 300), (70, 128, 2, 2, 260)])
+def test_decode_large_batch_one_chunk_per_sequence(dev, batch, heads, q_len, lo, hi):
+    """More than 16384 query rows and one chunk per sequence: every row has one partial, or two where a chunk border
+    falls inside its sequence, and the merge runs four rows per wavefront."""
+    case = O.make_decode_case(batch, heads, lo, hi, seed=batch, q_len=q_len)
+    ref, ref_lse = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                                     case["seq_lens"], case["scale"], return_lse=True)
+    got, lse = _run(case, dev, 1, with_lse=True)
+    attn_close(got, ref, MAX_ABS, MEAN_REL)
+    assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
+
+
 def test_decode_single_key_returns_the_row(dev):
     """L = 1: softmax over one key is 1, the output is that latent row exactly (in bf16)."""
     case = O.make_decode_case(3, 128, 1, 1, seed=5)
