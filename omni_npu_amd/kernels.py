@@ -278,12 +278,15 @@ def _vup_out(out: torch.Tensor, w_uv: torch.Tensor, t: int, n: int) -> torch.Ten
 
 # The fused merge + up-projection gives a row to ONE wavefront (six partials per round trip).  Past this many partials per
 # sequence (few sequences with long contexts) the separate merge, which puts a workgroup on every row, followed by the
-# library GEMM is faster.
+# library GEMM is faster ...
 VUP_MAX_SPLITS = 11
+# ... and past this many query tokens a workgroup of the fused kernel walks through many passes of 16 tokens one after
+# the other, while the separate merge keeps every row in flight (measured break-even at 128 heads: 256 tokens)
+VUP_MAX_TOKENS = 256
 
 
 def _reduce_vup(lib, ws_args, seq_lens, qsl, b, q_len, n, num_splits, t, w_uv, o3, st) -> None:
-    if num_splits > VUP_MAX_SPLITS:
+    if num_splits > VUP_MAX_SPLITS or t > VUP_MAX_TOKENS:
         o = torch.empty(n, t, D_NOPE, dtype=torch.bfloat16, device=o3.device)
         rc = lib.mla_splitkv_reduce(*ws_args, seq_lens.data_ptr(), qsl, b, q_len, n, num_splits, o.data_ptr(), o.stride(1),
                                     o.stride(0), None, st)

@@ -22,11 +22,11 @@ def _w_uv(n, seed):
 @pytest.mark.parametrize("batch,heads,q_len,lo,hi,splits", [(4, 16, 1, 128, 1024, 2), (64, 128, 1, 100, 700, 4),
                                                             (5, 128, 2, 1, 600, 3), (19, 40, 1, 50, 400, None),
                                                             (2, 128, 1, 3000, 6000, 11), (3, 128, 1, 50, 300, 9),
-                                                            (2, 128, 1, 3000, 6000, 40), (150, 128, 2, 2, 200, 1)])
+                                                            (2, 128, 1, 3000, 6000, 40), (125, 128, 2, 2, 200, 1), (150, 128, 2, 2, 200, 1)])
 def test_fused_merge_and_up_projection(dev, batch, heads, q_len, lo, hi, splits):
-    """Up to 11 chunks per sequence the fused kernel runs (rows of 7..12 partials take two rounds; the case with more
-    chunks than work units has empty chunks); the last case takes the route for many partials per row (separate merge
-    with a workgroup per row, then the library GEMM) behind the same call."""
+    """Up to 11 chunks per sequence and 256 tokens the fused kernel runs (rows of 7..12 partials take two rounds; the
+    case with more chunks than work units has empty chunks); the last two cases take the other route behind the same
+    call (separate merge, then the library GEMM): many partials per row, and more than 256 tokens."""
     from omni_npu_amd import kernels as K
     c = O.make_decode_case(batch, heads, lo, hi, seed=7 * batch + q_len, q_len=q_len)
     w = _w_uv(heads, seed=batch)
