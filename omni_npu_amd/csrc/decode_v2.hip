@@ -212,6 +212,28 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (kSparse ? 0 : (int64_t)b * p.bt_stride);
   ConstI32Ptr srows = (ConstI32Ptr)(p.sparse_rows) + (kSparse ? (int64_t)b * p.sparse_stride : 0);
   const int64_t max_row = p.num_pages * p.page_size - 1;
+  // Row list (kSparse): the 32 cache rows of the block whose copies go out next travel in one vector register, lane r
+  // holding the row of key r, and every copy picks its row with v_readlane.  (A scalar load per copy would need a full
+  // lgkmcnt wait in front of every copy, and that wait also drains the K-fragment reads of the QK phase in flight: nine
+  // drains per block.)  The load for block X+1 is issued in front of the copies of block X, so the wait that lets a
+  // block's copies land also covers it (vector memory returns in order).
+  uint32_t ids_cur = 0, ids_nxt = 0;
+  auto ids_load = [&](int blk_x) {
+    if constexpr (kSparse) {
+      int tok = blk_x * kBlk + (lane & 31);
+      tok = tok < L ? tok : L - 1;
+      tok = tok < 0 ? 0 : tok;
+      const int32_t* src = p.sparse_rows + (int64_t)b * p.sparse_stride + tok;
+      asm volatile("global_load_dword %0, %1, off" : "=v"(ids_nxt) : "v"(src) : "memory");
+    }
+  };
+  // after a wait that covers the load: the register is complete, hand it to the copies of the coming block
+  auto ids_rotate = [&] {
+    if constexpr (kSparse) {
+      asm volatile("" : "+v"(ids_nxt));
+      ids_cur = ids_nxt;
+    }
+  };
   auto load_page = [&](int page) -> int64_t {
     page = page < p.max_blocks ? page : p.max_blocks - 1;
     int64_t pg = bt[page];
@@ -251,9 +273,15 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     return c;
   };
   // kFull: every row of the block exists and the source is the paged cache: plain pointer increments
-  auto issue_piece = [&](IssueCtx& c, int k, auto full) {
+  // kVecIds (row list only): the rows come from ids_cur instead of scalar loads
+  auto issue_piece = [&](IssueCtx& c, int k, auto full, auto vec_ids) {
     constexpr bool kFull = decltype(full)::value && !kSparse;
+    constexpr bool kVecIds = decltype(vec_ids)::value && kSparse;
     auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
+    auto row_of = [&](int re) -> int32_t {
+      if constexpr (kVecIds) return (int32_t)__builtin_amdgcn_readlane((int)ids_cur, re);
+      else return srows[c.tok0 + re];
+    };
     if (k < 8) {
       const int j = k >> 1;
       const int r = (k & 1) * 16 + wave * 4 + j;
@@ -262,16 +290,16 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
         else { dma16_sv(c.a1, dma_off[j], c.nbuf + r * 1024); c.a0 += n_sr2; c.a1 += n_sr2; }
       } else {
         const int re = r < c.last ? r : c.last;
-        if constexpr (kSparse) dma16_sv(c.np + clampi(srows[c.tok0 + re]) * n_sr2, dma_off[j], c.nbuf + r * 1024);
+        if constexpr (kSparse) dma16_sv(c.np + clampi(row_of(re)) * n_sr2, dma_off[j], c.nbuf + r * 1024);
         else dma16_sv(c.np + (uint64_t)re * n_sr2, dma_off[j], c.nbuf + r * 1024);
       }
     } else {
       if constexpr (kSparse) {
-        int32_t mine = 0;                                     // lane's row = 8*wave + lane/8, picked from 8 scalar loads
+        int32_t mine = 0;                                     // lane's row = 8*wave + lane/8, picked from 8 uniform values
 #pragma unroll
         for (int j = 0; j < 8; j++) {
           const int r = wave * 8 + j;
-          const int32_t sj = srows[c.tok0 + (r < c.last ? r : c.last)];
+          const int32_t sj = row_of(r < c.last ? r : c.last);
           mine = (lane >> 3) == j ? sj : mine;
         }
         dma16_v(c.rp + clampi(mine) * r_sr2 + rope_off, c.rbuf + wave * 1024);
@@ -287,15 +315,41 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   auto issue_block = [&](int blk) {
     IssueCtx c = issue_begin(blk);
 #pragma unroll
-    for (int k = 0; k < 9; k++) issue_piece(c, k, std::false_type{});
+    for (int k = 0; k < 9; k++) issue_piece(c, k, std::false_type{}, std::integral_constant<bool, kSparse>{});
   };
+  // Row list: the rows of the first kLead blocks are fetched together (one round trip) before any copy goes out
+  uint32_t ids_head[kLead] = {};
   auto issue_first = [&]() {
     issue_reset();
+    if constexpr (kSparse) {
+#pragma unroll
+      for (int j = 0; j < kLead; j++) {
+        int tok = (blk_begin + j) * kBlk + (lane & 31);
+        tok = tok < L ? tok : L - 1;
+        tok = tok < 0 ? 0 : tok;
+        const int32_t* src = p.sparse_rows + (int64_t)b * p.sparse_stride + tok;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(ids_head[j]) : "v"(src) : "memory");
+      }
+      if constexpr (kLead == 3)
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(ids_head[0]), "+v"(ids_head[1]), "+v"(ids_head[2])::"memory");
+      else
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(ids_head[0]), "+v"(ids_head[1])::"memory");
+      ids_cur = ids_head[0];
+    }
     issue_block(blk_begin);
   };
   auto issue_next_two = [&]() {
+    if constexpr (kSparse) {
+#pragma unroll
+      for (int j = 1; j < kLead; j++)
+        if (j < nb) {
+          ids_cur = ids_head[j];
+          issue_block(blk_begin + j);
+        }
+    } else {
 #pragma unroll 1
-    for (int j = 1; j < kLead && j < nb; j++) issue_block(blk_begin + j);
+      for (int j = 1; j < kLead && j < nb; j++) issue_block(blk_begin + j);
+    }
   };
 
   // ---- prologue: the first block's copies go out, then the query loads; both are waited for together ----
@@ -374,7 +428,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
     const uint32_t nb32 = lds0 + (blk & 3) * kV2NopeBufB + kbase;     // buffers are 4 KiB aligned: the XORs below stay exact
     const uint32_t rb32 = lds0 + (blk % 3) * kV2RopeBufB + rbase;
     IssueCtx ic;
-    if constexpr (kIssue) ic = issue_begin(blk_issue);
+    if constexpr (kIssue) { ids_load(blk_issue + 1); ic = issue_begin(blk_issue); }
     bf16x8 ka[kQkAheadV2];
 #define MLA_K_READ(dst, kk)                                                                                         \
     do {                                                                                                            \
@@ -399,7 +453,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       if (kk == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(s) : "v"(ka[kk % D]), "v"(qf[kk]));
       else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(s) : "v"(ka[kk % D]), "v"(qf[kk]));
       if (kk + D < 36) MLA_K_READ(ka[kk % D], kk + D);
-      if constexpr (kIssue) if ((kk & 3) == 1) issue_piece(ic, kk >> 2, std::integral_constant<bool, kIssueMode == 2>{});
+      if constexpr (kIssue) if ((kk & 3) == 1) issue_piece(ic, kk >> 2, std::integral_constant<bool, kIssueMode == 2>{}, std::true_type{});
       if (kk == 27) mid_hook();
     }
 #undef MLA_K_READ
@@ -589,6 +643,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       issue_first();
       restart = false;
     }
+    ids_load(blk_begin + kLead);                              // (older than the copies below: their wait covers it)
     issue_next_two();
     // ---- block 0: QK, softmax, publish ----
     {
@@ -612,6 +667,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       const int blk = blk_begin + i;
       // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
       if (kLead > 2 && i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
+      ids_rotate();
       lds_barrier();
       const f32x4 fl = flags_read(blk);
       f32x16 s;
