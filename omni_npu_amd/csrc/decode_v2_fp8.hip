@@ -209,11 +209,18 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV
     int64_t pg = bt[page];
     return pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
   };
+  // The page of the block being copied and the next one are kept in scalar registers, so the block-table load is never
+  // waited for in the loop (blocks are requested in ascending order; a restart begins again at the first block)
+  int page_cur = -1;
+  int64_t pg_cur = 0, pg_nxt = 0;
   auto issue_block = [&](int blk) {
     const int last = L - 1 - blk * kBlk;                      // last valid row of the block (>= 0)
     const uint32_t raw = lds0 + kRawOff + (blk & 1) * kRawStageB;
     const uint32_t rbuf = lds0 + kV2RopeOff + (blk % 3) * kV2RopeBufB;
-    const char* src = (const char*)p.cache8 + load_page(blk >> 2) * p.c8_sp + (int64_t)(blk & 3) * kBlk * kFp8RowBytes;
+    const int page = blk >> 2;
+    if (blk == blk_begin) { page_cur = page; pg_cur = load_page(page); pg_nxt = load_page(page + 1); }
+    else if (page != page_cur) { page_cur = page; pg_cur = pg_nxt; pg_nxt = load_page(page + 1); }
+    const char* src = (const char*)p.cache8 + pg_cur * p.c8_sp + (int64_t)(blk & 3) * kBlk * kFp8RowBytes;
     if (last >= kBlk - 1) {
 #pragma unroll
       for (int j = 0; j < 5; j++)
