@@ -263,7 +263,14 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       c.rp = (const char*)p.rope;
     } else {
       const int page = blk >> 2;
-      if (page != page_cur) { page_cur = page; pg_cur = pg_nxt; pg_nxt = load_page(page + 1); }
+      if (page != page_cur) {
+        // the next page's number is only asked for here (raw: clamping it now would wait for the load); it is clamped
+        // when it becomes the current page, four blocks later
+        page_cur = page;
+        pg_cur = pg_nxt < 0 ? 0 : (pg_nxt >= p.num_pages ? p.num_pages - 1 : pg_nxt);
+        const int pn = page + 1 < p.max_blocks ? page + 1 : p.max_blocks - 1;
+        pg_nxt = bt[pn];
+      }
       const uint32_t row0 = (uint32_t)(blk & 3) * kBlk;
       c.np = (const char*)p.nope + pg_cur * p.nope_sp * 2 + (uint64_t)row0 * n_sr2;
       c.rp = (const char*)p.rope + pg_cur * p.rope_sp * 2 + (uint64_t)row0 * r_sr2;
