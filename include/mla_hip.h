@@ -175,12 +175,14 @@ int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_str
  * right-down causal, sparse_mode 3) and :415-431 (context chunk: no mask, softmax_lse_flag): q_nope [T,N,128],
  * q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64] shared by all heads (mla.py:579 repeats it), v [Tk,N,128];
  * cu_q / cu_k int32 [B+1] on the device; out [T,N,128] bf16 (0) or fp32 (1); lse_out fp32 [T,N] or NULL.
+ * window = w > 0 keeps only the newest w visible keys of each row: the band of mla.py:525-541 (sparse_mode 4,
+ * pre_tokens = sliding_window - 1, next_tokens 0); 0 = no window.
  * Rows with no visible key give zeros and lse = -inf. */
 int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
                        int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
                        int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v, int64_t v_stride_t,
                        int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k, int32_t batch, int32_t num_heads,
-                       int32_t max_q_len, int32_t causal, float scale, void* out, int64_t out_stride_t,
+                       int32_t max_q_len, int32_t causal, int32_t window, float scale, void* out, int64_t out_stride_t,
                        int64_t out_stride_h, int32_t out_dtype, float* lse_out, mlahip_stream_t stream);
 
 /* ---- DSA lightning indexer --------------------------------------------------------------------
@@ -234,6 +236,16 @@ int dsa_build_rows(const int32_t* indices, int64_t indices_stride, const int32_t
                    int32_t max_blocks, const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
                    int32_t max_q_len, int32_t k, int32_t page_size, int64_t num_pages, int32_t* rows,
                    int64_t rows_stride, int32_t* counts, mlahip_stream_t stream);
+
+/* The key set of decode with static sink tokens and a sliding window (attention/backends/mla.py:705-779: one
+ * attention over the sink pages, one over the last sliding_window keys behind them, merged by LSE) as one list of flat
+ * cache rows per query token, for dsa_sparse_decode_bf16: the sink_len rows of the first sink_len / page_size pages of
+ * the block-table row, then the newest `window` keys the token sees (token i of a request with s query tokens and
+ * seq_lens[b] = L keys behind the sink sees keys [0, L - s + i]), oldest first.  rows [T, >= sink_len + window]. */
+int mla_sink_window_rows(const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, const int32_t* seq_lens,
+                         const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t sink_len,
+                         int32_t window, int32_t page_size, int64_t num_pages, int32_t* rows, int64_t rows_stride,
+                         int32_t* counts, mlahip_stream_t stream);
 
 int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
                            int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,

@@ -39,7 +39,7 @@ SIGNATURES = {
     "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                   I32, I32, F32, P, I64, I64, P, P, SZ, I32, P]),
     "mla_prefill_varlen": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, P, I64, I64, P, P, I32, I32, I32, I32,
-                                     F32, P, I64, I64, I32, P, P]),
+                                     I32, F32, P, I64, I64, I32, P, P]),
     "dsa_indexer_scores_fp8": (c_int32, [P, I64, I64, P, I64, P, I64, P, I64, I64, P, I64, I64, I32, P, I64, I32, P, P, I32,
                                          I32, I32, I32, P, I64, P]),
     "dsa_quant_rows_fp8": (c_int32, [P, I64, I64, P, P, I64, I64, P, I64, I32, I64, P]),
@@ -47,6 +47,7 @@ SIGNATURES = {
     "dsa_topk": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, SZ, P]),
     "dsa_topk_rows": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, I64, I32, I32, I64, P, I64, P, P, SZ, P]),
     "dsa_build_rows": (c_int32, [P, I64, P, I64, I32, P, P, I32, I32, I32, I32, I64, P, I64, P, P]),
+    "mla_sink_window_rows": (c_int32, [P, I64, I32, P, P, I32, I32, I32, I32, I32, I64, P, I64, P, P]),
     "dsa_sparse_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, I32, P, I64, P, I32, I32,
                                          F32, P, I64, I64, P, P, SZ, I32, P]),
 }

@@ -7,7 +7,10 @@ single-GPU path; every vendor op there is replaced by a HIP kernel of libmla_hip
   FIA prefill (mla.py:574-590, 415-431)      -> kernels.prefill_varlen
   gather / merge (ops.py)                    -> kernels.gather_paged / merge_states
 The absorb and up-projection GEMMs stay torch.bmm (hipBLASLt), as in the reference (mla.py:309-315, 900-912).
-Out of scope and rejected loudly: decode context parallelism, static-sink / sliding-window variants, mc2 masks.
+Static sink tokens with or without a sliding window (mla.py:463-560, 705-779) run as ONE attention over the union of
+the keys: without a window the sink pages are simply the first pages of the block table; with one the key set of each
+token is listed by kernels.sink_window_rows and read by kernels.sparse_decode (prefill: kernels.prefill_varlen with a
+band).  Out of scope and rejected loudly: decode context parallelism, mc2 masks.
 """
 from __future__ import annotations
 
@@ -88,6 +91,9 @@ class NPUMLADecodeMetadata(MLACommonDecodeMetadata):
     q_len: int = 1
     max_seq_len: int = 0
     mc2_mask: torch.Tensor = None
+    # static sink tokens (reference mla.py:152-153): the sink keys sit in the first pages of every block-table row and
+    # ``seq_lens`` counts the keys behind them (the reference passes it next to block_table[:, num_sink_blocks:]).
+    seq_sink_len: list = None
 
 
 @dataclass
@@ -137,6 +143,9 @@ class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
 
     def build(self, common_prefix_len: int, common_attn_metadata, fast_build: bool = False) -> NPUMLAMetadata:
         metadata = super().build(common_prefix_len, common_attn_metadata, fast_build)
+        sink_len = getattr(self.kv_cache_spec, "sink_len", 0) or 0
+        if metadata.decode is not None and sink_len > 0:
+            metadata.decode.seq_sink_len = [sink_len] * metadata.num_decodes
         if metadata.prefill is not None:
             metadata.prefill.query_start_loc_list = metadata.prefill.query_start_loc.tolist()
             metadata.prefill.query_cumlens = common_attn_metadata.query_start_loc_cpu[1:].tolist()
@@ -162,8 +171,12 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             raise NotImplementedError(
                 "NPUMLAImpl does not support one of the following: "
                 "alibi_slopes, logits_soft_cap")
-        if sliding_window is not None:
-            raise NotImplementedError("NPUMLAImpl: the static-sink / sliding-window variant is not part of this build")
+        if sliding_window is not None and sliding_window < 1:
+            raise ValueError(f"NPUMLAImpl: sliding_window must be positive (got {sliding_window})")
+        # static sink tokens (reference mla.py:278-281); the window only acts together with them, as in the reference
+        self.sink_k_pe = None
+        self.sink_compressed_kv = None
+        self.sink_len = 0
         if attn_type != AttentionType.DECODER:
             raise NotImplementedError(
                 "Encoder self-attention and "
@@ -171,6 +184,12 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
                 "are not implemented for "
                 "NPUMLAImpl")
         self.fp8_cache = kv_cache_dtype in FP8_CACHE_DTYPES
+
+    def update_sink_kv(self, sink_k_pe: torch.Tensor, sink_compressed_kv: torch.Tensor) -> None:
+        """The latents of the static sink tokens, [S,64] and [S,512] (reference mla.py:304-307)."""
+        self.sink_k_pe = sink_k_pe.unsqueeze(1)
+        self.sink_compressed_kv = sink_compressed_kv
+        self.sink_len = sink_compressed_kv.shape[0]
 
     # ---- GEMMs around the kernels (library GEMMs, as in the reference) ----
     def _v_up_proj(self, x: torch.Tensor) -> torch.Tensor:
@@ -221,6 +240,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         """Causal suffix attention merged with the chunked context (reference mla.py:452-483, 573-616)."""
         prefill = attn_metadata.prefill
         assert prefill is not None
+        if self.sink_len > 0:
+            return self._forward_prefill_sink(q, kv_c_normed, k_pe, prefill)
         if self.fp8_cache and prefill.chunked_context is not None:
             raise NotImplementedError("chunked-context prefill over the fp8 cache is not implemented")
         t, n = q.shape[0], self.num_heads
@@ -240,6 +261,48 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
                 output = merged
         return output.to(torch.bfloat16).flatten(start_dim=-2)
 
+    def _forward_prefill_sink(self, q, kv_c_normed, k_pe, prefill) -> torch.Tensor:
+        """Prefill with static sink tokens (reference mla.py:463-560): the cached context is not read (mla.py:497).
+        Without a window the sink latents go in front of every sequence's new latents and one right-down causal attention
+        runs over sink_len + s_b keys.  With a window the reference runs a sink attention and a banded attention and merges
+        them by LSE; that is the same softmax over sink keys + band, computed here by the same two kernels calls."""
+        t, n, s_len = q.shape[0], self.num_heads, self.sink_len
+        q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
+        starts = prefill.query_start_loc_list
+        nb = len(starts) - 1
+        cu_q = prefill.query_start_loc.to(torch.int32).contiguous()
+        sink_pe = self.sink_k_pe.reshape(s_len, -1)
+        output = torch.empty(t, n, self.v_head_dim, dtype=q.dtype, device=q.device)
+        if self.sliding_window is None:
+            lat = self._insert_tensor_by_start_loc(kv_c_normed, self.sink_compressed_kv, starts)
+            pe = self._insert_tensor_by_start_loc(k_pe.reshape(t, -1), sink_pe, starts)
+            k_nope, v = self._kv_up(lat)
+            cu_k = cu_q + s_len * torch.arange(nb + 1, dtype=torch.int32, device=q.device)
+            K.prefill_varlen(q_nope, q_pe, k_nope, pe, v, cu_q, cu_k, prefill.max_query_len, self.scale, True, output)
+            return output.flatten(start_dim=-2)
+        ks_nope, vs = self._kv_up(self.sink_compressed_kv)
+        cu_s = s_len * torch.arange(nb + 1, dtype=torch.int32, device=q.device)
+        out_sink = torch.empty_like(output)
+        lse_sink = torch.empty(t, n, dtype=torch.float32, device=q.device)
+        K.prefill_varlen(q_nope, q_pe, ks_nope.repeat(nb, 1, 1), sink_pe.repeat(nb, 1), vs.repeat(nb, 1, 1), cu_q, cu_s,
+                         prefill.max_query_len, self.scale, False, out_sink, lse_sink)
+        k_nope, v = self._kv_up(kv_c_normed)
+        lse = torch.empty(t, n, dtype=torch.float32, device=q.device)
+        K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
+                         output, lse, window=self.sliding_window)
+        merged = torch.empty_like(output)
+        K.merge_states(out_sink, lse_sink, output, lse, merged)
+        return merged.flatten(start_dim=-2)
+
+    @staticmethod
+    def _insert_tensor_by_start_loc(raw_tensor: torch.Tensor, insert_segment: torch.Tensor, start_loc: list) -> torch.Tensor:
+        """insert_segment in front of every raw_tensor[start_loc[i]:start_loc[i+1]] (reference mla.py:929-949)."""
+        pieces = []
+        for i in range(len(start_loc) - 1):
+            pieces.append(insert_segment)
+            pieces.append(raw_tensor[start_loc[i]:start_loc[i + 1]])
+        return torch.cat(pieces, 0)
+
     # ---- decode ----
     def _fusable_w_uv(self, out: torch.Tensor) -> bool:
         """The fused merge + up-projection kernel takes bf16 W_UV [N,512,128] with contiguous rows and writes rows of 128."""
@@ -256,6 +319,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         d = attn_metadata.decode
         assert d is not None
         t = decode_ql_nope.shape[0]
+        if self.sink_len > 0:
+            return self._forward_decode_sink(decode_ql_nope, decode_q_pe, kv_cache, d, proj_out)
         kw = dict(q_len=d.q_len, query_start_loc=d.query_start_loc, max_seq_len=d.block_table.shape[1] * K.PAGE)
         if proj_out is not None:
             if self.fp8_cache:
@@ -272,6 +337,33 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         else:
             K.decode(decode_ql_nope, decode_q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens, self.scale,
                      o.transpose(0, 1), **kw)
+        return o
+
+    def _forward_decode_sink(self, ql_nope, q_pe, kv_cache, d, proj_out: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """Decode with static sink tokens (reference mla.py:705-779).  The reference attends to the sink pages and to the
+        sequence's own pages separately and merges the two by LSE; the result is one softmax over the union of the keys,
+        and that is what runs here: the sink pages are the first pages of every block-table row, so without a window it is
+        the plain decode over sink_len + seq_len keys, and with a window the keys of each token (sink rows, then the
+        newest ``sliding_window`` keys) are listed once and read by the sparse kernel."""
+        if self.sink_len % K.PAGE != 0:
+            raise ValueError(f"sink_len {self.sink_len} must align with block size")
+        if self.fp8_cache:
+            raise NotImplementedError("static sink tokens over the fp8 cache are not implemented")
+        t, dev = ql_nope.shape[0], ql_nope.device
+        o = None
+        if proj_out is None:
+            o = torch.empty(self.num_heads, t, self.kv_lora_rank, dtype=ql_nope.dtype, device=dev)
+        out = proj_out if proj_out is not None else o.transpose(0, 1)
+        w_uv = self.W_UV if proj_out is not None else None
+        if self.sliding_window is None:
+            K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens + self.sink_len, self.scale, out,
+                     q_len=d.q_len, query_start_loc=d.query_start_loc, max_seq_len=d.block_table.shape[1] * K.PAGE, w_uv=w_uv)
+            return o
+        rows = torch.empty(t, self.sink_len + self.sliding_window, dtype=torch.int32, device=dev)
+        counts = torch.empty(t, dtype=torch.int32, device=dev)
+        K.sink_window_rows(d.block_table, d.seq_lens, self.sink_len, self.sliding_window, kv_cache[0].shape[0], rows, counts,
+                           q_len=d.q_len, query_start_loc=d.query_start_loc)
+        K.sparse_decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], rows, counts, self.scale, out, w_uv=w_uv)
         return o
 
     def forward(self, layer, q: torch.Tensor, k_c_normed: torch.Tensor, k_pe: torch.Tensor,

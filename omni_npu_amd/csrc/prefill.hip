@@ -40,6 +40,7 @@ struct PrefillParams {
   const __bf16* v; int64_t v_st, v_sh;
   const int32_t* cu_q; const int32_t* cu_k;
   int32_t batch, num_heads, causal;
+  int32_t window;                                            // keep only the newest `window` visible keys of a row; 0 = all
   float scale_log2;
   void* out; int64_t o_st, o_sh; int32_t out_fp32;
   float* lse; // [T, N]
@@ -135,6 +136,20 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) { const int other = __shfl_xor(wave_min_limit, o, 64); wave_min_limit = other < wave_min_limit ? other : wave_min_limit; }
   wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
+  // Sliding window: a row sees keys [lo, limit).  lo grows with the row, so the first row of the workgroup gives the
+  // first key any row needs, and the largest lo of a wave tells which blocks need the mask at their front.
+  const int lo = (p.window > 0 && limit > p.window) ? limit - p.window : 0;
+  int wave_max_lo = lo;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) { const int other = __shfl_xor(wave_max_lo, o, 64); wave_max_lo = other > wave_max_lo ? other : wave_max_lo; }
+  wave_max_lo = __builtin_amdgcn_readfirstlane(wave_max_lo);
+  int wg_lo = 0;
+  if (p.window > 0) {
+    int lim0 = p.causal ? qb * kPfRows + shift + 1 : sk;
+    lim0 = lim0 < 0 ? 0 : (lim0 > sk ? sk : lim0);
+    wg_lo = lim0 > p.window ? lim0 - p.window : 0;
+  }
+  const int first_tile = wg_lo / kPfTile;
   // keys any row of this workgroup can see
   int wg_limit = sk;
   if (p.causal) {
@@ -163,7 +178,7 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
       if (fast_ok && first + kPfTile - 1 <= klast) pf_issue_full_tile(p, lane_off, first, head, buf, wave);
       else pf_issue_tile(p, first, klast, head, buf, wave, lane);
     };
-    issue(0, lds0);
+    issue(first_tile, lds0 + (first_tile & 1) * kPfBufB);
 
     bf16x8 qf[12];
     {
@@ -195,7 +210,7 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
       for (int db = 0; db < 4; db++) voff[rd][db] = kPfKnB + kPfKrB + rr * 256 + v_in + (((db * 4 + v_cl) ^ f) << 4);
     }
 
-    for (int tile = 0; tile < tiles; tile++) {
+    for (int tile = first_tile; tile < tiles; tile++) {
       const char* buf = lds + (tile & 1) * kPfBufB;
       if (tile + 1 < tiles) {
         issue(tile + 1, lds0 + ((tile + 1) & 1) * kPfBufB);
@@ -208,6 +223,7 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 #pragma unroll 1
       for (int tb = 0; tb < 2; tb++) {
         if (key_base + tb * 32 >= wg_limit) break;
+        if (key_base + tb * 32 + 32 <= wg_lo) continue;       // in front of every row's window
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
@@ -224,12 +240,12 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
         // Only blocks that some row of this wave cannot see in full pay for the mask (causal diagonal, end of the keys,
         // rows past the end of the sequence); everywhere else the scores go straight to the maximum.  The scale is
         // folded into the exponent's multiply-add (scale > 0, so the maximum of the raw scores is the raw maximum).
-        if (key_base + tb * 32 + 32 > wave_min_limit) {
+        if (key_base + tb * 32 + 32 > wave_min_limit || key_base + tb * 32 < wave_max_lo) {
           const int key_lane0 = key_base + tb * 32 + 4 * half;
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             const int key = key_lane0 + 8 * (r >> 2) + (r & 3);
-            s[r] = key < limit ? s[r] : -INFINITY;
+            s[r] = (key < limit && key >= lo) ? s[r] : -INFINITY;
           }
         }
         float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
@@ -300,18 +316,19 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 }  // namespace mlahip
 using namespace mlahip;
 
-// out_dtype: 0 = bf16, 1 = fp32.  q_nope [T,N,128], q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64], v [Tk,N,128].
+// out_dtype: 0 = bf16, 1 = fp32; window: 0 = every visible key, w = the newest w of them.  q_nope [T,N,128], q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64], v [Tk,N,128].
 extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
                                   int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
                                   int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v,
                                   int64_t v_stride_t, int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k,
-                                  int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, float scale,
-                                  void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype, float* lse_out,
-                                  hipStream_t stream) {
+                                  int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, int32_t window,
+                                  float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
+                                  float* lse_out, hipStream_t stream) {
   MLA_REQUIRE(q_nope && q_pe && k_nope && k_pe && v && cu_q && cu_k && out, MLA_ERR_NULL,
               "mla_prefill_varlen: null pointer argument");
-  MLA_REQUIRE(batch >= 0 && num_heads >= 1 && max_q_len >= 0 && batch <= 65535 && num_heads <= 65535, MLA_ERR_SHAPE,
-              "mla_prefill_varlen: batch=%d num_heads=%d max_q_len=%d", batch, num_heads, max_q_len);
+  MLA_REQUIRE(batch >= 0 && num_heads >= 1 && max_q_len >= 0 && batch <= 65535 && num_heads <= 65535 && window >= 0,
+              MLA_ERR_SHAPE, "mla_prefill_varlen: batch=%d num_heads=%d max_q_len=%d window=%d", batch, num_heads, max_q_len,
+              window);
   MLA_REQUIRE(out_dtype == 0 || out_dtype == 1, MLA_ERR_UNSUPPORTED, "mla_prefill_varlen: out dtype code %d", out_dtype);
   MLA_REQUIRE(scale > 0.f, MLA_ERR_UNSUPPORTED, "mla_prefill_varlen: the softmax scale must be positive (got %g)", (double)scale);
   MLA_REQUIRE(qn_stride_t % 8 == 0 && qn_stride_h % 8 == 0 && qp_stride_t % 8 == 0 && qp_stride_h % 8 == 0 &&
@@ -327,7 +344,7 @@ extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64
   p.k_nope = (const __bf16*)k_nope; p.kn_st = kn_stride_t; p.kn_sh = kn_stride_h;
   p.k_pe = (const __bf16*)k_pe; p.kp_st = kp_stride_t;
   p.v = (const __bf16*)v; p.v_st = v_stride_t; p.v_sh = v_stride_h;
-  p.cu_q = cu_q; p.cu_k = cu_k; p.batch = batch; p.num_heads = num_heads; p.causal = causal;
+  p.cu_q = cu_q; p.cu_k = cu_k; p.batch = batch; p.num_heads = num_heads; p.causal = causal; p.window = window;
   p.scale_log2 = scale * kLog2e;
   p.out = out; p.o_st = out_stride_t; p.o_sh = out_stride_h; p.out_fp32 = out_dtype;
   p.lse = lse_out;

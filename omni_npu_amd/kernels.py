@@ -501,6 +501,33 @@ def build_sparse_rows(indices: torch.Tensor, block_table: torch.Tensor, seq_lens
     _lib.check(rc, "dsa_build_rows")
 
 
+def sink_window_rows(block_table: torch.Tensor, seq_lens: torch.Tensor, sink_len: int, window: int, num_pages: int,
+                     rows: torch.Tensor, counts: torch.Tensor, q_len: int = 1,
+                     query_start_loc: Optional[torch.Tensor] = None, page_size: int = PAGE) -> None:
+    """Flat cache rows of the keys a decode token sees with static sink tokens and a sliding window (reference: the two
+    attentions of src/omni_npu/attention/backends/mla.py:723-756): the sink rows (the first sink_len / page_size pages of
+    the block-table row), then the newest ``window`` keys behind them, oldest first; ``seq_lens`` counts the keys behind
+    the sink.  rows int32 [T, >= sink_len + window], counts int32 [T]; the pair feeds sparse_decode."""
+    _need_cuda(block_table, seq_lens, rows, counts)
+    lib = _lib.load()
+    if sink_len % page_size != 0:
+        raise ValueError(f"sink_len {sink_len} must align with block size")
+    if block_table.dtype != torch.int32 or block_table.stride(-1) != 1 or seq_lens.dtype != torch.int32 or \
+            not seq_lens.is_contiguous() or rows.dtype != torch.int32 or rows.stride(-1) != 1 or counts.dtype != torch.int32 or \
+            not counts.is_contiguous():
+        raise TypeError("sink_window_rows: int32 block_table [B,max_blocks], seq_lens [B], rows [T,K], counts [T]")
+    b = seq_lens.numel()
+    t_min = b * q_len if query_start_loc is None else 1
+    if rows.shape[0] < t_min or counts.numel() < min(t_min, rows.shape[0]) or counts.numel() < rows.shape[0] or \
+            rows.shape[1] < sink_len + window or window < 1:
+        raise ValueError("sink_window_rows: rows [T, >= sink_len + window] and counts [T], T = batch * q_len tokens")
+    rc = lib.mla_sink_window_rows(block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
+                                  query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, sink_len,
+                                  window, page_size, num_pages, rows.data_ptr(), rows.stride(0), counts.data_ptr(),
+                                  _stream(rows))
+    _lib.check(rc, "mla_sink_window_rows")
+
+
 def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
                   rows: torch.Tensor, counts: torch.Tensor, scale: float, out: torch.Tensor,
                   lse_out: Optional[torch.Tensor] = None, num_splits: Optional[int] = None,
@@ -545,10 +572,13 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
 # ------------------------------------------------------------------------------------------------
 def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tensor, k_pe: torch.Tensor, v: torch.Tensor,
                    cu_q: torch.Tensor, cu_k: torch.Tensor, max_q_len: int, scale: float, causal: bool,
-                   out: torch.Tensor, lse_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   out: torch.Tensor, lse_out: Optional[torch.Tensor] = None, window: Optional[int] = None) -> torch.Tensor:
     """Varlen non-absorbed MLA attention (reference: the prefill FIA calls, src/omni_npu/attention/backends/mla.py:574-590
     and :415-431).  q_nope [T,N,128], q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64] (shared by the heads), v [Tk,N,128],
-    cu_q / cu_k int32 [B+1] device tensors, out [T,N,128] bf16 or fp32, lse_out fp32 [T,N]."""
+    cu_q / cu_k int32 [B+1] device tensors, out [T,N,128] bf16 or fp32, lse_out fp32 [T,N].  ``window`` keeps only the
+    newest ``window`` visible keys of each row (the sliding-window band of mla.py:525-541)."""
+    if window is not None and window < 1:
+        raise ValueError(f"prefill_varlen: window must be positive (got {window})")
     _need_cuda(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, out, lse_out)
     lib = _lib.load()
     t, n, p = q_nope.shape
@@ -576,7 +606,8 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
     rc = lib.mla_prefill_varlen(q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_pe.data_ptr(), q_pe.stride(0),
                                 q_pe.stride(1), k_nope.data_ptr(), k_nope.stride(0), k_nope.stride(1), k_pe.data_ptr(),
                                 k_pe.stride(0), v.data_ptr(), v.stride(0), v.stride(1), cu_q.data_ptr(), cu_k.data_ptr(),
-                                cu_q.numel() - 1, n, int(max_q_len), 1 if causal else 0, float(scale), out.data_ptr(),
+                                cu_q.numel() - 1, n, int(max_q_len), 1 if causal else 0, int(window or 0), float(scale),
+                                out.data_ptr(),
                                 out.stride(0), out.stride(1), _DT[out.dtype],
                                 lse_out.data_ptr() if lse_out is not None else None, _stream(q_nope))
     _lib.check(rc, "mla_prefill_varlen")

@@ -28,6 +28,14 @@ Pinning status (what checks each function beyond re-typing its formula lives in
                                   torch.nn.functional.scaled_dot_product_attention and the merge identity.
 * ``v_up_proj``                   restates attention/backends/mla.py:309-315; pinned by the identity-weight
                                   known answer of tests/unit/attention/backends/test_mla.py:190-259.
+* ``sink_decode``, ``sink_prefill``,
+  ``sink_window_rows``            restate the static-sink / sliding-window branches of
+                                  attention/backends/mla.py:463-560 and :705-779 (two attentions with LSE and
+                                  their merge; band mask pre_tokens = window - 1).  The reference holds no test
+                                  of them; pinned by a per-token brute force over the union of the sink keys and
+                                  the windowed keys, by "window >= L == no window", by "sink_len keys moved into
+                                  the sequence == plain decode", and against
+                                  torch.nn.functional.scaled_dot_product_attention with an explicit mask.
 * ``indexer_scores``, ``topk_stable``, ``sparse_decode``
                                   PARITY UNPINNED against the reference: its lightning indexer and sparse
                                   flash attention are closed vendor ops with mock-only tests
@@ -165,7 +173,8 @@ def v_up_proj(o_head_major: torch.Tensor, w_uv: torch.Tensor) -> torch.Tensor:
 # absorbed paged decode
 # --------------------------------------------------------------------------------------
 def absorbed_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale,
-                    query_start_loc: Optional[Sequence[int]] = None, return_lse: bool = False):
+                    query_start_loc: Optional[Sequence[int]] = None, return_lse: bool = False,
+                    causal: bool = True, window: Optional[int] = None):
     """Absorbed MLA decode over the paged latent cache.
 
     For sequence b with L_b cached tokens (new tokens included) and s_b query tokens, query token i
@@ -175,6 +184,10 @@ def absorbed_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_len
 
     q_nope [T,N,512], q_rope [T,N,64]; caches [nblk,page,512] / [nblk,page,64] (a singleton head dim is
     accepted); returns out fp32 [T,N,512] (token-major) and optionally lse [T,N].
+
+    ``causal=False`` lets every query token see all L_b keys (the sink call of mla.py:723-737 passes no mask);
+    ``window`` keeps only the last ``window`` visible keys of each row (sparse_mode=4 with
+    pre_tokens = sliding_window - 1, mla.py:740-756).
     """
     t_tot, n, _ = q_nope.shape
     nb = len(seq_lens)
@@ -199,11 +212,13 @@ def absorbed_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_len
         qn = q_nope[q0:q1].float().reshape(s * n, -1)
         qr = q_rope[q0:q1].float().reshape(s * n, -1)
         sc = (qn @ kc.t() + qr @ kr.t()) * scale             # [s*n, L]
-        if s > 1:
-            lim = (L - s + torch.arange(s) + 1).repeat_interleave(n)      # visible key count per row
+        lim = (L - s + torch.arange(s) + 1).repeat_interleave(n) if causal else torch.full((s * n,), L)
+        if s > 1 and causal:
             sc = sc.masked_fill(torch.arange(L).view(1, -1) >= lim.view(-1, 1), float("-inf"))
+        if window is not None:
+            sc = sc.masked_fill(torch.arange(L).view(1, -1) < (lim - window).view(-1, 1), float("-inf"))
         lse_b = torch.logsumexp(sc, dim=-1)
-        p = torch.softmax(sc, dim=-1)
+        p = torch.nan_to_num(torch.softmax(sc, dim=-1), nan=0.0)
         out[q0:q1] = (p @ kc).view(s, n, -1)
         lse[q0:q1] = lse_b.view(s, n)
     return (out, lse) if return_lse else out
@@ -219,12 +234,14 @@ def kv_up_proj(kv_c: torch.Tensor, w_kv_b: torch.Tensor, n_heads: int, p: int, v
     return kv[..., :p], kv[..., p:]
 
 
-def attention_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, scale, causal: bool):
+def attention_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, scale, causal: bool, window: Optional[int] = None):
     """Varlen non-absorbed attention with LSE.
 
     q_nope [T,N,P], q_pe [T,N,R], k_nope [Tk,N,P], k_pe [Tk,R] (shared by all heads,
     attention/backends/mla.py:579), v [Tk,N,V].  ``causal`` is right-down aligned
-    (sparse_mode=3, attention/backends/mla.py:584-585).  Empty key ranges give out = 0, lse = -inf.
+    (sparse_mode=3, attention/backends/mla.py:584-585); with ``window`` only the last ``window`` visible keys
+    of a row stay (sparse_mode=4, pre_tokens = sliding_window - 1, mla.py:525-541).  Empty key ranges give
+    out = 0, lse = -inf.
     Returns out fp32 [T,N,V], lse fp32 [T,N].
     """
     t, n, _ = q_nope.shape
@@ -238,7 +255,10 @@ def attention_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, scale, causal: b
         sc = (torch.einsum("tnd,snd->nts", q_nope[q0:q1].float(), k_nope[k0:k1].float())
               + torch.einsum("tnd,sd->nts", q_pe[q0:q1].float(), k_pe[k0:k1].float())) * scale
         if causal:
-            vis = torch.arange(sk).view(1, -1) <= (torch.arange(sq).view(-1, 1) + (sk - sq))
+            last = torch.arange(sq).view(-1, 1) + (sk - sq)                 # last visible key of each row
+            vis = torch.arange(sk).view(1, -1) <= last
+            if window is not None:
+                vis &= torch.arange(sk).view(1, -1) > last - window
             sc = sc.masked_fill(~vis.unsqueeze(0), float("-inf"))
         l = torch.logsumexp(sc, dim=-1)                       # [n, sq]
         p = torch.nan_to_num(torch.softmax(sc, dim=-1), nan=0.0)
@@ -415,6 +435,89 @@ def sparse_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens,
         lse[b] = torch.logsumexp(sc, -1)
         out[b] = torch.softmax(sc, -1) @ kc
     return (out, lse) if return_lse else out
+
+
+# --------------------------------------------------------------------------------------
+# static sink tokens (+ sliding window)
+# --------------------------------------------------------------------------------------
+def sink_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, sink_len: int, scale,
+                window: Optional[int] = None, query_start_loc: Optional[Sequence[int]] = None):
+    """Decode with static sink tokens (attention/backends/mla.py:705-779).
+
+    The first sink_len / 128 pages of every block-table row hold the sink keys (sink_len must be a multiple of the
+    page, mla.py:719-721); ``seq_lens`` counts the keys behind them.  One attention over the sink keys (no mask,
+    mla.py:723-737), one over the sequence's own keys through block_table[:, sink pages:] (causal tail for several
+    query tokens, optionally only the last ``window`` keys, mla.py:740-773), merged by their LSEs (mla.py:776-779).
+    Returns fp32 [T,N,512] token-major."""
+    page = nope_cache.shape[1]
+    if sink_len % page != 0:
+        raise ValueError(f"sink_len {sink_len} must align with block size")
+    nsb = sink_len // page
+    nb = len(seq_lens)
+    o_s, l_s = absorbed_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, [sink_len] * nb, scale,
+                               query_start_loc, return_lse=True, causal=False)
+    o_n, l_n = absorbed_decode(q_nope, q_rope, nope_cache, rope_cache, block_table[:, nsb:], seq_lens, scale,
+                               query_start_loc, return_lse=True, window=window)
+    m = torch.maximum(l_s, l_n)
+    w_s, w_n = torch.exp(l_s - m).unsqueeze(-1), torch.exp(l_n - m).unsqueeze(-1)
+    return (o_s * w_s + o_n * w_n) / (w_s + w_n)
+
+
+def sink_window_rows(block_table, seq_lens, sink_len: int, window: Optional[int], q_len: int = 1, page: int = PAGE):
+    """The keys of ``sink_decode`` as flat cache rows per query token: the sink rows first, then the visible keys
+    of the sequence (the last ``window`` of them when a window is given), oldest first.  Returns rows
+    [T, sink_len + width] int32 (unused tail = 0) and counts [T] int32, width = window or the longest sequence."""
+    nb = len(seq_lens)
+    width = int(window) if window is not None else int(max(int(x) for x in seq_lens))
+    rows = torch.zeros(nb * q_len, sink_len + width, dtype=torch.int32)
+    counts = torch.zeros(nb * q_len, dtype=torch.int32)
+    for b in range(nb):
+        L = int(seq_lens[b])
+        for i in range(q_len):
+            n_vis = max(0, L - q_len + i + 1)
+            lo = max(0, n_vis - window) if window is not None else 0
+            pos = torch.cat([torch.arange(sink_len), sink_len + torch.arange(lo, n_vis)])
+            t = b * q_len + i
+            rows[t, :pos.numel()] = (block_table[b, pos // page].long() * page + pos % page).to(torch.int32)
+            counts[t] = pos.numel()
+    return rows, counts
+
+
+def insert_sink_rows(x: torch.Tensor, sink: torch.Tensor, cu_q: Sequence[int]) -> torch.Tensor:
+    """The sink rows in front of every sequence's rows (mla.py:929-949)."""
+    parts = []
+    for b in range(len(cu_q) - 1):
+        parts += [sink, x[int(cu_q[b]):int(cu_q[b + 1])]]
+    return torch.cat(parts, 0)
+
+
+def sink_prefill(q, kv_c, k_pe, w_kv_b, sink_kv_c, sink_k_pe, cu_q, scale, window: Optional[int] = None,
+                 p_dim: int = 128, v_dim: int = 128):
+    """Prefill with static sink tokens (attention/backends/mla.py:463-560).  No cached context is read
+    (has_context is forced off, mla.py:497).
+
+    Without a window the sink latents are put in front of every sequence's new latents and one right-down causal
+    attention runs over sink_len + s_b keys (mla.py:463-491, 546-572).  With a window the sink keys get their own
+    unmasked attention, the new keys a causal band of ``window`` keys, and the two are merged by LSE with the
+    sink as the prefix (mla.py:498-557).  q [T,N,P+R]; kv_c [T,512], k_pe [T,64]; sink_kv_c [S,512], sink_k_pe
+    [S,64].  Returns fp32 [T, N*V]."""
+    t, n, _ = q.shape
+    q_nope, q_pe = q[..., :p_dim], q[..., p_dim:]
+    nb = len(cu_q) - 1
+    s_len = sink_kv_c.shape[0]
+    cu_q = [int(x) for x in cu_q]
+    if window is None:
+        k_nope, v = kv_up_proj(insert_sink_rows(kv_c, sink_kv_c, cu_q), w_kv_b, n, p_dim, v_dim)
+        cu_k = [cu_q[i] + s_len * i for i in range(nb + 1)]
+        out, _ = attention_varlen(q_nope, q_pe, k_nope, insert_sink_rows(k_pe, sink_k_pe, cu_q), v, cu_q, cu_k, scale, True)
+        return out.reshape(t, -1)
+    ks_nope, vs = kv_up_proj(sink_kv_c, w_kv_b, n, p_dim, v_dim)
+    o_s, l_s = attention_varlen(q_nope, q_pe, ks_nope.repeat(nb, 1, 1), sink_k_pe.repeat(nb, 1), vs.repeat(nb, 1, 1),
+                                cu_q, [s_len * i for i in range(nb + 1)], scale, False)
+    k_nope, v = kv_up_proj(kv_c, w_kv_b, n, p_dim, v_dim)
+    o_n, l_n = attention_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_q, scale, True, window=window)
+    out, _ = merge_attn_states(o_s, l_s.unsqueeze(-1), o_n, l_n.unsqueeze(-1))
+    return out.reshape(t, -1)
 
 
 # --------------------------------------------------------------------------------------

@@ -200,9 +200,32 @@ def test_impl_rejects_unsupported_features(cls):
     with pytest.raises(NotImplementedError):
         _impl(cls, logits_soft_cap=30.0)
     with pytest.raises(NotImplementedError):
-        _impl(cls, sliding_window=128)
-    with pytest.raises(NotImplementedError):
         _impl(cls, attn_type=V.AttentionType.ENCODER)
+    if cls is dsa.NPUDSAImpl:
+        with pytest.raises(NotImplementedError):
+            _impl(cls, sliding_window=128)
+    else:
+        # the MLA backend takes a window for its static-sink variant (reference mla.py:281) and keeps no sink by default
+        impl = _impl(cls, sliding_window=128)
+        assert impl.sliding_window == 128 and impl.sink_len == 0 and impl.sink_compressed_kv is None
+        with pytest.raises(ValueError, match="sliding_window"):
+            _impl(cls, sliding_window=0)
+
+
+def test_update_sink_kv_and_sink_metadata():
+    """update_sink_kv keeps the latents as the reference does (mla.py:304-307); the builder marks decode metadata with
+    the sink length of the cache spec (mla.py:152-153)."""
+    impl = _impl(mla.NPUMLAImpl)
+    impl.update_sink_kv(torch.zeros(128, 64), torch.zeros(128, 512))
+    assert impl.sink_len == 128 and impl.sink_k_pe.shape == (128, 1, 64) and impl.sink_compressed_kv.shape == (128, 512)
+    spec = V.AttentionSpec(128, 1, 576, torch.bfloat16)
+    spec.sink_len = 128
+    builder = mla.NPUMLAMetadataBuilder(spec, ["l0"], _cfg(), torch.device("cpu"))
+    md = builder.build(0, _common([1, 1, 1], [10, 200, 31]))
+    assert md.decode.seq_sink_len == [128, 128, 128]
+    md0 = mla.NPUMLAMetadataBuilder(V.AttentionSpec(128, 1, 576, torch.bfloat16), ["l0"], _cfg(), torch.device("cpu")).build(
+        0, _common([1, 1], [10, 20]))
+    assert md0.decode.seq_sink_len is None
 
 
 @pytest.mark.parametrize("cls", [mla.NPUMLAImpl, dsa.NPUDSAImpl])

@@ -1,0 +1,194 @@
+"""Static sink tokens with and without a sliding window on the GPU (reference attention/backends/mla.py:463-560 and
+:705-779) against the oracle: the row lists bit-exact, the attentions within the bf16 bar, at kernel level and through
+NPUMLAImpl.forward."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from omni_npu_amd import _vllm_compat as V
+from omni_npu_amd.attention.backends import mla
+from oracle import mla_oracle as O
+from tests.conftest import attn_close
+from tests.test_backend_gpu import _mk_impl, _to
+from tests.test_boundary import _cfg, _common
+from tests.test_sink_oracle import _sink_case
+
+pytestmark = pytest.mark.gpu
+MAX_ABS, MEAN_REL = 2e-2, 2e-3
+
+
+# ---- the row lists (integer work: bit-exact) ------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,lo,hi,sink_len,window,q_len", [
+    (5, 1, 700, 128, 64, 1), (4, 3, 900, 256, 300, 2), (3, 1, 40, 128, 1, 3), (6, 100, 2000, 0, 512, 1),
+    (2, 5000, 9000, 128, 4096, 2), (3, 10, 50, 384, 1000, 1)])
+def test_sink_window_rows_bit_exact(dev, batch, lo, hi, sink_len, window, q_len):
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(batch, 2, lo, hi, sink_len, q_len, seed=batch * 7 + q_len)
+    want_rows, want_counts = O.sink_window_rows(bt, c["seq_lens"], sink_len, window, q_len)
+    t = batch * q_len
+    rows = torch.full((t, sink_len + window + 5), -7, dtype=torch.int32, device=dev)     # wider than needed, strided
+    counts = torch.full((t,), -7, dtype=torch.int32, device=dev)
+    K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), sink_len, window, c["nope"].shape[0], rows, counts, q_len=q_len)
+    rows, counts = rows.cpu(), counts.cpu()
+    assert torch.equal(counts, want_counts)
+    for i in range(t):
+        n = int(counts[i])
+        assert torch.equal(rows[i, :n], want_rows[i, :n]) and (rows[i, n:] == -7).all()    # nothing written past the count
+
+
+def test_sink_window_rows_ragged_query_lengths_and_errors(dev):
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(3, 2, 50, 400, 128, 1, seed=2)
+    q_lens = [1, 3, 2]
+    qsl = torch.tensor([0, 1, 4, 6], dtype=torch.int32)
+    rows = torch.zeros(6, 128 + 32, dtype=torch.int32, device=dev)
+    counts = torch.zeros(6, dtype=torch.int32, device=dev)
+    K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), 128, 32, c["nope"].shape[0], rows, counts, q_len=3,
+                       query_start_loc=qsl.to(dev))
+    got_rows, got_counts = rows.cpu(), counts.cpu()
+    for b in range(3):
+        L, s = int(c["seq_lens"][b]), q_lens[b]
+        for i in range(s):
+            last = L - s + i
+            first = max(0, last - 31)
+            pos = torch.cat([torch.arange(128), 128 + torch.arange(first, last + 1)])
+            want = (bt[b, pos // 128].long() * 128 + pos % 128).to(torch.int32)
+            t = int(qsl[b]) + i
+            assert int(got_counts[t]) == pos.numel() and torch.equal(got_rows[t, :pos.numel()], want)
+    with pytest.raises(ValueError, match="must align with block size"):
+        K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), 100, 32, c["nope"].shape[0], rows, counts)
+    with pytest.raises(ValueError, match="sink_len \\+ window"):
+        K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), 128, 64, c["nope"].shape[0], rows, counts)
+
+
+# ---- decode at kernel level -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("batch,heads,lo,hi,sink_len,window,q_len", [
+    (4, 128, 200, 3000, 128, 512, 1), (3, 128, 1, 100, 128, 16, 1), (3, 16, 300, 900, 256, 100, 2),
+    (2, 128, 2000, 5000, 128, 4096, 1), (2, 128, 600, 700, 128, 1, 3)])
+def test_sink_window_decode_matches_oracle(dev, batch, heads, lo, hi, sink_len, window, q_len):
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(batch, heads, lo, hi, sink_len, q_len, seed=batch + heads + q_len)
+    t = batch * q_len
+    rows = torch.zeros(t, sink_len + window, dtype=torch.int32, device=dev)
+    counts = torch.zeros(t, dtype=torch.int32, device=dev)
+    K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), sink_len, window, c["nope"].shape[0], rows, counts, q_len=q_len)
+    out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.sparse_decode(c["q_nope"].to(dev), c["q_rope"].to(dev), c["nope"].to(dev), c["rope"].to(dev), rows, counts, c["scale"], out)
+    ref = O.sink_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], bt, c["seq_lens"], sink_len, c["scale"], window)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+
+
+def test_sink_decode_without_window_is_the_dense_kernel_over_the_longer_table(dev):
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(5, 128, 100, 2500, 256, 2, seed=21)
+    out = torch.full((10, 128, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.decode(c["q_nope"].to(dev), c["q_rope"].to(dev), c["nope"].to(dev), c["rope"].to(dev), bt.to(dev),
+             (c["seq_lens"] + 256).to(dev), c["scale"], out, q_len=2)
+    ref = O.sink_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], bt, c["seq_lens"], 256, c["scale"], None)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+
+
+# ---- prefill with a band ----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("q_lens,k_extra,window,heads", [
+    ([200], [0], 64, 4), ([37, 300, 1], [0, 0, 0], 7, 4), ([129, 64], [50, 300], 100, 8), ([500], [0], 1, 2),
+    ([260, 131], [0, 17], 128, 16), ([70], [0], 1000, 4), ([1000], [24], 129, 2)])
+def test_prefill_with_a_sliding_window_matches_oracle(dev, q_lens, k_extra, window, heads):
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(sum(q_lens) + window)
+    k_lens = [a + b for a, b in zip(q_lens, k_extra)]
+    cu_q = [0] + torch.tensor(q_lens).cumsum(0).tolist()
+    cu_k = [0] + torch.tensor(k_lens).cumsum(0).tolist()
+    t, tk = cu_q[-1], cu_k[-1]
+    qn, qp = torch.randn(t, heads, 128, generator=g).bfloat16(), torch.randn(t, heads, 64, generator=g).bfloat16()
+    kn, kp = torch.randn(tk, heads, 128, generator=g).bfloat16(), torch.randn(tk, 64, generator=g).bfloat16()
+    v = torch.randn(tk, heads, 128, generator=g).bfloat16()
+    scale = 192 ** -0.5
+    out = torch.full((t, heads, 128), float("nan"), dtype=torch.float32, device=dev)
+    lse = torch.full((t, heads), float("nan"), dtype=torch.float32, device=dev)
+    K.prefill_varlen(qn.to(dev), qp.to(dev), kn.to(dev), kp.to(dev), v.to(dev), torch.tensor(cu_q, dtype=torch.int32, device=dev),
+                     torch.tensor(cu_k, dtype=torch.int32, device=dev), max(q_lens), scale, True, out, lse, window=window)
+    ref, ref_lse = O.attention_varlen(qn, qp, kn, kp, v, cu_q, cu_k, scale, True, window=window)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+    assert (lse.cpu() - ref_lse).abs().max() < 2e-2
+    with pytest.raises(ValueError, match="window must be positive"):
+        K.prefill_varlen(qn.to(dev), qp.to(dev), kn.to(dev), kp.to(dev), v.to(dev), torch.tensor(cu_q, dtype=torch.int32, device=dev),
+                         torch.tensor(cu_k, dtype=torch.int32, device=dev), max(q_lens), scale, True, out, lse, window=0)
+
+
+# ---- through NPUMLAImpl.forward ---------------------------------------------------------------------------------
+def _with_sink_pages(common, nsb):
+    """Block tables of _common moved up by nsb pages, with the shared sink pages 0..nsb-1 in front of every row."""
+    bt = common.block_table_tensor + nsb
+    sink = torch.arange(nsb, dtype=torch.int32).view(1, -1).expand(bt.shape[0], -1)
+    common.block_table_tensor = torch.cat([sink, bt], 1).contiguous()
+    return common
+
+
+@pytest.mark.parametrize("window", [None, 48])
+@pytest.mark.parametrize("q_lens,seq_lens,n", [([1] * 4, [160, 7, 300, 129], 4), ([2, 2, 2], [500, 129, 1000], 128)])
+def test_impl_decode_with_sink_tokens(dev, q_lens, seq_lens, n, window):
+    g = torch.Generator().manual_seed(len(q_lens) + (window or 0))
+    sink_len, nsb = 128, 1
+    common = _with_sink_pages(_common(q_lens, seq_lens), nsb)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    q = torch.randn(t, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(t, 512, generator=g).bfloat16(), torch.randn(t, 1, 64, generator=g).bfloat16()
+    own = common.block_table_tensor[:, nsb:]
+    common.slot_mapping = torch.cat([O.slots_for(own, b, s - ql, s) for b, (ql, s) in enumerate(zip(q_lens, seq_lens))])
+    impl, w = _mk_impl(mla.NPUMLAImpl, n, dev, sliding_window=window)
+    impl.update_sink_kv(rope[0].to(dev), nope[0].to(dev))                       # the sink latents are what page 0 holds
+    spec = V.AttentionSpec(128, 1, 576, torch.bfloat16)
+    spec.sink_len = sink_len
+    builder = mla.NPUMLAMetadataBuilder(spec, ["l"], _cfg(cap=2), dev)
+    # oracle: write the new rows, absorb q, sink decode, up-project
+    O.cache_write(nope, common.slot_mapping, kvc)
+    O.cache_write(rope, common.slot_mapping, kpe.view(-1, 64))
+    kvw = w.float().view(512, n, 256)
+    ql = torch.einsum("tnp,lnp->tnl", q[..., :128].float(), kvw[..., :128]).bfloat16()    # the absorb GEMM stores bf16
+    qsl = common.query_start_loc_cpu.tolist()
+    o = O.sink_decode(ql, q[..., 128:].float(), nope, rope, common.block_table_tensor, common.seq_lens_cpu, sink_len,
+                      impl.scale, window, query_start_loc=qsl)
+    ref = torch.einsum("tnl,lnv->tnv", o, kvw[..., 128:]).reshape(t, -1)
+    meta = builder.build(0, _to(common, dev))
+    assert meta.decode.seq_sink_len == [sink_len] * len(q_lens)
+    # the cache before the write: the oracle's copy minus the new rows is not needed, the write puts the same rows
+    raw = torch.cat([nope.reshape(-1), rope.reshape(-1)]).to(dev).view(torch.uint8)
+    kv_cache = mla.NPUMLABackend.reshape_kv_cache(raw, nblk, 128, 1, 576, dtype=torch.bfloat16)
+    out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    impl.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), kv_cache, meta, output=out)
+    attn_close(out, ref, 3e-2, 8e-3)
+
+
+@pytest.mark.parametrize("window", [None, 20])
+def test_impl_prefill_with_sink_tokens(dev, window):
+    g = torch.Generator().manual_seed(31 + (window or 0))
+    n, sink_len, nsb = 4, 128, 1
+    q_lens = [16, 200, 37]
+    common = _with_sink_pages(_common(q_lens, q_lens), nsb)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    q = torch.randn(t, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(t, 512, generator=g).bfloat16(), torch.randn(t, 1, 64, generator=g).bfloat16()
+    sink_c, sink_pe = torch.randn(sink_len, 512, generator=g).bfloat16(), torch.randn(sink_len, 64, generator=g).bfloat16()
+    own = common.block_table_tensor[:, nsb:]
+    common.slot_mapping = torch.cat([O.slots_for(own, b, 0, s) for b, s in enumerate(q_lens)])
+    impl, w = _mk_impl(mla.NPUMLAImpl, n, dev, sliding_window=window)
+    impl.update_sink_kv(sink_pe.to(dev), sink_c.to(dev))
+    spec = V.AttentionSpec(128, 1, 576, torch.bfloat16)
+    spec.sink_len = sink_len
+    builder = mla.NPUMLAMetadataBuilder(spec, ["l"], _cfg(cap=2), dev)
+    ref = O.sink_prefill(q.float(), kvc, kpe.view(-1, 64), w, sink_c, sink_pe, common.query_start_loc_cpu.tolist(),
+                         impl.scale, window)
+    meta = builder.build(0, _to(common, dev))
+    raw = torch.zeros(nblk * 128 * 576, dtype=torch.bfloat16, device=dev).view(torch.uint8)
+    kv_cache = mla.NPUMLABackend.reshape_kv_cache(raw, nblk, 128, 1, 576, dtype=torch.bfloat16)
+    out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    impl.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), kv_cache, meta, output=out)
+    attn_close(out, ref, 3e-2, 8e-3)
+    # the new latents went into the pages behind the sink page
+    sm = common.slot_mapping.cpu()
+    assert torch.equal(kv_cache[0].view(-1, 512)[sm.to(dev)].cpu(), kvc)
