@@ -705,7 +705,9 @@ __global__ __launch_bounds__(256) void mla_sink_window_rows_kernel(const SinkRow
   const int lo = n_vis > p.window ? n_vis - p.window : 0;
   const int count = p.sink_len + n_vis - lo;
   int32_t* rows = p.rows + (int64_t)t * p.r_st;
-  for (int i = threadIdx.x; i < count; i += 256) {
+  // blockIdx.y strides over the list in pieces of 1024 entries, so that a few long lists still fill the device
+  for (int i0 = blockIdx.y * 1024; i0 < count; i0 += gridDim.y * 1024)
+  for (int i = i0 + threadIdx.x; i < i0 + 1024 && i < count; i += 256) {
     const int pos = i < p.sink_len ? i : i + lo;
     int pg = pos / p.page_size;
     const int off = pos - pg * p.page_size;
@@ -714,7 +716,7 @@ __global__ __launch_bounds__(256) void mla_sink_window_rows_kernel(const SinkRow
     blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
     rows[i] = (int32_t)(blk * p.page_size + off);
   }
-  if (threadIdx.x == 0) p.counts[t] = count;
+  if (threadIdx.x == 0 && blockIdx.y == 0) p.counts[t] = count;
 }
 
 }  // namespace mlahip
@@ -832,6 +834,8 @@ extern "C" int mla_sink_window_rows(const int32_t* block_table, int64_t bt_strid
   if (batch == 0) return MLA_OK;
   SinkRowsParams p{block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, sink_len, window,
                    page_size, num_pages, rows, rows_stride, counts};
-  hipLaunchKernelGGL(mla_sink_window_rows_kernel, dim3(batch * max_q_len), dim3(256), 0, stream, p);
+  const int64_t pieces = ((int64_t)sink_len + window + 1023) / 1024;
+  hipLaunchKernelGGL(mla_sink_window_rows_kernel, dim3(batch * max_q_len, (unsigned)(pieces < 64 ? pieces : 64)), dim3(256), 0,
+                     stream, p);
   return check_launch("mla_sink_window_rows_kernel");
 }
