@@ -347,8 +347,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         newest ``sliding_window`` keys) are listed once and read by the sparse kernel."""
         if self.sink_len % K.PAGE != 0:
             raise ValueError(f"sink_len {self.sink_len} must align with block size")
-        if self.fp8_cache:
-            raise NotImplementedError("static sink tokens over the fp8 cache are not implemented")
+        if self.fp8_cache and self.sliding_window is not None:
+            raise NotImplementedError("static sink tokens with a sliding window over the fp8 cache are not implemented")
         t, dev = ql_nope.shape[0], ql_nope.device
         o = None
         if proj_out is None:
@@ -356,8 +356,12 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         out = proj_out if proj_out is not None else o.transpose(0, 1)
         w_uv = self.W_UV if proj_out is not None else None
         if self.sliding_window is None:
-            K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens + self.sink_len, self.scale, out,
-                     q_len=d.q_len, query_start_loc=d.query_start_loc, max_seq_len=d.block_table.shape[1] * K.PAGE, w_uv=w_uv)
+            kw = dict(q_len=d.q_len, query_start_loc=d.query_start_loc, max_seq_len=d.block_table.shape[1] * K.PAGE, w_uv=w_uv)
+            if self.fp8_cache:
+                K.decode_fp8(ql_nope, q_pe, kv_cache[0], d.block_table, d.seq_lens + self.sink_len, self.scale, out, **kw)
+            else:
+                K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens + self.sink_len, self.scale, out,
+                         **kw)
             return o
         rows = torch.empty(t, self.sink_len + self.sliding_window, dtype=torch.int32, device=dev)
         counts = torch.empty(t, dtype=torch.int32, device=dev)

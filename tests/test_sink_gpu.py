@@ -8,6 +8,7 @@ import torch
 
 from omni_npu_amd import _vllm_compat as V
 from omni_npu_amd.attention.backends import mla
+from omni_npu_amd.compilation.acl_graph import HIPGraphWrapper
 from oracle import mla_oracle as O
 from tests.conftest import attn_close
 from tests.test_backend_gpu import _mk_impl, _to
@@ -192,3 +193,91 @@ def test_impl_prefill_with_sink_tokens(dev, window):
     # the new latents went into the pages behind the sink page
     sm = common.slot_mapping.cpu()
     assert torch.equal(kv_cache[0].view(-1, 512)[sm.to(dev)].cpu(), kvc)
+
+
+def test_impl_decode_with_sink_tokens_over_the_fp8_cache(dev):
+    """Without a window the sink pages are just the first pages of the table, for the fp8 cache as for the bf16 one; the
+    oracle reads the dequantised cache.  With a window the fp8 cache is rejected."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(77)
+    n, sink_len, nsb = 128, 128, 1
+    q_lens, seq_lens = [2, 2, 2], [300, 129, 700]
+    common = _with_sink_pages(_common(q_lens, seq_lens), nsb)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    q = torch.randn(t, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(t, 512, generator=g).bfloat16(), torch.randn(t, 1, 64, generator=g).bfloat16()
+    own = common.block_table_tensor[:, nsb:]
+    common.slot_mapping = torch.cat([O.slots_for(own, b, s - ql, s) for b, (ql, s) in enumerate(zip(q_lens, seq_lens))])
+    O.cache_write(nope, common.slot_mapping, kvc)
+    O.cache_write(rope, common.slot_mapping, kpe.view(-1, 64))
+    cache = torch.zeros(nblk, 128, K.FP8_ROW_BYTES, dtype=torch.uint8, device=dev)
+    K.cache_write_fp8(nope.view(-1, 512).to(dev), rope.view(-1, 64).to(dev), torch.arange(nblk * 128, device=dev), cache)
+    q8, sc = O.fp8_quant_block(nope.float())
+    nope_deq = O.fp8_dequant_block(q8, sc)
+    impl, w = _mk_impl(mla.NPUMLAImpl, n, dev, kv_cache_dtype="fp8")
+    impl.update_sink_kv(rope[0].to(dev), nope[0].to(dev))
+    spec = V.AttentionSpec(128, 1, 576, torch.bfloat16)
+    spec.sink_len = sink_len
+    meta = mla.NPUMLAMetadataBuilder(spec, ["l"], _cfg(cap=2), dev).build(0, _to(common, dev))
+    kvw = w.float().view(512, n, 256)
+    ql = torch.einsum("tnp,lnp->tnl", q[..., :128].float(), kvw[..., :128]).bfloat16()
+    o = O.sink_decode(ql, q[..., 128:].float(), nope_deq, rope, common.block_table_tensor.cpu(), common.seq_lens_cpu, sink_len,
+                      impl.scale, None, query_start_loc=common.query_start_loc_cpu.tolist())
+    ref = torch.einsum("tnl,lnv->tnv", o, kvw[..., 128:]).reshape(t, -1)
+    out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    impl.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), (cache,), meta, output=out)
+    attn_close(out, ref, 6e-2, 1.2e-2)
+    impl_w, _ = _mk_impl(mla.NPUMLAImpl, n, dev, kv_cache_dtype="fp8", sliding_window=64)
+    impl_w.update_sink_kv(rope[0].to(dev), nope[0].to(dev))
+    with pytest.raises(NotImplementedError, match="sliding window over the fp8 cache"):
+        impl_w.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), (cache,), meta, output=out)
+
+
+@pytest.mark.parametrize("window", [None, 200])
+def test_graph_replay_of_the_sink_decode_sees_new_lengths(dev, window):
+    """The sink paths add work in front of the attention kernel (a length add, or the row list); captured in a HIP graph
+    they must read the device tensors' new contents on every replay."""
+    n, sink_len, nsb = 128, 128, 1
+    q_lens, seq_lens = [1] * 5, [900, 130, 257, 64, 1000]
+    common = _with_sink_pages(_common(q_lens, seq_lens), nsb)
+    nblk = int(common.block_table_tensor.max()) + 1
+    g = torch.Generator().manual_seed(19)
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16().to(dev)
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16().to(dev)
+    impl, w = _mk_impl(mla.NPUMLAImpl, n, dev, sliding_window=window)
+    impl.update_sink_kv(rope[0], nope[0])
+    spec = V.AttentionSpec(128, 1, 576, torch.bfloat16)
+    spec.sink_len = sink_len
+    builder = mla.NPUMLAMetadataBuilder(spec, ["l"], _cfg(cap=1), dev)
+    own = common.block_table_tensor[:, nsb:].clone()
+    common.slot_mapping = torch.cat([O.slots_for(own, b, s - 1, s) for b, s in enumerate(seq_lens)])
+    meta = builder.build(0, _to(common, dev))
+    q = torch.randn(5, n, 192, generator=g).bfloat16().to(dev)
+    kvc, kpe = torch.randn(5, 512, generator=g).bfloat16().to(dev), torch.randn(5, 1, 64, generator=g).bfloat16().to(dev)
+    out = torch.zeros(5, n * 128, dtype=torch.bfloat16, device=dev)
+
+    def model(qq):
+        return impl.forward(None, qq, kvc, kpe, (nope, rope), meta, output=out)
+
+    model(q)
+    torch.cuda.synchronize()
+    wrapper = HIPGraphWrapper(model, _cfg(), V.CUDAGraphMode.FULL)
+    desc = V.BatchDescriptor(num_tokens=5, num_reqs=5, uniform=True)
+    seen = []
+    with V.set_forward_context({"l": meta}, desc, V.CUDAGraphMode.FULL):
+        wrapper(q)
+        for trial in range(3):
+            q.copy_(torch.randn(5, n, 192, generator=g).bfloat16())
+            new_lens = torch.tensor([s - 20 * (trial + 1) for s in seq_lens], dtype=torch.int32)
+            meta.decode.seq_lens.copy_(new_lens.to(dev))
+            meta.slot_mapping.copy_(torch.cat([O.slots_for(own, b, int(s) - 1, int(s)) for b, s in enumerate(new_lens)]).to(dev))
+            got = wrapper(q).clone()
+            torch.cuda.synchronize()
+            out.zero_()
+            eager = model(q).clone()
+            assert torch.equal(got, eager), f"replay {trial} differs from eager"
+            seen.append(got)
+    assert not torch.equal(seen[0], seen[1])
