@@ -570,7 +570,7 @@ def main():
         "step_hbm_gbs": round(ab["total"] / (dev_step_avg * 1e-6) / 1e9, 1),
         "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                                     / (dev_step_avg * 1e-6), 4),
-        "roofline": {"kernel": "mla_decode_v2_kernel<false>", "bound": "hbm", "achieved": round(achieved, 1),
+        "roofline": {"kernel": "mla_decode_v2_kernel<false, false>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "kernel_us_avg": round(k_avg, 2), "kernel_us_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),

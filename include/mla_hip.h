@@ -237,15 +237,25 @@ int dsa_build_rows(const int32_t* indices, int64_t indices_stride, const int32_t
                    int32_t max_q_len, int32_t k, int32_t page_size, int64_t num_pages, int32_t* rows,
                    int64_t rows_stride, int32_t* counts, mlahip_stream_t stream);
 
-/* The key set of decode with static sink tokens and a sliding window (attention/backends/mla.py:705-779: one
- * attention over the sink pages, one over the last sliding_window keys behind them, merged by LSE) as one list of flat
- * cache rows per query token, for dsa_sparse_decode_bf16: the sink_len rows of the first sink_len / page_size pages of
- * the block-table row, then the newest `window` keys the token sees (token i of a request with s query tokens and
- * seq_lens[b] = L keys behind the sink sees keys [0, L - s + i]), oldest first.  rows [T, >= sink_len + window]. */
-int mla_sink_window_rows(const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, const int32_t* seq_lens,
-                         const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t sink_len,
-                         int32_t window, int32_t page_size, int64_t num_pages, int32_t* rows, int64_t rows_stride,
-                         int32_t* counts, mlahip_stream_t stream);
+/* Decode with static sink tokens and a sliding window on the dense kernel (attention/backends/mla.py:705-779: the
+ * reference runs one attention over the sink pages, one over the last sliding_window keys behind them and merges the two
+ * by LSE; this is the same softmax over the union of the keys in one pass).  The first sink_len / 128 pages of every
+ * block-table row hold the sink keys; seq_lens counts the keys behind them; token i of a request with s query tokens
+ * sees the sink and keys [max(0, L - s + i + 1 - window), L - s + i] behind it.
+ * mla_window_plan writes, per sequence, the number of 32-key blocks between the sink and the oldest visible key (skip)
+ * and the length of the sequence without them (short_lens); mla_decode_bf16_window_split is mla_decode_bf16_split over
+ * those shortened sequences; the merge is mla_splitkv_reduce / mla_splitkv_reduce_vup with seq_lens = short_lens. */
+int mla_window_plan(const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch, int32_t max_q_len,
+                    int32_t sink_len, int32_t window, int32_t* short_lens, int32_t* skip, mlahip_stream_t stream);
+
+int mla_decode_bf16_window_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                 int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,
+                                 int64_t nope_row_stride, const void* rope_cache, int64_t rope_page_stride,
+                                 int64_t rope_row_stride, int64_t num_pages, const int32_t* block_table, int64_t bt_stride,
+                                 int32_t max_blocks, const int32_t* short_lens, const int32_t* skip,
+                                 const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                                 int32_t sink_len, int32_t window, float scale, void* workspace, size_t workspace_bytes,
+                                 int32_t num_splits, mlahip_stream_t stream);
 
 int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
                            int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,

@@ -34,6 +34,9 @@ SIGNATURES = {
     "mla_decode_workspace_bytes": (SZ, [I32, I32, I32, I32]),
     "mla_decode_bf16_split": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                         I32, I32, F32, P, SZ, I32, P]),
+    "mla_window_plan": (c_int32, [P, P, I32, I32, I32, I32, P, P, P]),
+    "mla_decode_bf16_window_split": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, P,
+                                               I32, I32, I32, I32, I32, F32, P, SZ, I32, P]),
     "mla_splitkv_reduce": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, P, I64, I64, P, P]),
     "mla_splitkv_reduce_vup": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, I32, P, I64, I64, P, I64, I64, P]),
     "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
@@ -47,7 +50,6 @@ SIGNATURES = {
     "dsa_topk": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, SZ, P]),
     "dsa_topk_rows": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, I64, I32, I32, I64, P, I64, P, P, SZ, P]),
     "dsa_build_rows": (c_int32, [P, I64, P, I64, I32, P, P, I32, I32, I32, I32, I64, P, I64, P, P]),
-    "mla_sink_window_rows": (c_int32, [P, I64, I32, P, P, I32, I32, I32, I32, I32, I64, P, I64, P, P]),
     "dsa_sparse_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, I32, P, I64, P, I32, I32,
                                          F32, P, I64, I64, P, P, SZ, I32, P]),
 }

@@ -8,9 +8,8 @@ single-GPU path; every vendor op there is replaced by a HIP kernel of libmla_hip
   gather / merge (ops.py)                    -> kernels.gather_paged / merge_states
 The absorb and up-projection GEMMs stay torch.bmm (hipBLASLt), as in the reference (mla.py:309-315, 900-912).
 Static sink tokens with or without a sliding window (mla.py:463-560, 705-779) run as ONE attention over the union of
-the keys: without a window the sink pages are simply the first pages of the block table; with one the key set of each
-token is listed by kernels.sink_window_rows and read by kernels.sparse_decode (prefill: kernels.prefill_varlen with a
-band).  Out of scope and rejected loudly: decode context parallelism, mc2 masks.
+the keys: without a window the sink pages are simply the first pages of the block table; with one the dense decode
+kernel leaves out the blocks between the sink and the window (prefill: kernels.prefill_varlen with a band).  Out of scope and rejected loudly: decode context parallelism, mc2 masks.
 """
 from __future__ import annotations
 
@@ -343,8 +342,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         """Decode with static sink tokens (reference mla.py:705-779).  The reference attends to the sink pages and to the
         sequence's own pages separately and merges the two by LSE; the result is one softmax over the union of the keys,
         and that is what runs here: the sink pages are the first pages of every block-table row, so without a window it is
-        the plain decode over sink_len + seq_len keys, and with a window the keys of each token (sink rows, then the
-        newest ``sliding_window`` keys) are listed once and read by the sparse kernel."""
+        the plain decode over sink_len + seq_len keys, and with a window the dense kernel walks each sequence with the
+        blocks between the sink and the window left out (kernels.decode(..., sink_len=, window=))."""
         if self.sink_len % K.PAGE != 0:
             raise ValueError(f"sink_len {self.sink_len} must align with block size")
         if self.fp8_cache and self.sliding_window is not None:
@@ -363,11 +362,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
                 K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens + self.sink_len, self.scale, out,
                          **kw)
             return o
-        rows = torch.empty(t, self.sink_len + self.sliding_window, dtype=torch.int32, device=dev)
-        counts = torch.empty(t, dtype=torch.int32, device=dev)
-        K.sink_window_rows(d.block_table, d.seq_lens, self.sink_len, self.sliding_window, kv_cache[0].shape[0], rows, counts,
-                           q_len=d.q_len, query_start_loc=d.query_start_loc)
-        K.sparse_decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], rows, counts, self.scale, out, w_uv=w_uv)
+        K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens, self.scale, out, q_len=d.q_len,
+                 query_start_loc=d.query_start_loc, w_uv=w_uv, sink_len=self.sink_len, window=self.sliding_window)
         return o
 
     def forward(self, layer, q: torch.Tensor, k_c_normed: torch.Tensor, k_pe: torch.Tensor,

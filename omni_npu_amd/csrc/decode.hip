@@ -39,7 +39,8 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
                                      const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
                                      int32_t max_q_len, int32_t num_heads, float scale, void* workspace,
                                      size_t workspace_bytes, int32_t num_splits, const int32_t* sparse_rows,
-                                     int64_t sparse_stride, int32_t page_size, bool fp8, hipStream_t stream) {
+                                     int64_t sparse_stride, int32_t page_size, bool fp8, hipStream_t stream,
+                                     const int32_t* win_skip = nullptr, int32_t win_sink = 0, int32_t win_size = 0) {
   MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && (block_table || sparse_rows) && seq_lens, MLA_ERR_NULL,
               "mla_decode_bf16: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && (sparse_rows || max_blocks >= 1) &&
@@ -79,9 +80,11 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   v.seg_ids = (int32_t*)(v.lse_part + 4 * rows);
   v.sparse_rows = sparse_rows; v.sparse_stride = sparse_stride; v.page_size = page_size;
   v.cache8 = fp8 ? (const uint8_t*)nope_cache : nullptr; v.c8_sp = nope_page_stride;
+  v.win_skip = win_skip; v.win_sink = win_sink; v.win_size = win_size;
   // one workgroup per (balanced chunk, group of 128 query rows)
   const dim3 grid((unsigned)(batch * num_splits), 1, (unsigned)((r_max + kRowsPerWg - 1) / kRowsPerWg));
   if (fp8) return launch_decode_v2_fp8(v, grid, stream);
+  if (win_skip) return launch_decode_v2_window(v, grid, stream);
   return launch_decode_v2(v, sparse_rows != nullptr, grid, stream);
 }
 
@@ -99,6 +102,57 @@ extern "C" int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, in
                            nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
                            block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
                            scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, false, stream);
+}
+
+// Static sink tokens + sliding window on the dense kernel.  mla_window_plan turns the lengths behind the sink into the
+// lengths of the shortened sequences the kernel walks (sink keys + the blocks that hold some token's window) and the
+// number of 32-key blocks left out; mla_decode_bf16_window_split is mla_decode_bf16_split over those, and the merge is
+// the ordinary one with the shortened lengths.
+namespace mlahip {
+__global__ void mla_window_plan_kernel(const int32_t* seq_lens, const int32_t* qsl, int32_t batch, int32_t max_q_len,
+                                       int32_t sink_len, int32_t window, int32_t* short_lens, int32_t* skip) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= batch) return;
+  int qlen = qsl ? qsl[b + 1] - qsl[b] : max_q_len;
+  qlen = qlen < max_q_len ? qlen : max_q_len;
+  const int len = seq_lens[b];
+  int n0 = len - qlen + 1;                                   // keys the request's first query token sees
+  n0 = n0 < 0 ? 0 : n0;
+  const int lo0 = n0 > window ? n0 - window : 0;             // the oldest key any of its tokens sees
+  const int sk = lo0 / 32;
+  skip[b] = sk;
+  short_lens[b] = len > 0 ? sink_len + len - sk * 32 : 0;
+}
+}  // namespace mlahip
+
+extern "C" int mla_window_plan(const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch, int32_t max_q_len,
+                               int32_t sink_len, int32_t window, int32_t* short_lens, int32_t* skip, hipStream_t stream) {
+  MLA_REQUIRE(seq_lens && short_lens && skip, MLA_ERR_NULL, "mla_window_plan: null pointer argument");
+  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && sink_len >= 0 && sink_len % kPage == 0 && window >= 1, MLA_ERR_SHAPE,
+              "mla_window_plan: batch=%d max_q_len=%d sink_len=%d window=%d", batch, max_q_len, sink_len, window);
+  if (batch == 0) return MLA_OK;
+  hipLaunchKernelGGL(mla_window_plan_kernel, dim3((batch + 255) / 256), dim3(256), 0, stream, seq_lens, query_start_loc, batch,
+                     max_q_len, sink_len, window, short_lens, skip);
+  return check_launch("mla_window_plan_kernel");
+}
+
+extern "C" int mla_decode_bf16_window_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                            int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                                            int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                                            int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                                            const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                            const int32_t* short_lens, const int32_t* skip, const int32_t* query_start_loc,
+                                            int32_t batch, int32_t max_q_len, int32_t num_heads, int32_t sink_len,
+                                            int32_t window, float scale, void* workspace, size_t workspace_bytes,
+                                            int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(block_table && skip, MLA_ERR_NULL, "mla_decode_bf16_window_split: null block table or skip counts");
+  MLA_REQUIRE(sink_len >= 0 && sink_len % kPage == 0 && window >= 1, MLA_ERR_SHAPE,
+              "mla_decode_bf16_window_split: sink_len=%d window=%d", sink_len, window);
+  return decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
+                           nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
+                           block_table, bt_stride, max_blocks, short_lens, query_start_loc, batch, max_q_len, num_heads,
+                           scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, false, stream, skip, sink_len,
+                           window);
 }
 
 // Phase 2: N-way log-sum-exp merge of the workspace partials into the bf16 output (and optional lse).

@@ -101,8 +101,13 @@ __device__ __forceinline__ int wave_incl_scan_i32(int v, int lane) {
 
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
-template <bool kSparse>
+// kWindow (dense only): static sink keys followed by a sliding window.  The kernel walks a shortened sequence: the
+// blocks between the sink and the first block of the window are left out of the block numbering (block v >= sink blocks
+// is block v + skip of the cache), so the chunk plan, the ring buffers and the end-of-sequence masking work on the
+// shortened length unchanged; what differs is the address of a block and one more mask at the window's front.
+template <bool kSparse, bool kWindow>
 __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Params p) {
+  static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -190,6 +195,9 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   const int head = row - t_local * p.num_heads;
   int limit = row_ok ? (L - qlen + t_local + 1) : 0;         // keys [0, limit) are visible to this row
   limit = limit < 0 ? 0 : limit;
+  // window variant: blocks left out behind the sink, and the first block that is not a sink block
+  const int win_skip = kWindow ? p.win_skip[b] : 0;
+  const int win_blk0 = kWindow ? p.win_sink / kBlk : 0;
   const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
 
   if (grp * 128 >= rows) {
@@ -243,7 +251,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   int64_t pg_cur = 0, pg_nxt = 0;
   auto issue_reset = [&]() {
     if constexpr (!kSparse) {
-      page_cur = blk_begin >> 2;
+      page_cur = (blk_begin + (kWindow && blk_begin >= win_blk0 ? win_skip : 0)) >> 2;
       pg_cur = load_page(page_cur);
       pg_nxt = load_page(page_cur + 1);
     }
@@ -262,16 +270,18 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
       c.np = (const char*)p.nope;
       c.rp = (const char*)p.rope;
     } else {
-      const int page = blk >> 2;
+      const int cblk = blk + (kWindow && blk >= win_blk0 ? win_skip : 0);   // block of the cache
+      const int page = cblk >> 2;
       if (page != page_cur) {
         // the next page's number is only asked for here (raw: clamping it now would wait for the load); it is clamped
         // when it becomes the current page, four blocks later
+        if (kWindow && page != page_cur + 1) pg_cur = load_page(page);         // the jump from the sink to the window
+        else pg_cur = pg_nxt < 0 ? 0 : (pg_nxt >= p.num_pages ? p.num_pages - 1 : pg_nxt);
         page_cur = page;
-        pg_cur = pg_nxt < 0 ? 0 : (pg_nxt >= p.num_pages ? p.num_pages - 1 : pg_nxt);
         const int pn = page + 1 < p.max_blocks ? page + 1 : p.max_blocks - 1;
         pg_nxt = bt[pn];
       }
-      const uint32_t row0 = (uint32_t)(blk & 3) * kBlk;
+      const uint32_t row0 = (uint32_t)(cblk & 3) * kBlk;
       c.np = (const char*)p.nope + pg_cur * p.nope_sp * 2 + (uint64_t)row0 * n_sr2;
       c.rp = (const char*)p.rope + pg_cur * p.rope_sp * 2 + (uint64_t)row0 * r_sr2;
     }
@@ -523,14 +533,21 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   // After the steps: the last blocks of a sequence hold keys that some rows must not see (causal multi-token queries,
   // rows past the end of the sequence); only those blocks pay for the masking.  Then P^T and the flag go to LDS.
   auto softmax_finish = [&](int blk, f32x16& s, SoftmaxState& st) {
-    if ((blk + 1) * kBlk > L - p.max_q_len + 1) {
+    // window variant: the blocks right behind the sink hold keys older than some row's window (fewer than 32 + the
+    // number of query tokens of them, so at most two blocks)
+    bool front = false;
+    if constexpr (kWindow) front = blk >= win_blk0 && blk * kBlk < L - p.win_size;
+    if ((blk + 1) * kBlk > L - p.max_q_len + 1 || front) {
       int blk_s = blk;                                        // opaque: keeps the compiler from carrying `rel` as a loop
       asm volatile("" : "+s"(blk_s));                         // variable of its own (one more register across the loop)
       const int rel = limit - blk_s * kBlk - ((lane_now() >> 3) & 4);   // score r is visible iff 8*(r/4) + r%4 < rel
+      // ... and, behind the sink, iff it is one of the row's newest win_size keys: 8*(r/4) + r%4 >= rel - win_size
+      const int rel_lo = (kWindow && blk >= win_blk0) ? rel - p.win_size : -64;
       st.psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        s[r] = (8 * (r >> 2) + (r & 3)) < rel ? s[r] : 0.f;
+        const int kpos = 8 * (r >> 2) + (r & 3);
+        s[r] = (kpos < rel && kpos >= rel_lo) ? s[r] : 0.f;
         st.psum += s[r];
       }
 #pragma unroll
@@ -713,11 +730,12 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
         slot = slot < 0 ? 0 : (slot > max_row ? max_row : slot);
         vrow = p.nope + slot * p.nope_sr;
       } else {
-        int page = top_tok / kPage;
+        const int ctok = top_tok + ((kWindow && top_tok >= p.win_sink) ? win_skip * kBlk : 0);   // position in the cache
+        int page = ctok / kPage;
         page = page < p.max_blocks ? page : p.max_blocks - 1;
         int64_t pg = p.block_table[(int64_t)b * p.bt_stride + page];
         pg = pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
-        vrow = p.nope + pg * p.nope_sp + (int64_t)(top_tok % kPage) * p.nope_sr;
+        vrow = p.nope + pg * p.nope_sp + (int64_t)(ctok % kPage) * p.nope_sr;
       }
     }
     if (half == 0) {
@@ -767,6 +785,7 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_kernel(const DecodeV2Par
   }
   }  // segments
 }
+
 
 // N-way merge of the partials of the query rows (src/omni_npu/attention/ops.py:109-141), for the chunk layout written
 // by mla_decode_v2_kernel.  The partials of sequence b are those of the chunks that hold blocks of it, numbered
@@ -990,11 +1009,18 @@ int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
 }
 
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream) {
-  const int rc = sparse ? ensure_dynamic_lds((const void*)mla_decode_v2_kernel<true>, kV2LdsB, "dsa_sparse_decode_bf16")
-                        : ensure_dynamic_lds((const void*)mla_decode_v2_kernel<false>, kV2LdsB, "mla_decode_bf16");
+  const int rc = sparse ? ensure_dynamic_lds((const void*)mla_decode_v2_kernel<true, false>, kV2LdsB, "dsa_sparse_decode_bf16")
+                        : ensure_dynamic_lds((const void*)mla_decode_v2_kernel<false, false>, kV2LdsB, "mla_decode_bf16");
   if (rc != MLA_OK) return rc;
-  if (sparse) hipLaunchKernelGGL(mla_decode_v2_kernel<true>, grid, dim3(256), kV2LdsB, stream, p);
-  else hipLaunchKernelGGL(mla_decode_v2_kernel<false>, grid, dim3(256), kV2LdsB, stream, p);
+  if (sparse) hipLaunchKernelGGL((mla_decode_v2_kernel<true, false>), grid, dim3(256), kV2LdsB, stream, p);
+  else hipLaunchKernelGGL((mla_decode_v2_kernel<false, false>), grid, dim3(256), kV2LdsB, stream, p);
+  return check_launch("mla_decode_v2_kernel");
+}
+
+int launch_decode_v2_window(const DecodeV2Params& p, dim3 grid, hipStream_t stream) {
+  const int rc = ensure_dynamic_lds((const void*)mla_decode_v2_kernel<false, true>, kV2LdsB, "mla_decode_bf16_window_split");
+  if (rc != MLA_OK) return rc;
+  hipLaunchKernelGGL((mla_decode_v2_kernel<false, true>), grid, dim3(256), kV2LdsB, stream, p);
   return check_launch("mla_decode_v2_kernel");
 }
 

@@ -22,6 +22,10 @@ struct DecodeV2Params {
   int32_t* seg_ids;              // [B][2]: partial number of the sequence's first / last segment
   const int32_t* sparse_rows; int64_t sparse_stride; int32_t page_size;
   const uint8_t* cache8; int64_t c8_sp;   // fp8 kernel: block-scaled cache, page stride in bytes (rows are 656 bytes apart)
+  // Sink + sliding window (dense bf16 kernel only): seq_lens then holds the length of the sequence with the 32-key
+  // blocks between the sink and the window taken out, win_skip[b] is how many were taken out, and a key behind the
+  // sink is visible to a row only if it is one of the newest win_size keys the row may see.
+  const int32_t* win_skip; int32_t win_sink, win_size;
 };
 
 struct ChunkReduceParams {
@@ -46,6 +50,8 @@ int launch_reduce_vup(const ChunkReduceParams& r, const void* w_uv, int64_t w_st
 
 // Launches mla_decode_v2_kernel<sparse> on `stream`; returns 0 or a negative error code.
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
+// The dense kernel with a sink and a sliding window (p.win_skip set).
+int launch_decode_v2_window(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
 // Launches mla_decode_v2_fp8_kernel (decode_v2_fp8.hip) over p.cache8.
 int launch_decode_v2_fp8(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
 

@@ -680,45 +680,6 @@ __global__ __launch_bounds__(256) void dsa_build_rows_kernel(const RowsParams p)
   if (tid == 255) p.counts[t] = base + s;                  // inclusive total of the last thread
 }
 
-// The key set of decode with static sink tokens and a sliding window, as flat cache rows per query token: the
-// sink_len rows of the sink pages (the first pages of the block-table row), then the newest `window` keys the token
-// may see, oldest first.  Token ti of a request with qlen query tokens and L keys behind the sink sees keys
-// [0, L - qlen + ti] of them.
-struct SinkRowsParams {
-  const int32_t* block_table; int64_t bt_stride; int32_t max_blocks;
-  const int32_t* seq_lens; const int32_t* qsl;
-  int32_t batch, max_q_len, sink_len, window, page_size;
-  int64_t num_pages;
-  int32_t* rows; int64_t r_st;
-  int32_t* counts;
-};
-
-__global__ __launch_bounds__(256) void mla_sink_window_rows_kernel(const SinkRowsParams p) {
-  const int b = blockIdx.x / p.max_q_len;
-  const int ti = blockIdx.x - b * p.max_q_len;
-  int q0, qlen;
-  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
-  if (ti >= qlen) return;
-  const int t = q0 + ti;
-  int n_vis = p.seq_lens[b] - qlen + ti + 1;
-  n_vis = n_vis < 0 ? 0 : n_vis;
-  const int lo = n_vis > p.window ? n_vis - p.window : 0;
-  const int count = p.sink_len + n_vis - lo;
-  int32_t* rows = p.rows + (int64_t)t * p.r_st;
-  // blockIdx.y strides over the list in pieces of 1024 entries, so that a few long lists still fill the device
-  for (int i0 = blockIdx.y * 1024; i0 < count; i0 += gridDim.y * 1024)
-  for (int i = i0 + threadIdx.x; i < i0 + 1024 && i < count; i += 256) {
-    const int pos = i < p.sink_len ? i : i + lo;
-    int pg = pos / p.page_size;
-    const int off = pos - pg * p.page_size;
-    pg = pg < p.max_blocks ? pg : p.max_blocks - 1;
-    int64_t blk = p.block_table[(int64_t)b * p.bt_stride + pg];
-    blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
-    rows[i] = (int32_t)(blk * p.page_size + off);
-  }
-  if (threadIdx.x == 0 && blockIdx.y == 0) p.counts[t] = count;
-}
-
 }  // namespace mlahip
 using namespace mlahip;
 
@@ -819,23 +780,4 @@ extern "C" int dsa_build_rows(const int32_t* indices, int64_t indices_stride, co
                k, page_size, num_pages, rows, rows_stride, counts};
   hipLaunchKernelGGL(dsa_build_rows_kernel, dim3(batch * max_q_len), dim3(256), 0, stream, p);
   return check_launch("dsa_build_rows_kernel");
-}
-
-extern "C" int mla_sink_window_rows(const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, const int32_t* seq_lens,
-                                    const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t sink_len,
-                                    int32_t window, int32_t page_size, int64_t num_pages, int32_t* rows, int64_t rows_stride,
-                                    int32_t* counts, hipStream_t stream) {
-  MLA_REQUIRE(block_table && seq_lens && rows && counts, MLA_ERR_NULL, "mla_sink_window_rows: null pointer argument");
-  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && page_size >= 1 && num_pages >= 1 && max_blocks >= 1 && sink_len >= 0 &&
-                  window >= 1 && sink_len % page_size == 0 && (int64_t)sink_len + window <= rows_stride &&
-                  num_pages * page_size < (1ll << 31),
-              MLA_ERR_SHAPE, "mla_sink_window_rows: batch=%d max_q_len=%d sink_len=%d window=%d page_size=%d rows_stride=%lld",
-              batch, max_q_len, sink_len, window, page_size, (long long)rows_stride);
-  if (batch == 0) return MLA_OK;
-  SinkRowsParams p{block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, sink_len, window,
-                   page_size, num_pages, rows, rows_stride, counts};
-  const int64_t pieces = ((int64_t)sink_len + window + 1023) / 1024;
-  hipLaunchKernelGGL(mla_sink_window_rows_kernel, dim3(batch * max_q_len, (unsigned)(pieces < 64 ? pieces : 64)), dim3(256), 0,
-                     stream, p);
-  return check_launch("mla_sink_window_rows_kernel");
 }

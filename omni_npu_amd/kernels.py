@@ -347,7 +347,7 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
            q_len: int = 1, query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
            num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
            workspace: Optional[torch.Tensor] = None, phase: str = "both",
-           w_uv: Optional[torch.Tensor] = None) -> torch.Tensor:
+           w_uv: Optional[torch.Tensor] = None, sink_len: int = 0, window: Optional[int] = None) -> torch.Tensor:
     """Absorbed-MLA paged decode (reference: FIA decode call, src/omni_npu/attention/backends/mla.py:781-804).
 
     q_nope [T,N,512], q_rope [T,N,64] (any token/head strides), caches [nblk,128,512] / [nblk,128,64],
@@ -358,7 +358,15 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
     ``phase`` = "both" | "split" | "reduce" runs the split-KV kernel, the reduction, or both (one C call).
     With ``w_uv`` (bf16 [N,512,128], the reference's W_UV) the value up-projection of mla.py:309-315 is fused into the
     reduction: ``out`` is then [T, N*128] (or a [T,N,128] view) and holds o[t,n,:] @ w_uv[n]; no lse_out.
+    With ``window`` the call is the static-sink + sliding-window decode of mla.py:705-779 as one attention: the first
+    ``sink_len`` keys of every block-table row are the sink, ``seq_lens`` counts the keys behind them, and a token sees
+    the sink plus the newest ``window`` keys it may see.
     """
+    if window is not None:
+        return _decode_window(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out, q_len,
+                              query_start_loc, lse_out, num_splits, max_seq_len, workspace, phase, w_uv, sink_len, window)
+    if sink_len:
+        raise ValueError("decode: sink_len goes with window (without one, pass seq_lens + sink_len)")
     if w_uv is not None:
         if lse_out is not None or phase == "split":
             raise ValueError("decode: w_uv goes with the reduction and without lse_out")
@@ -387,6 +395,40 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
         _lib.check(rc, "mla_splitkv_reduce")
     else:
         raise ValueError(f"decode: unknown phase {phase!r}")
+    return out
+
+
+def _decode_window(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out, q_len, query_start_loc,
+                   lse_out, num_splits, max_seq_len, workspace, phase, w_uv, sink_len, window):
+    """decode() with static sink keys and a sliding window: a plan kernel shortens every sequence to sink + window
+    blocks, the dense split kernel walks the shortened sequences, and the ordinary merge (or merge + up-projection)
+    follows with the shortened lengths."""
+    if phase != "both":
+        raise ValueError("decode: the windowed decode runs both phases")
+    if window < 1 or sink_len < 0 or sink_len % PAGE != 0:
+        raise ValueError(f"decode: window {window} must be positive and sink_len {sink_len} a whole number of pages")
+    if w_uv is not None and lse_out is not None:
+        raise ValueError("decode: w_uv goes without lse_out")
+    t, n, _ = q_nope.shape
+    o3 = _vup_out(out, w_uv, t, n) if w_uv is not None else None
+    longest = sink_len + window + 32 + q_len                  # keys of a shortened sequence
+    max_seq_len = longest if max_seq_len is None else min(max_seq_len, longest)
+    lib, front, ws_args, lse_p, st, qsl, seq_lens, b, n, num_splits = _decode_args(
+        q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out if o3 is None else o3,
+        D_NOPE if o3 is None else 128, q_len, query_start_loc, lse_out, num_splits, max_seq_len, workspace)
+    plan = torch.empty(2, b, dtype=torch.int32, device=q_nope.device)      # shortened lengths, blocks left out
+    short, skip = plan[0], plan[1]
+    _lib.check(lib.mla_window_plan(seq_lens.data_ptr(), qsl, b, q_len, sink_len, window, short.data_ptr(), skip.data_ptr(), st),
+               "mla_window_plan")
+    rc = lib.mla_decode_bf16_window_split(*front[:16], short.data_ptr(), skip.data_ptr(), qsl, b, q_len, n, sink_len, window,
+                                          float(scale), *ws_args, num_splits, st)
+    _lib.check(rc, "mla_decode_bf16_window_split")
+    if o3 is not None:
+        _reduce_vup(lib, ws_args, short, qsl, b, q_len, n, num_splits, t, w_uv, o3, st)
+    else:
+        rc = lib.mla_splitkv_reduce(*ws_args, short.data_ptr(), qsl, b, q_len, n, num_splits, out.data_ptr(), out.stride(0),
+                                    out.stride(1), lse_p, st)
+        _lib.check(rc, "mla_splitkv_reduce")
     return out
 
 
@@ -499,33 +541,6 @@ def build_sparse_rows(indices: torch.Tensor, block_table: torch.Tensor, seq_lens
                             query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, idx.shape[1],
                             page_size, num_pages, rows.data_ptr(), rows.stride(0), counts.data_ptr(), _stream(idx))
     _lib.check(rc, "dsa_build_rows")
-
-
-def sink_window_rows(block_table: torch.Tensor, seq_lens: torch.Tensor, sink_len: int, window: int, num_pages: int,
-                     rows: torch.Tensor, counts: torch.Tensor, q_len: int = 1,
-                     query_start_loc: Optional[torch.Tensor] = None, page_size: int = PAGE) -> None:
-    """Flat cache rows of the keys a decode token sees with static sink tokens and a sliding window (reference: the two
-    attentions of src/omni_npu/attention/backends/mla.py:723-756): the sink rows (the first sink_len / page_size pages of
-    the block-table row), then the newest ``window`` keys behind them, oldest first; ``seq_lens`` counts the keys behind
-    the sink.  rows int32 [T, >= sink_len + window], counts int32 [T]; the pair feeds sparse_decode."""
-    _need_cuda(block_table, seq_lens, rows, counts)
-    lib = _lib.load()
-    if sink_len % page_size != 0:
-        raise ValueError(f"sink_len {sink_len} must align with block size")
-    if block_table.dtype != torch.int32 or block_table.stride(-1) != 1 or seq_lens.dtype != torch.int32 or \
-            not seq_lens.is_contiguous() or rows.dtype != torch.int32 or rows.stride(-1) != 1 or counts.dtype != torch.int32 or \
-            not counts.is_contiguous():
-        raise TypeError("sink_window_rows: int32 block_table [B,max_blocks], seq_lens [B], rows [T,K], counts [T]")
-    b = seq_lens.numel()
-    t_min = b * q_len if query_start_loc is None else 1
-    if rows.shape[0] < t_min or counts.numel() < min(t_min, rows.shape[0]) or counts.numel() < rows.shape[0] or \
-            rows.shape[1] < sink_len + window or window < 1:
-        raise ValueError("sink_window_rows: rows [T, >= sink_len + window] and counts [T], T = batch * q_len tokens")
-    rc = lib.mla_sink_window_rows(block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),
-                                  query_start_loc.data_ptr() if query_start_loc is not None else None, b, q_len, sink_len,
-                                  window, page_size, num_pages, rows.data_ptr(), rows.stride(0), counts.data_ptr(),
-                                  _stream(rows))
-    _lib.check(rc, "mla_sink_window_rows")
 
 
 def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,

@@ -28,8 +28,7 @@ Pinning status (what checks each function beyond re-typing its formula lives in
                                   torch.nn.functional.scaled_dot_product_attention and the merge identity.
 * ``v_up_proj``                   restates attention/backends/mla.py:309-315; pinned by the identity-weight
                                   known answer of tests/unit/attention/backends/test_mla.py:190-259.
-* ``sink_decode``, ``sink_prefill``,
-  ``sink_window_rows``            restate the static-sink / sliding-window branches of
+* ``sink_decode``, ``sink_prefill``  restate the static-sink / sliding-window branches of
                                   attention/backends/mla.py:463-560 and :705-779 (two attentions with LSE and
                                   their merge; band mask pre_tokens = window - 1).  The reference holds no test
                                   of them; pinned by a per-token brute force over the union of the sink keys and
@@ -461,26 +460,6 @@ def sink_decode(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, s
     m = torch.maximum(l_s, l_n)
     w_s, w_n = torch.exp(l_s - m).unsqueeze(-1), torch.exp(l_n - m).unsqueeze(-1)
     return (o_s * w_s + o_n * w_n) / (w_s + w_n)
-
-
-def sink_window_rows(block_table, seq_lens, sink_len: int, window: Optional[int], q_len: int = 1, page: int = PAGE):
-    """The keys of ``sink_decode`` as flat cache rows per query token: the sink rows first, then the visible keys
-    of the sequence (the last ``window`` of them when a window is given), oldest first.  Returns rows
-    [T, sink_len + width] int32 (unused tail = 0) and counts [T] int32, width = window or the longest sequence."""
-    nb = len(seq_lens)
-    width = int(window) if window is not None else int(max(int(x) for x in seq_lens))
-    rows = torch.zeros(nb * q_len, sink_len + width, dtype=torch.int32)
-    counts = torch.zeros(nb * q_len, dtype=torch.int32)
-    for b in range(nb):
-        L = int(seq_lens[b])
-        for i in range(q_len):
-            n_vis = max(0, L - q_len + i + 1)
-            lo = max(0, n_vis - window) if window is not None else 0
-            pos = torch.cat([torch.arange(sink_len), sink_len + torch.arange(lo, n_vis)])
-            t = b * q_len + i
-            rows[t, :pos.numel()] = (block_table[b, pos // page].long() * page + pos % page).to(torch.int32)
-            counts[t] = pos.numel()
-    return rows, counts
 
 
 def insert_sink_rows(x: torch.Tensor, sink: torch.Tensor, cu_q: Sequence[int]) -> torch.Tensor:

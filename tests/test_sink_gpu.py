@@ -1,5 +1,5 @@
 """Static sink tokens with and without a sliding window on the GPU (reference attention/backends/mla.py:463-560 and
-:705-779) against the oracle: the row lists bit-exact, the attentions within the bf16 bar, at kernel level and through
+:705-779) against the oracle: the window plan bit-exact, the attentions within the bf16 bar, at kernel level and through
 NPUMLAImpl.forward."""
 from types import SimpleNamespace
 
@@ -19,65 +19,68 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, MEAN_REL = 2e-2, 2e-3
 
 
-# ---- the row lists (integer work: bit-exact) ------------------------------------------------------------------------
-@pytest.mark.parametrize("batch,lo,hi,sink_len,window,q_len", [
-    (5, 1, 700, 128, 64, 1), (4, 3, 900, 256, 300, 2), (3, 1, 40, 128, 1, 3), (6, 100, 2000, 0, 512, 1),
-    (2, 5000, 9000, 128, 4096, 2), (3, 10, 50, 384, 1000, 1)])
-def test_sink_window_rows_bit_exact(dev, batch, lo, hi, sink_len, window, q_len):
-    from omni_npu_amd import kernels as K
-    c, bt = _sink_case(batch, 2, lo, hi, sink_len, q_len, seed=batch * 7 + q_len)
-    want_rows, want_counts = O.sink_window_rows(bt, c["seq_lens"], sink_len, window, q_len)
-    t = batch * q_len
-    rows = torch.full((t, sink_len + window + 5), -7, dtype=torch.int32, device=dev)     # wider than needed, strided
-    counts = torch.full((t,), -7, dtype=torch.int32, device=dev)
-    K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), sink_len, window, c["nope"].shape[0], rows, counts, q_len=q_len)
-    rows, counts = rows.cpu(), counts.cpu()
-    assert torch.equal(counts, want_counts)
-    for i in range(t):
-        n = int(counts[i])
-        assert torch.equal(rows[i, :n], want_rows[i, :n]) and (rows[i, n:] == -7).all()    # nothing written past the count
-
-
-def test_sink_window_rows_ragged_query_lengths_and_errors(dev):
-    from omni_npu_amd import kernels as K
-    c, bt = _sink_case(3, 2, 50, 400, 128, 1, seed=2)
-    q_lens = [1, 3, 2]
-    qsl = torch.tensor([0, 1, 4, 6], dtype=torch.int32)
-    rows = torch.zeros(6, 128 + 32, dtype=torch.int32, device=dev)
-    counts = torch.zeros(6, dtype=torch.int32, device=dev)
-    K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), 128, 32, c["nope"].shape[0], rows, counts, q_len=3,
-                       query_start_loc=qsl.to(dev))
-    got_rows, got_counts = rows.cpu(), counts.cpu()
-    for b in range(3):
-        L, s = int(c["seq_lens"][b]), q_lens[b]
-        for i in range(s):
-            last = L - s + i
-            first = max(0, last - 31)
-            pos = torch.cat([torch.arange(128), 128 + torch.arange(first, last + 1)])
-            want = (bt[b, pos // 128].long() * 128 + pos % 128).to(torch.int32)
-            t = int(qsl[b]) + i
-            assert int(got_counts[t]) == pos.numel() and torch.equal(got_rows[t, :pos.numel()], want)
-    with pytest.raises(ValueError, match="must align with block size"):
-        K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), 100, 32, c["nope"].shape[0], rows, counts)
-    with pytest.raises(ValueError, match="sink_len \\+ window"):
-        K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), 128, 64, c["nope"].shape[0], rows, counts)
-
-
 # ---- decode at kernel level -------------------------------------------------------------------------------------
-@pytest.mark.parametrize("batch,heads,lo,hi,sink_len,window,q_len", [
-    (4, 128, 200, 3000, 128, 512, 1), (3, 128, 1, 100, 128, 16, 1), (3, 16, 300, 900, 256, 100, 2),
-    (2, 128, 2000, 5000, 128, 4096, 1), (2, 128, 600, 700, 128, 1, 3)])
-def test_sink_window_decode_matches_oracle(dev, batch, heads, lo, hi, sink_len, window, q_len):
+@pytest.mark.parametrize("batch,heads,lo,hi,sink_len,window,q_len,splits", [
+    (4, 128, 200, 3000, 128, 512, 1, None), (3, 128, 1, 100, 128, 16, 1, 1), (3, 16, 300, 900, 256, 100, 2, 3),
+    (2, 128, 2000, 5000, 128, 4096, 1, None), (2, 128, 600, 700, 128, 1, 3, 2), (5, 128, 1, 400, 0, 77, 2, None),
+    (6, 128, 30, 2000, 128, 31, 4, 4), (3, 128, 500, 9000, 384, 1000, 1, 8), (4, 128, 100, 160, 128, 129, 2, 1)])
+def test_dense_window_decode_matches_oracle(dev, batch, heads, lo, hi, sink_len, window, q_len, splits):
+    """The dense kernel over the shortened sequences (sink blocks + window blocks): plain and fused with W_UV."""
     from omni_npu_amd import kernels as K
-    c, bt = _sink_case(batch, heads, lo, hi, sink_len, q_len, seed=batch + heads + q_len)
+    c, bt = _sink_case(batch, heads, lo, hi, sink_len, q_len, seed=batch * 3 + heads + q_len + window)
     t = batch * q_len
-    rows = torch.zeros(t, sink_len + window, dtype=torch.int32, device=dev)
-    counts = torch.zeros(t, dtype=torch.int32, device=dev)
-    K.sink_window_rows(bt.to(dev), c["seq_lens"].to(dev), sink_len, window, c["nope"].shape[0], rows, counts, q_len=q_len)
     out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
-    K.sparse_decode(c["q_nope"].to(dev), c["q_rope"].to(dev), c["nope"].to(dev), c["rope"].to(dev), rows, counts, c["scale"], out)
+    lse = torch.full((t, heads), float("nan"), dtype=torch.float32, device=dev)
+    g = {k: c[k].to(dev) for k in ("q_nope", "q_rope", "nope", "rope", "seq_lens")}
+    K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], bt.to(dev), g["seq_lens"], c["scale"], out, q_len=q_len,
+             lse_out=lse, num_splits=splits, sink_len=sink_len, window=window)
     ref = O.sink_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], bt, c["seq_lens"], sink_len, c["scale"], window)
     attn_close(out, ref, MAX_ABS, MEAN_REL)
+    assert torch.isfinite(lse).all()
+    if heads == 128:
+        gw = torch.Generator().manual_seed(1)
+        w_uv = (torch.randn(heads, 512, 128, generator=gw) * 0.05).bfloat16()
+        out_v = torch.full((t, heads * 128), float("nan"), dtype=torch.bfloat16, device=dev)
+        K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], bt.to(dev), g["seq_lens"], c["scale"], out_v, q_len=q_len,
+                 num_splits=splits, sink_len=sink_len, window=window, w_uv=w_uv.to(dev))
+        ref_v = torch.einsum("tnl,nlv->tnv", ref, w_uv.float()).reshape(t, -1)
+        attn_close(out_v, ref_v, 3e-2, 8e-3)
+
+
+def test_dense_window_decode_ragged_queries_and_argument_errors(dev):
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(3, 128, 300, 1500, 128, 1, seed=8)
+    q_lens = [1, 3, 2]
+    qsl = [0, 1, 4, 6]
+    g0 = torch.Generator().manual_seed(4)
+    qn, qr = torch.randn(6, 128, 512, generator=g0).bfloat16(), torch.randn(6, 128, 64, generator=g0).bfloat16()
+    out = torch.full((6, 128, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    args = (qn.to(dev), qr.to(dev), c["nope"].to(dev), c["rope"].to(dev), bt.to(dev), c["seq_lens"].to(dev), c["scale"], out)
+    K.decode(*args, q_len=3, query_start_loc=torch.tensor(qsl, dtype=torch.int32, device=dev), sink_len=128, window=200)
+    ref = O.sink_decode(qn, qr, c["nope"], c["rope"], bt, c["seq_lens"], 128, c["scale"], 200, query_start_loc=qsl)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+    with pytest.raises(ValueError, match="whole number of pages"):
+        K.decode(*args, q_len=2, sink_len=100, window=64)
+    with pytest.raises(ValueError, match="sink_len goes with window"):
+        K.decode(*args, q_len=2, sink_len=128)
+    with pytest.raises(ValueError, match="both phases"):
+        K.decode(*args, q_len=2, sink_len=128, window=64, phase="split")
+
+
+def test_window_plan_bit_exact(dev):
+    from omni_npu_amd import _lib
+    lib = _lib.load()
+    lens = torch.tensor([0, 1, 31, 32, 33, 100, 128, 129, 4096, 4097, 5000, 70000], dtype=torch.int32)
+    for q_len, sink_len, window in [(1, 128, 64), (2, 128, 100), (4, 0, 1), (1, 256, 4096), (3, 128, 33)]:
+        short = torch.full((12,), -1, dtype=torch.int32, device=dev)
+        skip = torch.full((12,), -1, dtype=torch.int32, device=dev)
+        rc = lib.mla_window_plan(lens.to(dev).data_ptr(), None, 12, q_len, sink_len, window, short.data_ptr(), skip.data_ptr(),
+                                 torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        for i, L in enumerate(lens.tolist()):
+            lo0 = max(0, max(0, L - q_len + 1) - window)
+            assert int(skip[i]) == lo0 // 32
+            assert int(short[i]) == (sink_len + L - 32 * (lo0 // 32) if L > 0 else 0)
 
 
 def test_sink_decode_without_window_is_the_dense_kernel_over_the_longer_table(dev):

@@ -72,21 +72,6 @@ def test_sink_len_must_be_whole_pages():
         O.sink_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], bt, c["seq_lens"], 100, c["scale"])
 
 
-@pytest.mark.parametrize("window,q_len", [(None, 1), (16, 1), (5, 3), (1, 2)])
-def test_sink_window_rows_name_exactly_the_union(window, q_len):
-    c, bt = _sink_case(3, 2, 4, 300, 128, q_len, seed=9)
-    rows, counts = O.sink_window_rows(bt, c["seq_lens"], 128, window, q_len)
-    for b in range(3):
-        L = int(c["seq_lens"][b])
-        for i in range(q_len):
-            last = L - q_len + i
-            first = 0 if window is None else max(0, last - window + 1)
-            want = [int(bt[b, 0]) * 128 + j for j in range(128)]
-            want += [int(bt[b, 1 + j // 128]) * 128 + j % 128 for j in range(first, last + 1)]
-            t = b * q_len + i
-            assert int(counts[t]) == len(want) and rows[t, :len(want)].tolist() == want
-
-
 def test_windowed_varlen_attention_matches_sdpa_with_a_band_mask():
     g = torch.Generator().manual_seed(2)
     n, sq, sk, w = 3, 37, 50, 9
