@@ -441,6 +441,72 @@ def bench_epilogue(K, dev, args):
     }
 
 
+def bench_window(K, dev, args):
+    """Decode with static sink tokens and a sliding window (the reference's variant of attention/backends/mla.py:705-779):
+    B=64, 128 heads, 4096-8192 keys behind a 128-key sink, window 4096.  One step = window plan + dense split kernel over
+    the shortened sequences + merge, replayed as a HIP graph; the split kernel is also timed alone."""
+    import time
+    from oracle import mla_oracle as O
+    B, N, sink, win = 64, 128, 128, 4096
+    case = build_workload(args.seed, B, N, 4096, 8192, 1)
+    nsb = sink // 128
+    nblk = case["nope"].shape[0]
+    gen = torch.Generator().manual_seed(args.seed + 2)
+    sink_nope, sink_rope = torch.randn(nsb, 128, 512, generator=gen).bfloat16(), torch.randn(nsb, 128, 64, generator=gen).bfloat16()
+    nope_c, rope_c = torch.cat([case["nope"], sink_nope]), torch.cat([case["rope"], sink_rope])
+    bt_c = torch.cat([torch.arange(nblk, nblk + nsb, dtype=torch.int32).view(1, -1).expand(B, -1), case["block_table"]], 1).contiguous()
+    nope, rope, bt, lens = nope_c.to(dev), rope_c.to(dev), bt_c.to(dev), case["seq_lens"].to(dev)
+    qn, qr = case["q_nope"].to(dev), case["q_rope"].to(dev)
+    out = torch.empty(B, N, 512, dtype=torch.bfloat16, device=dev)
+    splits = args.splits or None
+
+    def step():
+        K.decode(qn, qr, nope, rope, bt, lens, case["scale"], out, num_splits=splits, sink_len=sink, window=win)
+
+    for _ in range(max(args.warmup, 2)):
+        step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(args.steps):
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        ts.append(a.elapsed_time(e) * 1e3)
+    t_step = sum(ts) / len(ts)
+    visible = int((torch.clamp(case["seq_lens"], max=win) + sink).sum())
+    alg_bytes = visible * 1152 + B * N * 576 * 2 + B * N * 512 * 2
+    sample = 4
+    t0 = time.perf_counter()
+    ref = O.sink_decode(case["q_nope"][:sample], case["q_rope"][:sample], nope_c, rope_c, bt_c[:sample], case["seq_lens"][:sample],
+                        sink, case["scale"], win)
+    cpu_s = time.perf_counter() - t0
+    err = (out[:sample].float().cpu() - ref).abs().max().item()
+    return {
+        "metric": "MLA decode with static sink + sliding window, us/layer (B=64, ctx 4k-8k, sink 128, window 4096, 128 heads, bf16)",
+        "value": round(t_step, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "static sink tokens + sliding window decode (plan + split + merge, graph replay)", "batch": B,
+                   "heads": N, "sink_len": sink, "window": win, "visible_keys": visible, "seed": args.seed},
+        "roofline": {"kernel": "plan + mla_decode_v2_kernel<false, true> + merge (whole step)", "bound": "hbm",
+                     "achieved": round(alg_bytes / t_step / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(alg_bytes / t_step / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": alg_bytes},
+        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", "cores": torch.get_num_threads(),
+                         "kind": "port", "sample": f"oracle sink_decode (torch fp32) of {sample} of {B} sequences, scaled by sequence count",
+                         "gpu_vs_oracle_max_abs": err},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -460,7 +526,7 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue", "window"],
                     help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
@@ -494,6 +560,9 @@ def main():
         return
     if args.workload == "epilogue":
         print(json.dumps(bench_epilogue(K, dev, args)))
+        return
+    if args.workload == "window":
+        print(json.dumps(bench_window(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len
