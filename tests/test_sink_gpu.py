@@ -284,3 +284,75 @@ def test_graph_replay_of_the_sink_decode_sees_new_lengths(dev, window):
             assert torch.equal(got, eager), f"replay {trial} differs from eager"
             seen.append(got)
     assert not torch.equal(seen[0], seen[1])
+
+
+# ---- seeded sweeps --------------------------------------------------------------------------------------------------
+def _window_cases(n, seed):
+    import random
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        q_len = rng.choice([1, 1, 2, 3, 4])
+        heads = rng.choice([8, 16, 64, 128, 128])
+        batch = rng.randint(1, 7)
+        sink_len = rng.choice([0, 128, 128, 256])
+        window = rng.choice([1, 2, 31, 32, 33, 63, 64, 100, 128, 129, 500, 1000])
+        lo = rng.choice([q_len, q_len, 31, 32, 33, 64, 100, 129, 700])
+        hi = lo + rng.choice([0, 1, 35, 300, 1500])
+        splits = rng.choice([None, 1, 2, 3, 7, 30])
+        out.append((i, batch, heads, q_len, sink_len, window, lo, hi, splits))
+    return out
+
+
+@pytest.mark.parametrize("i,batch,heads,q_len,sink_len,window,lo,hi,splits", _window_cases(48, seed=77))
+def test_dense_window_decode_random_shapes(dev, i, batch, heads, q_len, sink_len, window, lo, hi, splits):
+    """Window starts at every offset inside a 32-key block, windows shorter and longer than the sequences, sequences no
+    longer than their query tokens, with and without a sink, split counts from one to more chunks than there is work."""
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(batch, heads, lo, hi, sink_len, q_len, seed=3000 + i)
+    t = batch * q_len
+    out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.full((t, heads), float("nan"), dtype=torch.float32, device=dev)
+    K.decode(c["q_nope"].to(dev), c["q_rope"].to(dev), c["nope"].to(dev), c["rope"].to(dev), bt.to(dev), c["seq_lens"].to(dev),
+             c["scale"], out, q_len=q_len, lse_out=lse, num_splits=splits, sink_len=sink_len, window=window)
+    if sink_len:
+        ref = O.sink_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], bt, c["seq_lens"], sink_len, c["scale"], window)
+    else:
+        ref = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], bt, c["seq_lens"], c["scale"], window=window)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+    assert torch.isfinite(lse).all()
+
+
+def _prefill_window_cases(n, seed):
+    import random
+    rng = random.Random(seed)
+    out = []
+    for i in range(n):
+        nseq = rng.randint(1, 3)
+        q_lens = [rng.choice([1, 5, 31, 32, 33, 127, 128, 129, 300, 700]) for _ in range(nseq)]
+        k_extra = [rng.choice([0, 0, 1, 40, 200]) for _ in range(nseq)]
+        window = rng.choice([1, 2, 31, 32, 33, 64, 65, 127, 128, 129, 400, 5000])
+        heads = rng.choice([1, 2, 8])
+        out.append((i, q_lens, k_extra, window, heads))
+    return out
+
+
+@pytest.mark.parametrize("i,q_lens,k_extra,window,heads", _prefill_window_cases(24, seed=5))
+def test_prefill_window_random_shapes(dev, i, q_lens, k_extra, window, heads):
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(4000 + i)
+    k_lens = [a + b for a, b in zip(q_lens, k_extra)]
+    cu_q = [0] + torch.tensor(q_lens).cumsum(0).tolist()
+    cu_k = [0] + torch.tensor(k_lens).cumsum(0).tolist()
+    t, tk = cu_q[-1], cu_k[-1]
+    qn, qp = torch.randn(t, heads, 128, generator=g).bfloat16(), torch.randn(t, heads, 64, generator=g).bfloat16()
+    kn, kp = torch.randn(tk, heads, 128, generator=g).bfloat16(), torch.randn(tk, 64, generator=g).bfloat16()
+    v = torch.randn(tk, heads, 128, generator=g).bfloat16()
+    scale = 192 ** -0.5
+    out = torch.full((t, heads, 128), float("nan"), dtype=torch.float32, device=dev)
+    lse = torch.full((t, heads), float("nan"), dtype=torch.float32, device=dev)
+    K.prefill_varlen(qn.to(dev), qp.to(dev), kn.to(dev), kp.to(dev), v.to(dev), torch.tensor(cu_q, dtype=torch.int32, device=dev),
+                     torch.tensor(cu_k, dtype=torch.int32, device=dev), max(q_lens), scale, True, out, lse, window=window)
+    ref, ref_lse = O.attention_varlen(qn, qp, kn, kp, v, cu_q, cu_k, scale, True, window=window)
+    attn_close(out, ref, MAX_ABS, MEAN_REL)
+    assert (lse.cpu() - ref_lse).abs().max() < 2e-2
