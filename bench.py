@@ -264,7 +264,7 @@ def bench_fp8(K, dev, args):
         "config": {"workload": "configs[4]: fp8 cache, high-batch MTP decode", "batch": B, "heads": N, "q_len": QL,
                    "seq_lens": "uniform[16384,32768]", "sum_seq_len": sum_l, "kv_splits": splits, "seed": args.seed},
         "step_us": {"hip_graph_replay": round(t_graph, 1), "eager_launches": round(t_eager, 1)},
-        "roofline": {"kernel": "mla_decode_v2_fp8_kernel", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
+        "roofline": {"kernel": "mla_decode_v2_fp8_kernel<false>", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                      # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)

@@ -257,6 +257,16 @@ int mla_decode_bf16_window_split(const void* q_nope, int64_t qn_stride_t, int64_
                                  int32_t sink_len, int32_t window, float scale, void* workspace, size_t workspace_bytes,
                                  int32_t num_splits, mlahip_stream_t stream);
 
+/* The same split phase over the fp8 block-scaled cache of mla_decode_fp8 (no counterpart call in the reference, which has
+ * no fp8 latent cache; the variant is the one of mla.py:705-779). */
+int mla_decode_fp8_window_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                int64_t qr_stride_t, int64_t qr_stride_h, const void* cache, int64_t page_stride_bytes,
+                                int64_t row_stride_bytes, int64_t num_pages, const int32_t* block_table, int64_t bt_stride,
+                                int32_t max_blocks, const int32_t* short_lens, const int32_t* skip,
+                                const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                                int32_t sink_len, int32_t window, float scale, void* workspace, size_t workspace_bytes,
+                                int32_t num_splits, mlahip_stream_t stream);
+
 int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
                            int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,
                            int64_t nope_row_stride, const void* rope_cache, int64_t rope_page_stride,

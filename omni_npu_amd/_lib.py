@@ -37,6 +37,8 @@ SIGNATURES = {
     "mla_window_plan": (c_int32, [P, P, I32, I32, I32, I32, P, P, P]),
     "mla_decode_bf16_window_split": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, P,
                                                I32, I32, I32, I32, I32, F32, P, SZ, I32, P]),
+    "mla_decode_fp8_window_split": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, P, I32, I32, I32,
+                                              I32, I32, F32, P, SZ, I32, P]),
     "mla_splitkv_reduce": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, P, I64, I64, P, P]),
     "mla_splitkv_reduce_vup": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, I32, P, I64, I64, P, I64, I64, P]),
     "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,

@@ -346,8 +346,6 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         blocks between the sink and the window left out (kernels.decode(..., sink_len=, window=))."""
         if self.sink_len % K.PAGE != 0:
             raise ValueError(f"sink_len {self.sink_len} must align with block size")
-        if self.fp8_cache and self.sliding_window is not None:
-            raise NotImplementedError("static sink tokens with a sliding window over the fp8 cache are not implemented")
         t, dev = ql_nope.shape[0], ql_nope.device
         o = None
         if proj_out is None:
@@ -362,8 +360,11 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
                 K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens + self.sink_len, self.scale, out,
                          **kw)
             return o
-        K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens, self.scale, out, q_len=d.q_len,
-                 query_start_loc=d.query_start_loc, w_uv=w_uv, sink_len=self.sink_len, window=self.sliding_window)
+        kw = dict(q_len=d.q_len, query_start_loc=d.query_start_loc, w_uv=w_uv, sink_len=self.sink_len, window=self.sliding_window)
+        if self.fp8_cache:
+            K.decode_fp8(ql_nope, q_pe, kv_cache[0], d.block_table, d.seq_lens, self.scale, out, **kw)
+        else:
+            K.decode(ql_nope, q_pe, kv_cache[0], kv_cache[1], d.block_table, d.seq_lens, self.scale, out, **kw)
         return o
 
     def forward(self, layer, q: torch.Tensor, k_c_normed: torch.Tensor, k_pe: torch.Tensor,

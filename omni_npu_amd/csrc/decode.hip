@@ -155,6 +155,26 @@ extern "C" int mla_decode_bf16_window_split(const void* q_nope, int64_t qn_strid
                            window);
 }
 
+// The windowed split phase over the fp8 block-scaled cache (same plan, same merge).
+extern "C" int mla_decode_fp8_window_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                           int64_t qr_stride_t, int64_t qr_stride_h, const void* cache, int64_t page_stride_bytes,
+                                           int64_t row_stride_bytes, int64_t num_pages, const int32_t* block_table,
+                                           int64_t bt_stride, int32_t max_blocks, const int32_t* short_lens, const int32_t* skip,
+                                           const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                                           int32_t sink_len, int32_t window, float scale, void* workspace,
+                                           size_t workspace_bytes, int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(cache && block_table && skip, MLA_ERR_NULL, "mla_decode_fp8_window_split: null pointer argument");
+  MLA_REQUIRE(row_stride_bytes == kFp8RowB && page_stride_bytes >= (int64_t)kPage * kFp8RowB && page_stride_bytes % 16 == 0,
+              MLA_ERR_UNSUPPORTED, "mla_decode_fp8_window_split: rows must be exactly 656 bytes apart, pages 128 rows (got %lld / %lld)",
+              (long long)row_stride_bytes, (long long)page_stride_bytes);
+  MLA_REQUIRE(sink_len >= 0 && sink_len % kPage == 0 && window >= 1, MLA_ERR_SHAPE,
+              "mla_decode_fp8_window_split: sink_len=%d window=%d", sink_len, window);
+  return decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, cache, page_stride_bytes,
+                           kFp8RowB + 8, cache, page_stride_bytes, kFp8RowB + 8, num_pages, block_table, bt_stride, max_blocks,
+                           short_lens, query_start_loc, batch, max_q_len, num_heads, scale, workspace, workspace_bytes,
+                           num_splits, nullptr, 0, kPage, true, stream, skip, sink_len, window);
+}
+
 // Phase 2: N-way log-sum-exp merge of the workspace partials into the bf16 output (and optional lse).
 extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes, const int32_t* seq_lens,
                                   const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,

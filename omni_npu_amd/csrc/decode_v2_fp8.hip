@@ -93,6 +93,10 @@ __device__ __forceinline__ int wave_incl_scan_i32(int v, int lane) {
 
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
+// kWindow: static sink keys followed by a sliding window, as in the bf16 kernel: the sequence is walked without the
+// blocks between the sink and the window (block v at or behind the first non-sink block is block v + skip of the cache),
+// and the blocks right behind the sink mask the keys older than a row's window.
+template <bool kWindow>
 __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV2Params p) {
   constexpr bool kSparse = false;
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -180,6 +184,8 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV
   const int head = row - t_local * p.num_heads;
   int limit = row_ok ? (L - qlen + t_local + 1) : 0;         // keys [0, limit) are visible to this row
   limit = limit < 0 ? 0 : limit;
+  const int win_skip = kWindow ? p.win_skip[b] : 0;
+  const int win_blk0 = kWindow ? p.win_sink / kBlk : 0;
   const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
 
   if (grp * 128 >= rows) {
@@ -217,10 +223,15 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV
     const int last = L - 1 - blk * kBlk;                      // last valid row of the block (>= 0)
     const uint32_t raw = lds0 + kRawOff + (blk & 1) * kRawStageB;
     const uint32_t rbuf = lds0 + kV2RopeOff + (blk % 3) * kV2RopeBufB;
-    const int page = blk >> 2;
+    const int cblk = blk + (kWindow && blk >= win_blk0 ? win_skip : 0);   // block of the cache
+    const int page = cblk >> 2;
     if (blk == blk_begin) { page_cur = page; pg_cur = load_page(page); pg_nxt = load_page(page + 1); }
-    else if (page != page_cur) { page_cur = page; pg_cur = pg_nxt; pg_nxt = load_page(page + 1); }
-    const char* src = (const char*)p.cache8 + pg_cur * p.c8_sp + (int64_t)(blk & 3) * kBlk * kFp8RowBytes;
+    else if (page != page_cur) {
+      pg_cur = (kWindow && page != page_cur + 1) ? load_page(page) : pg_nxt;   // the jump from the sink to the window
+      page_cur = page;
+      pg_nxt = load_page(page + 1);
+    }
+    const char* src = (const char*)p.cache8 + pg_cur * p.c8_sp + (int64_t)(cblk & 3) * kBlk * kFp8RowBytes;
     if (last >= kBlk - 1) {
 #pragma unroll
       for (int j = 0; j < 5; j++)
@@ -409,14 +420,19 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV
   // After the steps: the last blocks of a sequence hold keys that some rows must not see (causal multi-token queries,
   // rows past the end of the sequence); only those blocks pay for the masking.  Then P^T and the flag go to LDS.
   auto softmax_finish = [&](int blk, f32x16& s, SoftmaxState& st) {
-    if ((blk + 1) * kBlk > L - p.max_q_len + 1) {
+    bool front = false;                                       // window: a block with keys older than some row's window
+    if constexpr (kWindow) front = blk >= win_blk0 && blk * kBlk < L - p.win_size;
+    if ((blk + 1) * kBlk > L - p.max_q_len + 1 || front) {
       int blk_s = blk;                                        // opaque: keeps the compiler from carrying `rel` as a loop
       asm volatile("" : "+s"(blk_s));                         // variable of its own (one more register across the loop)
       const int rel = limit - blk_s * kBlk - ((lane_now() >> 3) & 4);   // score r is visible iff 8*(r/4) + r%4 < rel
+      // ... and, behind the sink, iff it is one of the row's newest win_size keys: 8*(r/4) + r%4 >= rel - win_size
+      const int rel_lo = (kWindow && blk >= win_blk0) ? rel - p.win_size : -64;
       st.psum = 0.f;
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        s[r] = (8 * (r >> 2) + (r & 3)) < rel ? s[r] : 0.f;
+        const int kpos = 8 * (r >> 2) + (r & 3);
+        s[r] = (kpos < rel && kpos >= rel_lo) ? s[r] : 0.f;
         st.psum += s[r];
       }
 #pragma unroll
@@ -631,9 +647,11 @@ __global__ __launch_bounds__(256, 1) void mla_decode_v2_fp8_kernel(const DecodeV
 }  // namespace f8v2
 
 int launch_decode_v2_fp8(const DecodeV2Params& p, dim3 grid, hipStream_t stream) {
-  const int rc = ensure_dynamic_lds((const void*)f8v2::mla_decode_v2_fp8_kernel, f8v2::kV2LdsB, "mla_decode_fp8");
+  const void* kernel = p.win_skip ? (const void*)f8v2::mla_decode_v2_fp8_kernel<true> : (const void*)f8v2::mla_decode_v2_fp8_kernel<false>;
+  const int rc = ensure_dynamic_lds(kernel, f8v2::kV2LdsB, "mla_decode_fp8");
   if (rc != MLA_OK) return rc;
-  hipLaunchKernelGGL(f8v2::mla_decode_v2_fp8_kernel, grid, dim3(256), f8v2::kV2LdsB, stream, p);
+  if (p.win_skip) hipLaunchKernelGGL(f8v2::mla_decode_v2_fp8_kernel<true>, grid, dim3(256), f8v2::kV2LdsB, stream, p);
+  else hipLaunchKernelGGL(f8v2::mla_decode_v2_fp8_kernel<false>, grid, dim3(256), f8v2::kV2LdsB, stream, p);
   return check_launch("mla_decode_v2_fp8_kernel");
 }
 

@@ -633,9 +633,15 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
                seq_lens: torch.Tensor, scale: float, out: torch.Tensor, q_len: int = 1,
                query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
                num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
-               workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None) -> torch.Tensor:
+               workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None, sink_len: int = 0,
+               window: Optional[int] = None) -> torch.Tensor:
     """Absorbed-MLA paged decode over the fp8 block-scaled cache (uint8 [num_blocks, 128, 656], see cache_write_fp8).
-    With ``w_uv`` (bf16 [N,512,128]) the value up-projection is fused into the merge: out is [T, N*128] / [T,N,128]."""
+    With ``w_uv`` (bf16 [N,512,128]) the value up-projection is fused into the merge: out is [T, N*128] / [T,N,128].
+    ``sink_len`` / ``window``: static sink keys + sliding window as in decode()."""
+    if window is None and sink_len:
+        raise ValueError("decode_fp8: sink_len goes with window (without one, pass seq_lens + sink_len)")
+    if window is not None and (window < 1 or sink_len < 0 or sink_len % PAGE != 0):
+        raise ValueError(f"decode_fp8: window {window} must be positive and sink_len {sink_len} a whole number of pages")
     _need_cuda(q_nope, q_rope, cache, block_table, seq_lens, out)
     lib = _lib.load()
     t, n, _ = q_nope.shape
@@ -658,10 +664,35 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
         raise ValueError(f"decode_fp8: {t} query tokens != batch {b} x q_len {q_len}")
     if max_seq_len is None:
         max_seq_len = block_table.shape[1] * PAGE
+    if window is not None:
+        max_seq_len = min(max_seq_len, sink_len + window + 32 + q_len)         # keys of a shortened sequence
     if num_splits is None:
         num_splits = default_num_splits(b, q_len, n, max_seq_len)
     need = lib.mla_decode_workspace_bytes(b, q_len, n, num_splits)
     ws = workspace if workspace is not None else _workspace(q_nope.device, need)
+    if window is not None:
+        if not seq_lens.is_contiguous():
+            seq_lens = seq_lens.contiguous()
+        st = _stream(q_nope)
+        qsl = query_start_loc.data_ptr() if query_start_loc is not None else None
+        ws_args = (ws.data_ptr(), ws.numel() * ws.element_size())
+        plan = torch.empty(2, b, dtype=torch.int32, device=q_nope.device)  # shortened lengths, blocks left out
+        short, skip = plan[0], plan[1]
+        _lib.check(lib.mla_window_plan(seq_lens.data_ptr(), qsl, b, q_len, sink_len, window, short.data_ptr(),
+                                       skip.data_ptr(), st), "mla_window_plan")
+        rc = lib.mla_decode_fp8_window_split(
+            q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
+            cache.data_ptr(), cache.stride(0), cache.stride(1), cache.shape[0], block_table.data_ptr(), block_table.stride(0),
+            block_table.shape[1], short.data_ptr(), skip.data_ptr(), qsl, b, q_len, n, sink_len, window, float(scale),
+            *ws_args, num_splits, st)
+        _lib.check(rc, "mla_decode_fp8_window_split")
+        if o3 is not None:
+            _reduce_vup(lib, ws_args, short, qsl, b, q_len, n, num_splits, t, w_uv, o3, st)
+        else:
+            rc = lib.mla_splitkv_reduce(*ws_args, short.data_ptr(), qsl, b, q_len, n, num_splits, out.data_ptr(), out.stride(0),
+                                        out.stride(1), lse_out.data_ptr() if lse_out is not None else None, st)
+            _lib.check(rc, "mla_splitkv_reduce")
+        return out
     rc = lib.mla_decode_fp8(q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0),
                             q_rope.stride(1), cache.data_ptr(), cache.stride(0), cache.stride(1), cache.shape[0],
                             block_table.data_ptr(), block_table.stride(0), block_table.shape[1], seq_lens.data_ptr(),

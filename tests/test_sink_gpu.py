@@ -199,8 +199,7 @@ def test_impl_prefill_with_sink_tokens(dev, window):
 
 
 def test_impl_decode_with_sink_tokens_over_the_fp8_cache(dev):
-    """Without a window the sink pages are just the first pages of the table, for the fp8 cache as for the bf16 one; the
-    oracle reads the dequantised cache.  With a window the fp8 cache is rejected."""
+    """Sink tokens over the fp8 cache, without and with a window; the oracle reads the dequantised cache."""
     from omni_npu_amd import kernels as K
     g = torch.Generator().manual_seed(77)
     n, sink_len, nsb = 128, 128, 1
@@ -233,10 +232,38 @@ def test_impl_decode_with_sink_tokens_over_the_fp8_cache(dev):
     out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
     impl.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), (cache,), meta, output=out)
     attn_close(out, ref, 6e-2, 1.2e-2)
+    # ... and with a window
     impl_w, _ = _mk_impl(mla.NPUMLAImpl, n, dev, kv_cache_dtype="fp8", sliding_window=64)
     impl_w.update_sink_kv(rope[0].to(dev), nope[0].to(dev))
-    with pytest.raises(NotImplementedError, match="sliding window over the fp8 cache"):
-        impl_w.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), (cache,), meta, output=out)
+    o_w = O.sink_decode(ql, q[..., 128:].float(), nope_deq, rope, common.block_table_tensor.cpu(), common.seq_lens_cpu, sink_len,
+                        impl.scale, 64, query_start_loc=common.query_start_loc_cpu.tolist())
+    ref_w = torch.einsum("tnl,lnv->tnv", o_w, kvw[..., 128:]).reshape(t, -1)
+    out_w = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    impl_w.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), (cache,), meta, output=out_w)
+    attn_close(out_w, ref_w, 6e-2, 1.2e-2)
+
+
+@pytest.mark.parametrize("batch,heads,lo,hi,sink_len,window,q_len,splits", [
+    (4, 128, 200, 3000, 128, 512, 1, None), (3, 128, 1, 100, 128, 16, 1, 1), (3, 16, 300, 900, 256, 100, 2, 3),
+    (2, 128, 600, 700, 128, 1, 3, 2), (5, 128, 1, 400, 0, 77, 2, None), (6, 64, 30, 2000, 128, 31, 4, 4),
+    (3, 128, 500, 9000, 384, 1000, 1, 8), (4, 128, 100, 160, 128, 129, 2, 1)])
+def test_fp8_window_decode_matches_oracle(dev, batch, heads, lo, hi, sink_len, window, q_len, splits):
+    from omni_npu_amd import kernels as K
+    c, bt = _sink_case(batch, heads, lo, hi, sink_len, q_len, seed=batch * 5 + heads + q_len + window)
+    t = batch * q_len
+    q8, sc = O.fp8_quant_block(c["nope"].float())
+    deq = O.fp8_dequant_block(q8, sc)
+    nblk = c["nope"].shape[0]
+    cache = torch.zeros(nblk, 128, K.FP8_ROW_BYTES, dtype=torch.uint8, device=dev)
+    K.cache_write_fp8(c["nope"].view(-1, 512).to(dev), c["rope"].view(-1, 64).to(dev), torch.arange(nblk * 128, device=dev), cache)
+    out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.decode_fp8(c["q_nope"].to(dev), c["q_rope"].to(dev), cache, bt.to(dev), c["seq_lens"].to(dev), c["scale"], out, q_len=q_len,
+                 num_splits=splits, sink_len=sink_len, window=window)
+    if sink_len:
+        ref = O.sink_decode(c["q_nope"], c["q_rope"], deq, c["rope"], bt, c["seq_lens"], sink_len, c["scale"], window)
+    else:
+        ref = O.absorbed_decode(c["q_nope"], c["q_rope"], deq, c["rope"], bt, c["seq_lens"], c["scale"], window=window)
+    attn_close(out, ref, 6e-2, 6e-3)
 
 
 @pytest.mark.parametrize("window", [None, 200])
