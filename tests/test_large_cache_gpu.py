@@ -60,6 +60,13 @@ def test_bf16_cache_beyond_4gib_write_decode_sparse_gather(dev):
     ref = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], c["scale"])
     attn_close(out, ref, MAX_ABS, MEAN_REL)
 
+    # the same with a sliding window of 100 keys behind the first page taken as the sink (the blocks in between are skipped)
+    out_w = torch.full((4, 128, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.decode(c["q_nope"].to(dev), c["q_rope"].to(dev), nope, rope, bt_far.to(dev), (c["seq_lens"] - 128).to(dev), c["scale"],
+             out_w, q_len=1, num_splits=2, sink_len=128, window=100)
+    ref_w = O.sink_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"] - 128, 128, c["scale"], 100)
+    attn_close(out_w, ref_w, MAX_ABS, MEAN_REL)
+
     # sparse decode: every third position of each sequence, named by flat cache rows of the big allocation
     k = 320
     idx = torch.full((4, k), -1, dtype=torch.int32)
