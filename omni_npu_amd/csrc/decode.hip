@@ -84,6 +84,8 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   // one workgroup per (balanced chunk, group of 128 query rows)
   const dim3 grid((unsigned)(batch * num_splits), 1, (unsigned)((r_max + kRowsPerWg - 1) / kRowsPerWg));
   if (fp8) return launch_decode_v2_fp8(v, grid, stream);
+  static const bool use_v2 = getenv("MLA_DECODE_V2") != nullptr;
+  if (!use_v2) return launch_decode_v3(v, sparse_rows != nullptr, grid, stream);
   if (win_skip) return launch_decode_v2_window(v, grid, stream);
   return launch_decode_v2(v, sparse_rows != nullptr, grid, stream);
 }

@@ -52,6 +52,8 @@ int launch_reduce_vup(const ChunkReduceParams& r, const void* w_uv, int64_t w_st
 int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
 // The dense kernel with a sink and a sliding window (p.win_skip set).
 int launch_decode_v2_window(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
+// The eight-wavefront kernel (decode_v3.hip): dense, row-list (sparse) and, with p.win_skip set, sink + window.
+int launch_decode_v3(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
 // Launches mla_decode_v2_fp8_kernel (decode_v2_fp8.hip) over p.cache8.
 int launch_decode_v2_fp8(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
 

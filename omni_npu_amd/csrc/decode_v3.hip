@@ -1,0 +1,833 @@
+// Absorbed-MLA paged decode over the bf16 cache: split-KV kernel with eight wavefronts per workgroup (two per SIMD).
+//
+// Contract: the reference's decode call (src/omni_npu/attention/backends/mla.py:781-804); dense paged source, per-token
+// row lists (src/omni_npu/attention/backends/dsa.py:259-291) and the sink + sliding-window variant
+// (src/omni_npu/attention/backends/mla.py:705-779) are instantiations of one kernel.
+//
+// A query row is a (token, head) pair; a workgroup handles 128 rows and streams 32-key blocks of the latent cache
+// through LDS.  With one 512-register wavefront per SIMD every instruction of the block loop is issued in series and the
+// matrix pipe idles during each LDS read, softmax instruction and wait; with two 256-register wavefronts per SIMD the
+// other wavefront's MFMAs fill those gaps, and the CU's LDS read rate doubles (a wavefront cannot draw more than ~32 B
+// per clock by itself).  The register file holds the same data either way: 256 KiB of fp32 output accumulators and
+// 144 KiB of query, spread over eight wavefronts:
+//   S^T = K Q^T      wave w owns query rows 16w..16w+15 (its 576-wide query stays in 72 registers) and all 32 keys of a
+//                    block: 36 v_mfma_f32_16x16x32_bf16, one 16-byte LDS row read (the K fragment) each;
+//   O^T += V^T P^T   wave w owns output columns [64w, 64w+64) for ALL 128 rows (128 accumulation registers): 16
+//                    v_mfma_f32_32x32x16_bf16 per block, V^T fragments by transposed LDS reads of the same rows.
+// P^T (bf16) travels through LDS once per block (8 KiB, double buffered), one workgroup barrier per block.
+//
+// Pipeline:  body i = [barrier] QK(i+1) with the copies of block i+3 spread between its MFMAs | PV(i) with the softmax of
+// block i+1 cut into steps between the MFMA groups | publish P(i+1).
+//
+// Softmax with a fixed reference (no accumulator rescaling: vector ALU instructions cannot touch the accumulation
+// registers): every row fixes m_ref at the largest score of its first block and uses P = exp2(s - m_ref) from then on;
+// bf16 and fp32 share an exponent range, so P may grow to 2^100 without loss of relative precision.  A score more than
+// 100 (log2) above the reference raises a flag; the workgroup then restarts its segment with the maxima seen so far.
+// In the steady state nothing crosses lanes: the four lanes that hold a row's scores keep their own sums and candidates
+// for the row's most probable key, and combine them in the epilogue.
+// Partials: normalised fp16 through an LDS transpose, fp32 natural-log LSE, and the dominant-key correction record that
+// mla_chunk_reduce_kernel applies (the bf16 rounding of the largest probability is the biggest single error of P.V).
+#include "decode_v2_params.hpp"
+#include <type_traits>
+#include <cstdlib>
+
+namespace mlahip {
+namespace v3 {
+
+constexpr int kBlk = 32;                                   // keys per block
+constexpr int kNopeBufB = kBlk * 1024;                     // 32768
+constexpr int kRopeBufB = kBlk * 128;                      // 4096
+constexpr int kRopeOff = 4 * kNopeBufB;                    // 131072
+constexpr int kPOff = kRopeOff + 3 * kRopeBufB;            // 143360
+constexpr int kPBufB = 8192;                               // 4 row groups x 2 k-blocks x 64 lanes x 16 B
+constexpr int kFlagOff = kPOff + 2 * kPBufB;               // 159744: restart flags, 2 x 8 dwords
+constexpr int kLimitOff = kFlagOff + 64;                   // per row of the group: number of visible keys (read by masking blocks only)
+constexpr int kSeenOff = kLimitOff + 512;                  // per lane: the score that raised its restart flag
+constexpr int kLdsB = kSeenOff + 2048;
+static_assert(kLdsB <= 160 * 1024, "LDS budget");
+constexpr int kLead = 3;                                   // block i + kLead is copied while block i is consumed
+constexpr int kCopies = 5;                                 // copy instructions per wavefront and block (4 nope rows + rope)
+#ifndef MLA_V3_AHEAD
+#define MLA_V3_AHEAD 4
+#endif
+constexpr int kAhead = MLA_V3_AHEAD;                                  // K fragments read ahead of the MFMA that consumes them
+constexpr float kRestartThreshold = 100.f;                 // log2 units above a row's reference
+constexpr int kSegCost = kPlanSegCost;
+static_assert(kBlk == kPlanBlk, "the merge kernels recompute the chunk plan with these constants");
+
+// XOR swizzles of the 16-byte granules of a row: linear over GF(2), so swz(a ^ b) = swz(a) ^ swz(b)
+__device__ __forceinline__ int swz_nope(int r) {
+  int r0 = r & 1, r1 = (r >> 1) & 1, r2 = (r >> 2) & 1, r3 = (r >> 3) & 1;
+  return ((r1 ^ r3) << 3) | (r0 << 2) | (r1 << 1) | r2;
+}
+__device__ __forceinline__ int swz_rope(int r) {
+  int r0 = r & 1, r1 = (r >> 1) & 1, r2 = (r >> 2) & 1, r3 = (r >> 3) & 1;
+  return ((r0 ^ r3) << 2) | (r1 << 1) | r2;
+}
+__device__ __forceinline__ int num_blocks(int len) { return len > 0 ? (len + kBlk - 1) / kBlk : 0; }
+__device__ __forceinline__ int work_units(int len) { return len > 0 ? (len + kBlk - 1) / kBlk + kSegCost : 0; }
+__device__ __forceinline__ int wave_sum_i32(int v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+  return v;
+}
+__device__ __forceinline__ int wave_max_i32(int v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v = max(v, __shfl_xor(v, d, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_incl_scan_i32(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) { const int t = __shfl_up(v, d, 64); v += lane >= d ? t : 0; }
+  return v;
+}
+typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
+
+#ifdef MLA_V3_TRACE
+__device__ unsigned long long* g_trace;                     // [workgroup][wave][8]: clock sums per phase, block count
+#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0
+#define TR_STAMP(x) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x)::"memory")
+#define TR_ADD(k) do { TR_STAMP(tr_b); tr_t[k] += tr_b - tr_a; tr_a = tr_b; } while (0)
+#else
+#define TR_DECL
+#define TR_STAMP(x)
+#define TR_ADD(k)
+#endif
+
+template <bool kSparse, bool kWindow>
+__global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params p) {
+  static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // 0..7
+  const int l16 = lane & 15;                                  // QK: query row of the wave / key of a 16-key group
+  const int g = lane >> 4;                                    // QK: 8-element group of a 32-deep contraction step
+  const int h32 = lane & 31;
+  const int half = lane >> 5;
+  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has its own L2.  Two families of workgroups
+  // read the same bytes and are renumbered to sit on one XCD: the row groups of one chunk (more than 128 query rows)
+  // stream the same cache rows; consecutive chunks belong to the same sequence and load the same queries, so every XCD
+  // takes a contiguous eighth of the chunks.
+  int chunk = blockIdx.x, grp = blockIdx.z;
+  if ((gridDim.x & 7) == 0) {
+    const int lin = blockIdx.x + gridDim.x * blockIdx.z;    // launch order
+    const int j = lin >> 3;                                  // j-th workgroup of XCD lin & 7
+    grp = j % gridDim.z;
+    chunk = (lin & 7) * (gridDim.x >> 3) + j / gridDim.z;
+  }
+  const int r_max = p.max_q_len * p.num_heads;
+  if (grp * 128 >= r_max) return;
+  const uint32_t lds0 = lds_addr_of(lds);
+
+  // ---- which blocks are mine: the balanced chunk plan (see mla_chunk_reduce_kernel, which recomputes it) ----
+  // Every non-empty sequence is kSegCost units of start-up followed by its 32-key blocks, the sequences end to end, and
+  // that line is cut into gridDim.x chunks of equal length; a chunk that crosses a sequence boundary runs several
+  // segments; the segment of sequence b in chunk c writes partial number c + b.
+  int seg_b;
+  int64_t v_cur, v_end, v_seq;
+  {
+    int tot = 0;
+    for (int i = lane; i < p.batch; i += 64) tot += work_units(p.seq_lens[i]);
+    tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
+    const int64_t cb = (int64_t)chunk * tot / gridDim.x, ce = (int64_t)(chunk + 1) * tot / gridDim.x;
+    if (cb == ce) return;
+    int carry = 0, b0 = 0, pb0 = 0;
+    for (int base = 0; base < p.batch; base += 64) {
+      const int i = base + lane;
+      const int c = i < p.batch ? work_units(p.seq_lens[i]) : 0;
+      const int pe = wave_incl_scan_i32(c, lane) + carry;
+      const bool le = i < p.batch && pe <= cb;
+      b0 += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+      pb0 = max(pb0, wave_max_i32(le ? pe : 0));
+      carry = __builtin_amdgcn_readlane(pe, 63);
+    }
+    seg_b = __builtin_amdgcn_readfirstlane(b0) - 1;
+    v_seq = __builtin_amdgcn_readfirstlane(pb0);
+    v_cur = cb;
+    v_end = ce;
+  }
+
+  TR_DECL;
+  while (v_cur < v_end) {
+  seg_b++;
+  if (seg_b >= p.batch) break;
+  const int b = seg_b;
+  const int L = p.seq_lens[b];
+  const int64_t v_b = v_seq;
+  v_seq += work_units(L);
+  const int64_t v_hi = v_seq < v_end ? v_seq : v_end;
+  int blk_begin = (int)(v_cur - v_b) - kSegCost;
+  int blk_end = (int)(v_hi - v_b) - kSegCost;
+  blk_begin = blk_begin < 0 ? 0 : blk_begin;
+  blk_end = blk_end < 0 ? 0 : blk_end;
+  v_cur = v_hi;
+  const int nb = blk_end - blk_begin;
+  if (nb <= 0) continue;
+  if (threadIdx.x == 0) {
+    if (blk_begin == 0) p.seg_ids[2 * b] = chunk + b;
+    if (blk_end == num_blocks(L)) p.seg_ids[2 * b + 1] = chunk + b;
+  }
+  lds_barrier();                                              // the previous segment's epilogue is done with the buffers
+
+  int q0, qlen;
+  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
+  qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
+  const int rows = qlen * p.num_heads;
+
+  // this lane's query row for QK / softmax; the four lanes l16 + 16*g share it
+  const int rloc = wave * 16 + l16;                           // row inside the group of 128
+  const int row = grp * 128 + rloc;
+  const bool row_ok = row < rows && L > 0;
+  const int t_local = row / p.num_heads;
+  const int head = row - t_local * p.num_heads;
+  {
+    int limit = row_ok ? (L - qlen + t_local + 1) : 0;       // keys [0, limit) are visible to this row
+    limit = limit < 0 ? 0 : limit;
+    if (g == 0) *(int*)(lds + kLimitOff + rloc * 4) = limit;  // read back by the blocks that have to mask (the last ones)
+    *(float*)(lds + kSeenOff + threadIdx.x * 4) = -INFINITY;
+  }
+  const int win_skip = kWindow ? p.win_skip[b] : 0;
+  const int win_blk0 = kWindow ? p.win_sink / kBlk : 0;
+  const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
+
+  if (grp * 128 >= rows) {
+    if (row < r_max && g == 0) { p.lse_part[part_base + rloc] = -INFINITY; p.corr_scale[part_base + rloc] = 0.f; }
+    continue;
+  }
+
+  // ---- global -> LDS copies: per wave and block four nope rows (1 KiB each) and four rope rows (lanes 0..31) ----
+  // Row r of a block goes to nope buffer row r (granule gr at position gr ^ swz(r)) and rope buffer row r.  Wave w copies
+  // rows 4w..4w+3: swz(4w + j) = swz(4w) ^ swz(j), so one per-lane offset serves all four rows.
+  // The per-lane offsets are worked out from the hardware lane number at every use (a handful of vector ALU
+  // instructions per block, in the phase where that unit idles) instead of occupying registers through the loop.
+  const uint32_t n_sr2 = (uint32_t)p.nope_sr * 2u, r_sr2 = (uint32_t)p.rope_sr * 2u;       // row strides in bytes
+  const int swz_nw = swz_nope((wave * 4) & 15), swz_rw = swz_rope((wave * 4) & 15);        // scalars
+
+  ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (kSparse ? 0 : (int64_t)b * p.bt_stride);
+  ConstI32Ptr srows = (ConstI32Ptr)(p.sparse_rows) + (kSparse ? (int64_t)b * p.sparse_stride : 0);
+  const int64_t max_row = p.num_pages * p.page_size - 1;
+  // Row list (kSparse): the 32 cache rows of the block whose copies go out next travel in one vector register, lane r
+  // holding the row of key r, and every copy picks its row with v_readlane.  The load for block X+1 is issued in front of
+  // the copies of block X, so the wait that lets a block's copies land also covers it (vector memory returns in order).
+  uint32_t ids_cur = 0, ids_nxt = 0;
+  auto ids_load = [&](int blk_x) {
+    if constexpr (kSparse) {
+      int tok = blk_x * kBlk + (lane & 31);
+      tok = tok < L ? tok : L - 1;
+      tok = tok < 0 ? 0 : tok;
+      const int32_t* src = p.sparse_rows + (int64_t)b * p.sparse_stride + tok;
+      asm volatile("global_load_dword %0, %1, off" : "=v"(ids_nxt) : "v"(src) : "memory");
+    }
+  };
+  auto ids_rotate = [&] {
+    if constexpr (kSparse) {
+      asm volatile("" : "+v"(ids_nxt));
+      ids_cur = ids_nxt;
+    }
+  };
+  auto load_page = [&](int page) -> int64_t {
+    page = page < p.max_blocks ? page : p.max_blocks - 1;
+    int64_t pg = bt[page];
+    return pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
+  };
+  int page_cur = 0;
+  int64_t pg_nxt = 0;
+  const char* np_page = (const char*)p.nope;                  // first rows of the current page (64-bit products once per page)
+  const char* rp_page = (const char*)p.rope;
+  auto set_page = [&](int64_t pg) {
+    np_page = (const char*)p.nope + pg * p.nope_sp * 2;
+    rp_page = (const char*)p.rope + pg * p.rope_sp * 2;
+  };
+  auto issue_reset = [&]() {
+    if constexpr (!kSparse) {
+      page_cur = (blk_begin + (kWindow && blk_begin >= win_blk0 ? win_skip : 0)) >> 2;
+      set_page(load_page(page_cur));
+      pg_nxt = load_page(page_cur + 1);
+    }
+  };
+  // The five copies of a block are issued one at a time ("pieces") so that they can be spread over the MFMAs of the QK
+  // phase.  Rows past the end of the sequence re-read its last row (their scores are masked).
+  // rope buffer of a block: (blk - blk_begin + rope_ph) % 3 without a division (rope_ph = blk_begin % 3 once per segment)
+  const int rope_ph = blk_begin % 3;
+  auto rope_buf_of = [&](int blk) -> int {
+    int r = (blk - blk_begin + rope_ph);                      // counts up by one per block from a value below 3
+    r -= 3 * (int)(((uint32_t)r * 43691u) >> 17);             // r / 3 for r < 98304: one multiply, no division sequence
+    return r;
+  };
+  struct IssueCtx { const char* np; const char* rp; const char* a0; uint32_t nbuf, rbuf; int last, tok0; };
+  auto issue_begin = [&](int blk) -> IssueCtx {
+    IssueCtx c;
+    c.tok0 = blk * kBlk;
+    c.last = L - 1 - c.tok0;                                  // last valid row of the block (>= 0)
+    c.nbuf = lds0 + (blk & 3) * kNopeBufB;
+    c.rbuf = lds0 + kRopeOff + rope_buf_of(blk) * kRopeBufB;
+    if constexpr (kSparse) {
+      c.np = (const char*)p.nope;
+      c.rp = (const char*)p.rope;
+    } else {
+      const int cblk = blk + (kWindow && blk >= win_blk0 ? win_skip : 0);   // block of the cache
+      const int page = cblk >> 2;
+      if (page != page_cur) {
+        // the next page's number is only asked for here (raw: clamping it now would wait for the load); it is clamped
+        // when it becomes the current page, four blocks later
+        if (kWindow && page != page_cur + 1) set_page(load_page(page));        // the jump from the sink to the window
+        else set_page(pg_nxt < 0 ? 0 : (pg_nxt >= p.num_pages ? p.num_pages - 1 : pg_nxt));
+        page_cur = page;
+        const int pn = page + 1 < p.max_blocks ? page + 1 : p.max_blocks - 1;
+        pg_nxt = bt[pn];
+      }
+      const uint32_t row0 = (uint32_t)(cblk & 3) * kBlk;
+      c.np = np_page + (uint64_t)row0 * n_sr2;
+      c.rp = rp_page + (uint64_t)row0 * r_sr2;
+    }
+    c.a0 = c.np + (uint64_t)(wave * 4) * n_sr2;               // full dense blocks: running row address
+    return c;
+  };
+  // The hardware lane number behind an opaque (and volatile) statement: what is derived from it inside the loop is
+  // computed inside the loop.  Left alone the compiler hoists every loop-invariant LDS address out of the block loop, a
+  // dozen registers of them, and then spills them - and a scratch reload waits for every copy in flight.
+  auto lane_now = [] {
+    int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(ln));
+    return ln;
+  };
+  auto rope_lane_row = [&] { return (lane_now() >> 3) & 3; };                               // lane's row among the wave's four
+  auto rope_lane_off = [&]() -> uint32_t {
+    const int ln = lane_now(), t = (ln >> 3) & 3;
+    return (uint32_t)(((ln & 7) ^ swz_rw ^ ((t & 1) << 2) ^ (t & 2)) << 4);                 // swz_rope(t) = (t0 << 2) | (t1 << 1)
+  };
+  // kFull: every row of the block exists and the source is the paged cache; kVecIds (row list): rows come from ids_cur
+  auto issue_piece = [&](IssueCtx& c, int k, auto full, auto vec_ids) {
+    constexpr bool kFull = decltype(full)::value && !kSparse;
+    constexpr bool kVecIds = decltype(vec_ids)::value && kSparse;
+    auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
+    auto row_of = [&](int re) -> int32_t {
+      if constexpr (kVecIds) return (int32_t)__builtin_amdgcn_readlane((int)ids_cur, re);
+      else return srows[c.tok0 + re];
+    };
+    if (k < 4) {
+      const int r = wave * 4 + k;
+      const uint32_t off = (uint32_t)((lane_now() ^ swz_nw ^ swz_nope(k)) << 4);
+      if constexpr (kFull) {
+        dma16_sv(c.a0, off, c.nbuf + r * 1024);
+        c.a0 += n_sr2;
+      } else {
+        const int re = r < c.last ? r : c.last;
+        if constexpr (kSparse) dma16_sv(c.np + clampi(row_of(re)) * n_sr2, off, c.nbuf + r * 1024);
+        else dma16_sv(c.np + (uint64_t)re * n_sr2, off, c.nbuf + r * 1024);
+      }
+    } else {
+      // the wave's four rope rows, 128 bytes each: half an instruction (lanes 32..63 sit out)
+      if constexpr (kSparse) {
+        int32_t mine = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const int r = wave * 4 + j;
+          const int32_t sj = row_of(r < c.last ? r : c.last);
+          mine = rope_lane_row() == j ? sj : mine;
+        }
+        dma16_v_lo32(c.rp + clampi(mine) * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+      } else if constexpr (kFull) {
+        dma16_sv_lo32(c.rp + (uint64_t)(wave * 4) * r_sr2, (uint32_t)rope_lane_row() * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+      } else {
+        const int r = wave * 4 + rope_lane_row();
+        const int re = r < c.last ? r : c.last;
+        dma16_sv_lo32(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+      }
+    }
+  };
+  auto issue_block = [&](int blk) {
+    IssueCtx c = issue_begin(blk);
+#pragma unroll
+    for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{}, std::integral_constant<bool, kSparse>{});
+  };
+  uint32_t ids_head[kLead] = {};
+  auto issue_first = [&]() {
+    issue_reset();
+    if constexpr (kSparse) {
+#pragma unroll
+      for (int j = 0; j < kLead; j++) {
+        int tok = (blk_begin + j) * kBlk + (lane & 31);
+        tok = tok < L ? tok : L - 1;
+        tok = tok < 0 ? 0 : tok;
+        const int32_t* src = p.sparse_rows + (int64_t)b * p.sparse_stride + tok;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(ids_head[j]) : "v"(src) : "memory");
+      }
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(ids_head[0]), "+v"(ids_head[1]), "+v"(ids_head[2])::"memory");
+      ids_cur = ids_head[0];
+    }
+    issue_block(blk_begin);
+  };
+  auto issue_next_two = [&]() {
+    if constexpr (kSparse) {
+#pragma unroll
+      for (int j = 1; j < kLead; j++)
+        if (j < nb) {
+          ids_cur = ids_head[j];
+          issue_block(blk_begin + j);
+        }
+    } else {
+#pragma unroll 1
+      for (int j = 1; j < kLead && j < nb; j++) issue_block(blk_begin + j);
+    }
+  };
+
+  // ---- prologue: the first block's copies go out, then the query loads; both are waited for together ----
+  issue_first();
+  bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
+  {
+    const int64_t tq = row_ok ? (q0 + t_local) : q0;         // rows that do not exist read row 0 of the sequence
+    const int64_t hq = row_ok ? head : 0;
+    // Contraction step kk of the latent part covers the 16-byte granules 16*(kk/4) + 4g' + kk%4, g' = 0..3, and lane group
+    // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
+    // in one aligned 32-byte piece of a row, or the LDS serves the instruction at half rate (measured: 126 against 227
+    // bytes per clock and CU with eight wavefronts reading).
+    const __bf16* qn = p.q_nope + tq * p.qn_st + hq * p.qn_sh + g * 32;
+    const __bf16* qr = p.q_rope + tq * p.qr_st + hq * p.qr_sh + g * 16;
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++)
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[kk]) : "v"(qn), "i"((kk >> 2) * 256 + (kk & 3) * 16));
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[16 + kk]) : "v"(qr), "i"(kk * 16));
+    __builtin_amdgcn_s_waitcnt(0x0F70);                                         // vmcnt(0)
+#pragma unroll
+    for (int kk = 0; kk < 18; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
+  }
+
+  f32x16 acc[2][4];                                          // [32-column block of this wave's 64][row group]
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  float m_ref = -INFINITY;       // the row's softmax reference (log2 domain), the same in its four lanes
+  float l_run = 0.f;             // this lane's share of the row's sum
+  float top_p = 0.f;             // largest probability among this lane's visible keys so far ...
+  int top_tag = -1;              // ... and where: (block << 3) | element number
+
+  // ---- per-lane LDS offsets ----
+  const uint32_t kbase = (uint32_t)(l16 * 1024 + (((g << 2) ^ swz_nope(l16)) << 4));      // ^ ((kk&3) << 4), offset kg*16384 + (kk>>2)*256
+  const uint32_t rbase = (uint32_t)(kRopeOff + l16 * 128 + (((g << 1) ^ swz_rope(l16)) << 4));   // ^ ((kk-16) << 4), offset kg*2048
+  const int g16 = lane >> 4, j16 = lane & 15;
+  const int v_row = 4 * (g16 >> 1) + (j16 >> 2);              // + 8*rd + 16*kb
+  const int v_cl = 2 * (g16 & 1) + ((j16 & 3) >> 1);
+  const int v_in = (j16 & 1) * 8;
+  uint32_t vbase[2];                                          // [rd]: ^ (db << 6), + kb*16384, + buffer
+#pragma unroll
+  for (int rd = 0; rd < 2; rd++) {
+    const int rr = v_row + 8 * rd;
+    vbase[rd] = (uint32_t)(rr * 1024 + v_in + (((8 * wave + v_cl) ^ swz_nope(rr & 15)) << 4));
+  }
+  // P^T in LDS, in the order the P.V MFMAs read it: fragment (row group rg, k-block kb) is 64 lanes x 16 B, lane
+  // (n = row % 32, h) holding keys 16kb + {4h..4h+3, 8+4h..8+4h+3}.  The QK lane (row l16 of wave w, group g) holds keys
+  // 16kg + 4g + {0..3}: they are the first (g < 2) or second (g >= 2) 8 bytes of lane (n, h = g & 1).
+  const uint32_t p_w_off = (uint32_t)(kPOff + (((wave >> 1) * 2) * 64 + (g & 1) * 32 + (wave & 1) * 16 + l16) * 16 + (g >> 1) * 8);   // + kg*1024 + parity*8192
+  const uint32_t p_r_off = (uint32_t)(kPOff + lane * 16);     // + (rg*2 + kb)*1024 + parity*8192
+
+  // S^T for block `blk`: hand-placed K-fragment reads kAhead fragments ahead of the MFMA that consumes them, explicit
+  // lgkmcnt waits, MFMAs as assembly with the scores in ordinary vector registers (the accumulation file is full of
+  // output accumulators).  Dependent MFMAs of one shape with identical C and D need no padding; the two accumulators
+  // alternate.  The wait after the last one (MFMA result read by the vector ALU) is the s_nop pair at the end.
+  auto qk_block = [&](int blk, f32x4 (&s)[2], auto issue, int blk_issue) {
+    constexpr int kIssueMode = decltype(issue)::value;       // 0: no copies; 1: any block; 2: a full block of the paged cache
+    constexpr bool kIssue = kIssueMode != 0;
+    // the six addresses the 36 reads use (the rest is immediate offsets)
+    uint32_t na[4], ra[2];
+    na[0] = lds0 + (blk & 3) * kNopeBufB + kbase;
+    ra[0] = lds0 + rope_buf_of(blk) * kRopeBufB + rbase;
+#pragma unroll
+    for (int b4 = 1; b4 < 4; b4++) na[b4] = na[0] ^ (uint32_t)(b4 << 4);
+    ra[1] = ra[0] ^ 16u;
+    IssueCtx ic;
+    if constexpr (kIssue) { ids_load(blk_issue + 1); ic = issue_begin(blk_issue); }
+    bf16x8 ka[kAhead];
+    // fragment j: contraction step kk = j >> 1, key group kg = j & 1; each statement is wait + MFMA + the read that
+    // refills the fragment register (one statement, so that nothing is scheduled or padded in between)
+#define MLA_K_ADDR(j) (((j) >> 1) < 16 ? na[((j) >> 1) & 3] : ra[((j) >> 1) - 16])
+#define MLA_K_OFF(j) (((j) >> 1) < 16 ? ((j) & 1) * 16384 + ((j) >> 3) * 256 : ((j) & 1) * 2048)
+#if defined(ABL_QK_NOREAD)
+#define RD "; "
+#else
+#define RD
+#endif
+#if defined(ABL_QK_NOMFMA)
+#define MF "; "
+#else
+#define MF
+#endif
+#pragma unroll
+    for (int i = 0; i < kAhead; i++) asm volatile(RD "ds_read_b128 %0, %1 offset:%2" : "=v"(ka[i]) : "v"(MLA_K_ADDR(i)), "i"(MLA_K_OFF(i)));
+#pragma unroll
+    for (int j = 0; j < 36; j++) {
+      constexpr int D = kAhead;
+      const int younger = (36 - 1 - j) < (D - 1) ? (36 - 1 - j) : (D - 1);
+      if (j < 2)
+        asm volatile("s_waitcnt lgkmcnt(%5)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0\n\t" RD "ds_read_b128 %1, %3 offset:%4"
+                     : "=&v"(s[j & 1]), "+v"(ka[j % D]) : "v"(qf[j >> 1]), "v"(MLA_K_ADDR(j + D)), "i"(MLA_K_OFF(j + D)), "i"(younger));
+      else if (j + D < 36)
+        asm volatile("s_waitcnt lgkmcnt(%5)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\t" RD "ds_read_b128 %1, %3 offset:%4"
+                     : "+v"(s[j & 1]), "+v"(ka[j % D]) : "v"(qf[j >> 1]), "v"(MLA_K_ADDR(j + D)), "i"(MLA_K_OFF(j + D)), "i"(younger));
+      else
+        asm volatile("s_waitcnt lgkmcnt(%3)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                     : "+v"(s[j & 1]) : "v"(ka[j % D]), "v"(qf[j >> 1]), "i"(younger));
+      if constexpr (kIssue) if (j % 7 == 3) issue_piece(ic, j / 7, std::integral_constant<bool, kIssueMode == 2>{}, std::true_type{});
+    }
+#undef MLA_K_ADDR
+#undef MLA_K_OFF
+    asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s[0]), "+v"(s[1]));
+  };
+
+  // ---- softmax + P.V, hand-ordered ----
+  // The vector ALU is the second bottleneck of this kernel: two wavefronts share one, an MFMA of one wavefront hides about
+  // four ordinary vector instructions of the other, and v_exp_f32 runs at quarter rate.  So the softmax of block i+1 is
+  // written as short assembly statements placed between the P.V MFMAs of block i (the compiler would otherwise gather the
+  // vector work behind the MFMAs), and it is kept to the minimum: per score one tag, one FMA, one exponential, one add,
+  // half a conversion.  The lane's eight raw scores (key 16*(r/4) + 4g + r%4 at sc[r]) first get their element number r
+  // into the three low mantissa bits (7 ulp: 1e-5 of a probability), so the float maximum of the tagged scores names
+  // the lane's most probable key and its probability without a second pass over the probabilities.
+  // Nothing here crosses lanes: sums and dominant-key candidates are per lane and are combined in the epilogue.
+  struct Sm { float t, pm, psum; uint32_t mx; uint32_t pw[4]; };   // t = scaled max score - reference (log2), pm = exp2(t); pw: bf16 pairs
+#define SM_TAG(r) asm volatile("v_and_or_b32 %0, %0, -8, %1" : "+v"(sc[r]) : "n"(r))
+#define SM_EXP2(a, b)                                                                                                   \
+  asm volatile("v_fma_f32 %0, %0, %2, -%3\n\tv_fma_f32 %1, %1, %2, -%3\n\tv_exp_f32 %0, %0\n\tv_exp_f32 %1, %1"          \
+               : "+v"(sc[a]), "+v"(sc[b]) : "s"(p.scale_log2), "v"(m_ref))
+  auto sm_head = [&](float (&sc)[8], Sm& st) {               // tags and the lane's maximum (12 instructions)
+    SM_TAG(0); SM_TAG(1); SM_TAG(2); SM_TAG(3); SM_TAG(4); SM_TAG(5); SM_TAG(6); SM_TAG(7);
+    asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(st.mx) : "v"(sc[0]), "v"(sc[1]), "v"(sc[2]));
+    asm volatile("v_max3_f32 %0, %0, %1, %2\n\tv_max3_f32 %0, %0, %3, %4\n\tv_max_f32 %0, %0, %5"
+                 : "+v"(st.mx) : "v"(sc[3]), "v"(sc[4]), "v"(sc[5]), "v"(sc[6]), "v"(sc[7]));
+  };
+  auto sm_pm = [&](Sm& st) {
+    asm volatile("v_fma_f32 %0, %2, %3, -%4\n\ts_nop 0\n\tv_exp_f32 %1, %0\n\ts_nop 0" : "=&v"(st.t), "=v"(st.pm) : "v"(st.mx), "s"(p.scale_log2), "v"(m_ref));
+  };
+  auto sm_sum_lo = [&](float (&sc)[8], Sm& st) {
+    asm volatile("v_add_f32 %0, %2, %3\n\tv_cvt_pk_bf16_f32 %1, %2, %3" : "=&v"(st.psum), "=v"(st.pw[0]) : "v"(sc[0]), "v"(sc[1]));
+    asm volatile("v_add_f32 %0, %0, %2\n\tv_cvt_pk_bf16_f32 %1, %2, %3\n\tv_add_f32 %0, %0, %3"
+                 : "+v"(st.psum), "=v"(st.pw[1]) : "v"(sc[2]), "v"(sc[3]));
+  };
+  auto sm_sum_hi = [&](float (&sc)[8], Sm& st) {
+    asm volatile("v_add_f32 %0, %0, %2\n\tv_cvt_pk_bf16_f32 %1, %2, %3\n\tv_add_f32 %0, %0, %3"
+                 : "+v"(st.psum), "=v"(st.pw[2]) : "v"(sc[4]), "v"(sc[5]));
+    asm volatile("v_add_f32 %0, %0, %2\n\tv_cvt_pk_bf16_f32 %1, %2, %3\n\tv_add_f32 %0, %0, %3"
+                 : "+v"(st.psum), "=v"(st.pw[3]) : "v"(sc[6]), "v"(sc[7]));
+  };
+  // O^T += V^T P^T for block `blk` (this wave's 64 output columns, all four row groups; kPv) with the softmax of the next
+  // block's scores sc riding along (kSm).  Per k-block the two V^T fragments are held while the four P^T fragments go by
+  // (two registers quads, each refilled as soon as its MFMAs are issued), every fragment feeding two MFMAs.
+  auto pv_softmax = [&](int blk, auto with_pv, auto with_sm, float (&sc)[8], Sm& st) {
+    constexpr bool kPv = decltype(with_pv)::value, kSm = decltype(with_sm)::value;
+    const uint32_t vb = lds0 + (blk & 3) * kNopeBufB;
+    const uint32_t a0 = vb + vbase[0], a1 = vb + vbase[1];    // ^ 64 for the second 32 columns, + 16384 for the second k-block
+    const uint32_t a0x = a0 ^ 64u, a1x = a1 ^ 64u;
+    const uint32_t pa = lds0 + (blk & 1) * kPBufB + p_r_off;  // + (rg*2 + kb)*1024
+    bf16x4 v0l, v0h, v1l, v1h;
+    bf16x8 pr0, pr1;
+#define PV_VREAD(kb)                                                                                                   \
+    asm volatile("ds_read_b64_tr_b16 %0, %4 offset:%8\n\tds_read_b64_tr_b16 %1, %5 offset:%8\n\t"                          \
+                 "ds_read_b64_tr_b16 %2, %6 offset:%8\n\tds_read_b64_tr_b16 %3, %7 offset:%8"                              \
+                 : "=&v"(v0l), "=&v"(v0h), "=&v"(v1l), "=&v"(v1h) : "v"(a0), "v"(a1), "v"(a0x), "v"(a1x), "i"((kb) * 16384))
+#define PV_PREAD(dst, rg, kb) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(pa), "i"(((rg) * 2 + (kb)) * 1024))
+#define PV_MFMA2(rg, pr, cnt)                                                                                          \
+    do {                                                                                                               \
+      const bf16x8 va0 = __builtin_shufflevector(v0l, v0h, 0, 1, 2, 3, 4, 5, 6, 7);                                    \
+      const bf16x8 va1 = __builtin_shufflevector(v1l, v1h, 0, 1, 2, 3, 4, 5, 6, 7);                                    \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_f32_32x32x16_bf16 %0, %2, %4, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %3, %4, %1" \
+                   : "+a"(acc[0][rg]), "+a"(acc[1][rg]) : "v"(va0), "v"(va1), "v"(pr), "i"(cnt));                      \
+    } while (0)
+    if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 1, 0); }
+    if constexpr (kSm) sm_head(sc, st);
+    if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_PREAD(pr0, 2, 0); }
+    if constexpr (kSm) SM_EXP2(0, 1);
+    if constexpr (kPv) { PV_MFMA2(1, pr1, 1); PV_PREAD(pr1, 3, 0); }
+    if constexpr (kSm) SM_EXP2(2, 3);
+    if constexpr (kPv) { PV_MFMA2(2, pr0, 1); PV_PREAD(pr0, 0, 1); }
+    if constexpr (kSm) SM_EXP2(4, 5);
+    if constexpr (kPv) { PV_MFMA2(3, pr1, 1); PV_VREAD(1); PV_PREAD(pr1, 1, 1); }
+    if constexpr (kSm) { SM_EXP2(6, 7); sm_pm(st); }
+    if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_PREAD(pr0, 2, 1); }
+    if constexpr (kSm) sm_sum_lo(sc, st);
+    if constexpr (kPv) { PV_MFMA2(1, pr1, 1); PV_PREAD(pr1, 3, 1); }
+    if constexpr (kSm) sm_sum_hi(sc, st);
+    if constexpr (kPv) { PV_MFMA2(2, pr0, 1); PV_MFMA2(3, pr1, 0); }
+#undef PV_VREAD
+#undef PV_PREAD
+#undef PV_MFMA2
+  };
+  // After the softmax: the last blocks of a sequence hold keys that some rows must not see (causal multi-token queries,
+  // rows past the end of the sequence); only those blocks pay for the masking.  Then P^T and the restart flag go to LDS.
+  auto softmax_finish = [&](int blk, float (&sc)[8], Sm& st) {
+    bool front = false;
+    if constexpr (kWindow) front = blk >= win_blk0 && blk * kBlk < L - p.win_size;
+    if ((blk + 1) * kBlk > L - p.max_q_len + 1 || front) {
+      int blk_s = blk;
+      asm volatile("" : "+s"(blk_s));
+      const int limit = *(const int*)(lds + kLimitOff + (wave * 16 + (lane_now() & 15)) * 4);
+      const int rel = limit - blk_s * kBlk - ((lane_now() >> 4) << 2);   // score r is visible iff 16*(r/4) + r%4 < rel
+      const int rel_lo = (kWindow && blk >= win_blk0) ? rel - p.win_size : -64;
+      st.psum = 0.f;
+      float pv = 0.f;
+      int best = 0;
+#pragma unroll
+      for (int r = 0; r < 8; r++) {
+        const int kpos = 16 * (r >> 2) + (r & 3);
+        const float v = (kpos < rel && kpos >= rel_lo) ? sc[r] : 0.f;
+        sc[r] = v;
+        st.psum += v;
+        best = v > pv ? r : best;
+        pv = fmaxf(pv, v);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const bf16x2 pr2 = {(__bf16)sc[2 * j], (__bf16)sc[2 * j + 1]};
+        st.pw[j] = __builtin_bit_cast(uint32_t, pr2);
+      }
+      st.pm = pv;                                             // largest VISIBLE probability of the lane in this block
+      st.mx = (uint32_t)best;
+    }
+    // Remember the most probable key: the bf16 rounding of its probability is the largest single error of the P.V
+    // product when the softmax is peaked, and the merge kernel takes it out again.
+    {
+      const bool nw = st.pm > top_p;
+      top_p = nw ? st.pm : top_p;
+      top_tag = nw ? (int)((uint32_t)(blk << 3) | (st.mx & 7u)) : top_tag;   // decoded in the epilogue
+    }
+    l_run += st.psum;
+    const uint32_t pw = lds0 + (blk & 1) * kPBufB + p_w_off;
+    const u32x2 w0 = {st.pw[0], st.pw[1]}, w1 = {st.pw[2], st.pw[3]};
+    asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %2 offset:1024" :: "v"(pw), "v"(w0), "v"(w1) : "memory");
+    const bool flag = st.t > kRestartThreshold;               // asks the workgroup to restart with better references
+    const bool any = __builtin_amdgcn_ballot_w64(flag) != 0;
+    if (any) {
+      // (rare) the scores that outgrew the reference are remembered: they become the references of the restart
+      float* seen = (float*)(lds + kSeenOff + (wave * 64 + lane_now()) * 4);
+      if (flag) *seen = fmaxf(*seen, st.t + m_ref);
+    }
+    if (lane_now() == 0) *(int*)(lds + kFlagOff + (blk & 1) * 32 + wave * 4) = any ? 1 : 0;
+  };
+  // every wave reads the same eight flags: a uniform decision
+  auto flags_read = [&](int blk) -> int { return *(const int*)(lds + kFlagOff + (blk & 1) * 32 + (lane_now() & 7) * 4); };
+  auto flags_ask_restart = [&](int fl) -> bool { return __builtin_amdgcn_ballot_w64(fl != 0) != 0; };
+  auto unpack_scores = [&](const f32x4 (&s)[2], float (&sc)[8]) {
+#pragma unroll
+    for (int r = 0; r < 8; r++) sc[r] = s[r >> 2][r & 3];
+  };
+
+  bool restart = false;
+  int restarts_left = 4;         // every restart raises a reference by more than 2^100: fp32 has room for three
+  do {
+    if (restart) {
+      // a row outgrew its reference: drain, take the maxima seen so far as references, clear the sums, start over
+      MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      float ms = *(const float*)(lds + kSeenOff + (wave * 64 + lane_now()) * 4);
+      ms = fmaxf(ms, __shfl_xor(ms, 16, 64));
+      ms = fmaxf(ms, __shfl_xor(ms, 32, 64));
+      m_ref = fmaxf(m_ref, ms);
+      l_run = 0.f;
+      top_p = 0.f;
+      top_tag = -1;
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+      issue_first();
+      restart = false;
+    }
+    ids_load(blk_begin + kLead);                              // (older than the copies below: their wait covers it)
+    issue_next_two();
+    // ---- block 0: QK, softmax, publish ----
+    {
+      if (nb > 2) MLA_WAIT_VMCNT(10); else if (nb > 1) MLA_WAIT_VMCNT(5); else MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      f32x4 s[2];
+      Sm st;
+      qk_block(blk_begin, s, std::integral_constant<int, 0>{}, 0);
+      if (m_ref == -INFINITY) {
+        // the first block fixes the reference: the row's largest score over all 32 keys (visible or not: any finite
+        // reference within 2^100 of the true maximum is as good as another), the same value in the row's four lanes
+        float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                         fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        m_ref = mx * p.scale_log2;
+      }
+      float sc[8];
+      unpack_scores(s, sc);
+      pv_softmax(blk_begin, std::false_type{}, std::true_type{}, sc, st);
+      softmax_finish(blk_begin, sc, st);
+    }
+    // Everything the loop keeps in registers is touched here: a value that was parked in scratch during the prologue is
+    // brought back (and waited for) now, not at its first use inside the loop.
+    asm volatile("" :: "v"(kbase), "v"(rbase), "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(p_r_off), "v"(p_w_off));
+    // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
+    for (int i = 0; i + 1 < nb; i++) {
+      const int blk = blk_begin + i;
+      TR_STAMP(tr_a);
+      // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
+      if (i + 2 < nb) MLA_WAIT_VMCNT(5); else MLA_WAIT_VMCNT(0);
+      TR_ADD(0);
+      ids_rotate();
+      lds_barrier();
+      TR_ADD(1);
+      const int fl = flags_read(blk);
+      f32x4 s[2];
+#ifdef ABL_NO_QK
+      s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0];
+      if (true) {}                                            // no QK and no copies at all (never a copy past the segment)
+#elif defined(ABL_NO_COPY)
+      if (true) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
+#else
+      if (i + kLead >= nb) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
+#endif
+      else if (kSparse || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead);
+      else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + kLead);
+      TR_ADD(2);
+      if (restarts_left > 0 && flags_ask_restart(fl)) { restart = true; restarts_left--; break; }
+      Sm st;
+      float sc[8];
+      unpack_scores(s, sc);
+#ifdef ABL_NO_PV
+      pv_softmax(blk, std::false_type{}, std::true_type{}, sc, st);
+#elif defined(ABL_NO_SOFTMAX)
+      st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
+      st.pw[0] = st.pw[1] = st.pw[2] = st.pw[3] = 0;
+      pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st);
+#else
+      pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st);
+#endif
+      TR_ADD(3);
+#ifndef ABL_NO_FINISH
+      softmax_finish(blk + 1, sc, st);
+#else
+      l_run += st.psum + (float)st.pw[0];
+#endif
+      TR_ADD(4);
+#ifdef MLA_V3_TRACE
+      tr_n++;
+#endif
+    }
+    if (!restart) {
+      const int blk = blk_end - 1;
+      MLA_WAIT_VMCNT(0);
+      lds_barrier();
+      if (restarts_left > 0 && flags_ask_restart(flags_read(blk))) { restart = true; restarts_left--; }
+      else { float sc[8]; Sm st; pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st); }
+    }
+  } while (restart);
+
+  // ---- epilogue ----
+  // (lane-derived values are worked out again from the hardware lane number: nothing of them has to live through the loop)
+  lds_barrier();                                              // all PV done; tile buffers and P buffers are free
+  const int e_ln = lane_now();
+  const int e_l16 = e_ln & 15, e_g = e_ln >> 4, e_h32 = e_ln & 31, e_half = e_ln >> 5;
+  const int e_rloc = wave * 16 + e_l16;
+  {
+    const int e_row = grp * 128 + e_rloc;
+    const bool e_row_ok = e_row < rows && L > 0;
+    // the row's four lanes combine their sums and their candidates for the dominant key
+    float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+    l_tot += __shfl_xor(l_tot, 32, 64);
+    int top_tok = top_tag < 0 ? -1 : (top_tag >> 3) * kBlk + 16 * ((top_tag >> 2) & 1) + 4 * e_g + (top_tag & 3);
+#pragma unroll
+    for (int d = 16; d <= 32; d <<= 1) {
+      const float op = __shfl_xor(top_p, d, 64);
+      const int ot = __shfl_xor(top_tok, d, 64);
+      const bool take = op > top_p || (op == top_p && ot >= 0 && (top_tok < 0 || ot < top_tok));
+      top_p = take ? op : top_p;
+      top_tok = take ? ot : top_tok;
+    }
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    // Rows whose most probable key carries more than 1/16 of the weight leave a note for the merge kernel: the rounding
+    // error of that key's probability (already divided by l) and the address of its latent vector in the cache.
+    float corr = 0.f;
+    const __bf16* vrow = p.nope;
+    if (e_row_ok && top_tok >= 0 && top_p * 16.f > l_tot) {
+      corr = (top_p - (float)(__bf16)top_p) * inv;
+      if constexpr (kSparse) {
+        int64_t slot = p.sparse_rows[(int64_t)b * p.sparse_stride + top_tok];
+        slot = slot < 0 ? 0 : (slot > max_row ? max_row : slot);
+        vrow = p.nope + slot * p.nope_sr;
+      } else {
+        const int ctok = top_tok + ((kWindow && top_tok >= p.win_sink) ? win_skip * kBlk : 0);   // position in the cache
+        int page = ctok / kPage;
+        page = page < p.max_blocks ? page : p.max_blocks - 1;
+        int64_t pg = p.block_table[(int64_t)b * p.bt_stride + page];
+        pg = pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
+        vrow = p.nope + pg * p.nope_sp + (int64_t)(ctok % kPage) * p.nope_sr;
+      }
+    }
+    if (e_g == 0) {
+      *(float*)(lds + kPOff + (e_rloc & 31) * 16 + (e_rloc >> 5) * 4) = inv;
+      if (e_row < r_max) {
+        const int64_t pr = part_base + e_rloc;
+        p.lse_part[pr] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        p.corr_scale[pr] = corr;
+        p.corr_row[pr] = vrow;
+      }
+    }
+  }
+  lds_barrier();
+  const f32x4 inv4 = *(const f32x4*)(lds + kPOff + e_h32 * 16);
+  // transpose through this wave's private 16 KiB: 128 rows x 64 columns, fp16 (128 bytes per row, 8-byte slots XORed
+  // with the row so that neither the writes nor the reads collide)
+  char* stage = lds + wave * 16384;
+#pragma unroll
+  for (int rg = 0; rg < 4; rg++) {
+    const int srow = rg * 32 + e_h32;
+#pragma unroll
+    for (int db = 0; db < 2; db++)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; q4++) {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        h4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = (_Float16)(acc[db][rg][q4 * 4 + e] * inv4[rg]);
+        const int g8 = db * 8 + q4 * 2 + e_half;              // 8-byte slot in the row (16 per row)
+        *(h4*)(stage + srow * 128 + ((g8 ^ ((srow >> 1) & 15)) << 3)) = v;
+      }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // read back: 16 lanes read one row (128 B), four rows per instruction
+#pragma unroll 4
+  for (int it = 0; it < 32; it++) {
+    const int srow = it * 4 + e_g;
+    const u32x2 v = *(const u32x2*)(stage + srow * 128 + ((e_l16 ^ ((srow >> 1) & 15)) << 3));
+    if (grp * 128 + srow < r_max)
+      *(u32x2*)(p.o_part + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }  // segments
+#ifdef MLA_V3_TRACE
+  if (g_trace && lane == 0) {
+    unsigned long long* t = g_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.z) * 8 + wave) * 8;
+    for (int k = 0; k < 6; k++) t[k] = tr_t[k];
+    t[6] = tr_n;
+  }
+#endif
+}
+
+}  // namespace v3
+
+int launch_decode_v3(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream) {
+  const void* kernel = sparse ? (const void*)v3::mla_decode_v3_kernel<true, false>
+                              : (p.win_skip ? (const void*)v3::mla_decode_v3_kernel<false, true>
+                                            : (const void*)v3::mla_decode_v3_kernel<false, false>);
+  const int rc = ensure_dynamic_lds(kernel, v3::kLdsB, "mla_decode_v3_kernel");
+  if (rc != MLA_OK) return rc;
+#ifdef MLA_V3_TRACE
+  {
+    const char* e = getenv("MLA_V3_TRACE_PTR");
+    unsigned long long* ptr = e ? (unsigned long long*)strtoull(e, nullptr, 16) : nullptr;
+    hipMemcpyToSymbol(HIP_SYMBOL(v3::g_trace), &ptr, sizeof(ptr));
+  }
+#endif
+  if (sparse) hipLaunchKernelGGL((v3::mla_decode_v3_kernel<true, false>), grid, dim3(512), v3::kLdsB, stream, p);
+  else if (p.win_skip) hipLaunchKernelGGL((v3::mla_decode_v3_kernel<false, true>), grid, dim3(512), v3::kLdsB, stream, p);
+  else hipLaunchKernelGGL((v3::mla_decode_v3_kernel<false, false>), grid, dim3(512), v3::kLdsB, stream, p);
+  return check_launch("mla_decode_v3_kernel");
+}
+
+}  // namespace mlahip

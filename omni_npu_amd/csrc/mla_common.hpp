@@ -77,6 +77,23 @@ __device__ __forceinline__ void dma16_v(const void* gaddr, uint32_t lds_addr_uni
                : "memory", "m0");
 }
 
+// The same two copies issued by lanes 0..31 only (512 bytes): the upper half of the execution mask is cleared around
+// the instruction inside the assembly, so the operands stay in the registers a uniform call site gives them.
+__device__ __forceinline__ void dma16_sv_lo32(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  uint32_t save;
+  asm volatile("s_mov_b32 %0, exec_hi\n\ts_mov_b32 exec_hi, 0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 exec_hi, %0"
+               : "=&s"(save)
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_v_lo32(const void* gaddr, uint32_t lds_addr_uniform) {
+  uint32_t save;
+  asm volatile("s_mov_b32 %0, exec_hi\n\ts_mov_b32 exec_hi, 0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 exec_hi, %0"
+               : "=&s"(save)
+               : "s"(lds_addr_uniform), "v"(gaddr)
+               : "memory", "m0");
+}
+
 // Transposed LDS read: within each group of 16 lanes the 16 addresses name a 4 x 16 block of
 // 16-bit elements (lane 4e+c points at row e, columns 4c..4c+3); lane j receives column j,
 // i.e. the four rows' elements at that column.
