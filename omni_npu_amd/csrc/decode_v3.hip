@@ -43,7 +43,9 @@ constexpr int kPBufB = 8192;                               // 4 row groups x 2 k
 constexpr int kFlagOff = kPOff + 2 * kPBufB;               // 159744: restart flags, 2 x 8 dwords
 constexpr int kLimitOff = kFlagOff + 64;                   // per row of the group: number of visible keys (read by masking blocks only)
 constexpr int kSeenOff = kLimitOff + 512;                  // per lane: the score that raised its restart flag
-constexpr int kLdsB = kSeenOff + 2048;
+constexpr int kKTabOff = kSeenOff + 2048;                  // per lane: LDS offsets of its K-fragment reads (latent, rope)
+constexpr int kIdsOff = kKTabOff + 512;                    // row lists: 4 blocks x 8 waves x the wave's four cache rows
+constexpr int kLdsB = kIdsOff + 512;
 static_assert(kLdsB <= 160 * 1024, "LDS budget");
 constexpr int kLead = 3;                                   // block i + kLead is copied while block i is consumed
 constexpr int kCopies = 5;                                 // copy instructions per wavefront and block (4 nope rows + rope)
@@ -118,6 +120,15 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   const int r_max = p.max_q_len * p.num_heads;
   if (grp * 128 >= r_max) return;
   const uint32_t lds0 = lds_addr_of(lds);
+  // Arguments that only the start and the end of a segment need are read from the argument block where they are used
+  // (through a pointer the compiler cannot see through), not held in scalar registers across the block loop: the loop
+  // needs most of them itself, and scalar registers that overflow are parked in vector registers, which are short here.
+  typedef __attribute__((address_space(4))) const DecodeV2Params* KernArgPtr;
+  auto cold = [] {
+    KernArgPtr kp = (KernArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(kp));
+    return kp;
+  };
 
   // ---- which blocks are mine: the balanced chunk plan (see mla_chunk_reduce_kernel, which recomputes it) ----
   // Every non-empty sequence is kSegCost units of start-up followed by its 32-key blocks, the sequences end to end, and
@@ -164,14 +175,20 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   const int nb = blk_end - blk_begin;
   if (nb <= 0) continue;
   if (threadIdx.x == 0) {
-    if (blk_begin == 0) p.seg_ids[2 * b] = chunk + b;
-    if (blk_end == num_blocks(L)) p.seg_ids[2 * b + 1] = chunk + b;
+    int32_t* seg_ids = cold()->seg_ids;
+    if (blk_begin == 0) seg_ids[2 * b] = chunk + b;
+    if (blk_end == num_blocks(L)) seg_ids[2 * b + 1] = chunk + b;
   }
   lds_barrier();                                              // the previous segment's epilogue is done with the buffers
 
   int q0, qlen;
-  if (p.qsl) { q0 = p.qsl[b]; qlen = p.qsl[b + 1] - q0; } else { q0 = b * p.max_q_len; qlen = p.max_q_len; }
-  qlen = qlen < p.max_q_len ? qlen : p.max_q_len;
+  {
+    KernArgPtr kp = cold();
+    const int32_t* qsl = kp->qsl;
+    const int mq = kp->max_q_len;
+    if (qsl) { q0 = qsl[b]; qlen = qsl[b + 1] - q0; } else { q0 = b * mq; qlen = mq; }
+    qlen = qlen < mq ? qlen : mq;
+  }
   const int rows = qlen * p.num_heads;
 
   // this lane's query row for QK / softmax; the four lanes l16 + 16*g share it
@@ -185,13 +202,20 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     limit = limit < 0 ? 0 : limit;
     if (g == 0) *(int*)(lds + kLimitOff + rloc * 4) = limit;  // read back by the blocks that have to mask (the last ones)
     *(float*)(lds + kSeenOff + threadIdx.x * 4) = -INFINITY;
+    // the two per-lane offsets of the K-fragment reads live in LDS and are fetched at the start of every QK phase (one
+    // read instead of two registers held through the P.V phase, where registers are short)
+    if (wave == 0) {
+      const u32x2 kr = {(uint32_t)(l16 * 1024 + (((g << 2) ^ swz_nope(l16)) << 4)),
+                        (uint32_t)(kRopeOff + l16 * 128 + (((g << 1) ^ swz_rope(l16)) << 4))};
+      *(u32x2*)(lds + kKTabOff + lane * 8) = kr;
+    }
   }
   const int win_skip = kWindow ? p.win_skip[b] : 0;
   const int win_blk0 = kWindow ? p.win_sink / kBlk : 0;
   const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
 
   if (grp * 128 >= rows) {
-    if (row < r_max && g == 0) { p.lse_part[part_base + rloc] = -INFINITY; p.corr_scale[part_base + rloc] = 0.f; }
+    if (row < r_max && g == 0) { KernArgPtr kp = cold(); kp->lse_part[part_base + rloc] = -INFINITY; kp->corr_scale[part_base + rloc] = 0.f; }
     continue;
   }
 
@@ -202,27 +226,47 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   // instructions per block, in the phase where that unit idles) instead of occupying registers through the loop.
   const uint32_t n_sr2 = (uint32_t)p.nope_sr * 2u, r_sr2 = (uint32_t)p.rope_sr * 2u;       // row strides in bytes
   const int swz_nw = swz_nope((wave * 4) & 15), swz_rw = swz_rope((wave * 4) & 15);        // scalars
+  // full blocks of the paged cache: the wave's row offsets ride in the per-lane offset (32 rows stay below 2^31 bytes,
+  // checked where the mode is chosen), so a copy is one vector instruction, one scalar add into M0 and the load
+  const bool full_ok = n_sr2 <= (1u << 25) && r_sr2 <= (1u << 25);
+  const uint32_t dma_off = (uint32_t)((lane ^ swz_nw) << 4);
+  uint32_t s_rowoff[4];
+#pragma unroll
+  for (int k = 0; k < 4; k++) s_rowoff[k] = (uint32_t)(wave * 4 + k) * n_sr2;
 
   ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (kSparse ? 0 : (int64_t)b * p.bt_stride);
-  ConstI32Ptr srows = (ConstI32Ptr)(p.sparse_rows) + (kSparse ? (int64_t)b * p.sparse_stride : 0);
   const int64_t max_row = p.num_pages * p.page_size - 1;
-  // Row list (kSparse): the 32 cache rows of the block whose copies go out next travel in one vector register, lane r
-  // holding the row of key r, and every copy picks its row with v_readlane.  The load for block X+1 is issued in front of
-  // the copies of block X, so the wait that lets a block's copies land also covers it (vector memory returns in order).
-  uint32_t ids_cur = 0, ids_nxt = 0;
-  auto ids_load = [&](int blk_x) {
+  // The hardware lane number behind an opaque (and volatile) statement: what is derived from it inside the loop is
+  // computed inside the loop.  Left alone the compiler hoists every loop-invariant LDS address out of the block loop, a
+  // dozen registers of them, and then spills them - and a scratch reload waits for every copy in flight.
+  auto lane_now = [] {
+    int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(ln));
+    return ln;
+  };
+  // Row list (kSparse): a wave copies rows 4w..4w+3 of a block and needs the cache rows of exactly those four keys.  They
+  // are fetched one block ahead by a four-lane global -> LDS copy into the wave's own slot (no register is the target of
+  // a load in flight, so nothing the compiler does with registers in between can lose them), issued in front of the
+  // copies of the previous block so that the wait that lets those land covers it, and read back when the copies are due.
+  // Keys past the end of the list name its last key (their scores are masked).
+  int32_t ids_rope = 0;                                       // cache row of this lane's rope row (lanes 0..31)
+  int32_t ids_row[4] = {0, 0, 0, 0};                          // cache rows of the wave's four keys (uniform)
+  auto ids_dma = [&](int blk_x) {
     if constexpr (kSparse) {
-      int tok = blk_x * kBlk + (lane & 31);
+      int tok = blk_x * kBlk + wave * 4 + (lane_now() & 3);
       tok = tok < L ? tok : L - 1;
       tok = tok < 0 ? 0 : tok;
-      const int32_t* src = p.sparse_rows + (int64_t)b * p.sparse_stride + tok;
-      asm volatile("global_load_dword %0, %1, off" : "=v"(ids_nxt) : "v"(src) : "memory");
+      dma4_sv_lanes4(p.sparse_rows + (int64_t)b * p.sparse_stride, (uint32_t)tok * 4u, lds0 + kIdsOff + (blk_x & 3) * 128 + wave * 16);
     }
   };
-  auto ids_rotate = [&] {
+  auto ids_fetch = [&](int blk_x) {
     if constexpr (kSparse) {
-      asm volatile("" : "+v"(ids_nxt));
-      ids_cur = ids_nxt;
+      const int ln = lane_now();
+      const char* slot = lds + kIdsOff + (blk_x & 3) * 128 + wave * 16;
+      const int32_t mine = *(const int32_t*)(slot + (ln & 3) * 4);
+      ids_rope = *(const int32_t*)(slot + ((ln >> 3) & 3) * 4);
+#pragma unroll
+      for (int k = 0; k < 4; k++) ids_row[k] = __builtin_amdgcn_readlane(mine, k);
     }
   };
   auto load_page = [&](int page) -> int64_t {
@@ -232,16 +276,20 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   };
   int page_cur = 0;
   int64_t pg_nxt = 0;
-  const char* np_page = (const char*)p.nope;                  // first rows of the current page (64-bit products once per page)
-  const char* rp_page = (const char*)p.rope;
-  auto set_page = [&](int64_t pg) {
-    np_page = (const char*)p.nope + pg * p.nope_sp * 2;
-    rp_page = (const char*)p.rope + pg * p.rope_sp * 2;
+  // Blocks are copied in order, so the address of the next block's first row is a running pointer: 32 rows further
+  // inside a page, recomputed (64-bit products) only where a new page starts.
+  const char* np_blk = (const char*)p.nope;
+  const char* rp_blk = (const char*)p.rope;
+  const uint64_t n_blk_b = (uint64_t)n_sr2 * kBlk, r_blk_b = (uint64_t)r_sr2 * kBlk;
+  auto set_page = [&](int64_t pg, int cblk) {
+    np_blk = (const char*)p.nope + pg * p.nope_sp * 2 + (uint64_t)((cblk & 3) * kBlk) * n_sr2;
+    rp_blk = (const char*)p.rope + pg * p.rope_sp * 2 + (uint64_t)((cblk & 3) * kBlk) * r_sr2;
   };
   auto issue_reset = [&]() {
     if constexpr (!kSparse) {
-      page_cur = (blk_begin + (kWindow && blk_begin >= win_blk0 ? win_skip : 0)) >> 2;
-      set_page(load_page(page_cur));
+      const int cblk = blk_begin + (kWindow && blk_begin >= win_blk0 ? win_skip : 0);
+      page_cur = cblk >> 2;
+      set_page(load_page(page_cur), cblk);
       pg_nxt = load_page(page_cur + 1);
     }
   };
@@ -254,7 +302,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     r -= 3 * (int)(((uint32_t)r * 43691u) >> 17);             // r / 3 for r < 98304: one multiply, no division sequence
     return r;
   };
-  struct IssueCtx { const char* np; const char* rp; const char* a0; uint32_t nbuf, rbuf; int last, tok0; };
+  struct IssueCtx { const char* np; const char* rp; uint32_t nbuf, rbuf; int last, tok0; };
   auto issue_begin = [&](int blk) -> IssueCtx {
     IssueCtx c;
     c.tok0 = blk * kBlk;
@@ -270,65 +318,47 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       if (page != page_cur) {
         // the next page's number is only asked for here (raw: clamping it now would wait for the load); it is clamped
         // when it becomes the current page, four blocks later
-        if (kWindow && page != page_cur + 1) set_page(load_page(page));        // the jump from the sink to the window
-        else set_page(pg_nxt < 0 ? 0 : (pg_nxt >= p.num_pages ? p.num_pages - 1 : pg_nxt));
+        if (kWindow && page != page_cur + 1) set_page(load_page(page), cblk);  // the jump from the sink to the window
+        else set_page(pg_nxt < 0 ? 0 : (pg_nxt >= p.num_pages ? p.num_pages - 1 : pg_nxt), cblk);
         page_cur = page;
         const int pn = page + 1 < p.max_blocks ? page + 1 : p.max_blocks - 1;
         pg_nxt = bt[pn];
       }
-      const uint32_t row0 = (uint32_t)(cblk & 3) * kBlk;
-      c.np = np_page + (uint64_t)row0 * n_sr2;
-      c.rp = rp_page + (uint64_t)row0 * r_sr2;
+      c.np = np_blk;
+      c.rp = rp_blk;
+      np_blk += n_blk_b;
+      rp_blk += r_blk_b;
     }
-    c.a0 = c.np + (uint64_t)(wave * 4) * n_sr2;               // full dense blocks: running row address
     return c;
-  };
-  // The hardware lane number behind an opaque (and volatile) statement: what is derived from it inside the loop is
-  // computed inside the loop.  Left alone the compiler hoists every loop-invariant LDS address out of the block loop, a
-  // dozen registers of them, and then spills them - and a scratch reload waits for every copy in flight.
-  auto lane_now = [] {
-    int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    asm volatile("" : "+v"(ln));
-    return ln;
   };
   auto rope_lane_row = [&] { return (lane_now() >> 3) & 3; };                               // lane's row among the wave's four
   auto rope_lane_off = [&]() -> uint32_t {
     const int ln = lane_now(), t = (ln >> 3) & 3;
     return (uint32_t)(((ln & 7) ^ swz_rw ^ ((t & 1) << 2) ^ (t & 2)) << 4);                 // swz_rope(t) = (t0 << 2) | (t1 << 1)
   };
-  // kFull: every row of the block exists and the source is the paged cache; kVecIds (row list): rows come from ids_cur
-  auto issue_piece = [&](IssueCtx& c, int k, auto full, auto vec_ids) {
+  // kFull: every row of the block exists and the source is the paged cache
+  auto issue_piece = [&](IssueCtx& c, int k, auto full) {
     constexpr bool kFull = decltype(full)::value && !kSparse;
-    constexpr bool kVecIds = decltype(vec_ids)::value && kSparse;
     auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
-    auto row_of = [&](int re) -> int32_t {
-      if constexpr (kVecIds) return (int32_t)__builtin_amdgcn_readlane((int)ids_cur, re);
-      else return srows[c.tok0 + re];
-    };
+
     if (k < 4) {
       const int r = wave * 4 + k;
-      const uint32_t off = (uint32_t)((lane_now() ^ swz_nw ^ swz_nope(k)) << 4);
       if constexpr (kFull) {
-        dma16_sv(c.a0, off, c.nbuf + r * 1024);
-        c.a0 += n_sr2;
+        uint32_t d = dma_off;
+        asm volatile("" : "+v"(d));                           // (opaque: the four offsets are not precomputed and spilled)
+        dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + wave * 4096, k * 1024);
       } else {
+        const uint32_t off = (uint32_t)((lane_now() ^ swz_nw ^ swz_nope(k)) << 4);
         const int re = r < c.last ? r : c.last;
-        if constexpr (kSparse) dma16_sv(c.np + clampi(row_of(re)) * n_sr2, off, c.nbuf + r * 1024);
+        if constexpr (kSparse) dma16_sv(c.np + clampi(ids_row[k]) * n_sr2, off, c.nbuf + r * 1024);
         else dma16_sv(c.np + (uint64_t)re * n_sr2, off, c.nbuf + r * 1024);
       }
     } else {
       // the wave's four rope rows, 128 bytes each: half an instruction (lanes 32..63 sit out)
       if constexpr (kSparse) {
-        int32_t mine = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          const int r = wave * 4 + j;
-          const int32_t sj = row_of(r < c.last ? r : c.last);
-          mine = rope_lane_row() == j ? sj : mine;
-        }
-        dma16_v_lo32(c.rp + clampi(mine) * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+        dma16_v_lo32(c.rp + clampi(ids_rope) * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
       } else if constexpr (kFull) {
-        dma16_sv_lo32(c.rp + (uint64_t)(wave * 4) * r_sr2, (uint32_t)rope_lane_row() * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+        dma16_sv_lo32(c.rp, (uint32_t)(wave * 4 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
       } else {
         const int r = wave * 4 + rope_lane_row();
         const int re = r < c.last ? r : c.last;
@@ -339,36 +369,24 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   auto issue_block = [&](int blk) {
     IssueCtx c = issue_begin(blk);
 #pragma unroll
-    for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{}, std::integral_constant<bool, kSparse>{});
+    for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{});
   };
-  uint32_t ids_head[kLead] = {};
+  // Row list: the rows of the first kLead blocks are fetched together (one round trip) before any copy goes out
   auto issue_first = [&]() {
     issue_reset();
     if constexpr (kSparse) {
 #pragma unroll
-      for (int j = 0; j < kLead; j++) {
-        int tok = (blk_begin + j) * kBlk + (lane & 31);
-        tok = tok < L ? tok : L - 1;
-        tok = tok < 0 ? 0 : tok;
-        const int32_t* src = p.sparse_rows + (int64_t)b * p.sparse_stride + tok;
-        asm volatile("global_load_dword %0, %1, off" : "=v"(ids_head[j]) : "v"(src) : "memory");
-      }
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(ids_head[0]), "+v"(ids_head[1]), "+v"(ids_head[2])::"memory");
-      ids_cur = ids_head[0];
+      for (int j = 0; j < kLead; j++) ids_dma(blk_begin + j);
+      MLA_WAIT_VMCNT(0);
+      ids_fetch(blk_begin);
     }
     issue_block(blk_begin);
   };
   auto issue_next_two = [&]() {
-    if constexpr (kSparse) {
-#pragma unroll
-      for (int j = 1; j < kLead; j++)
-        if (j < nb) {
-          ids_cur = ids_head[j];
-          issue_block(blk_begin + j);
-        }
-    } else {
 #pragma unroll 1
-      for (int j = 1; j < kLead && j < nb; j++) issue_block(blk_begin + j);
+    for (int j = 1; j < kLead && j < nb; j++) {
+      ids_fetch(blk_begin + j);
+      issue_block(blk_begin + j);
     }
   };
 
@@ -378,15 +396,16 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   {
     const int64_t tq = row_ok ? (q0 + t_local) : q0;         // rows that do not exist read row 0 of the sequence
     const int64_t hq = row_ok ? head : 0;
-    // Contraction step kk of the latent part covers the 16-byte granules 16*(kk/4) + 4g' + kk%4, g' = 0..3, and lane group
+    // Contraction step kk of the latent part covers the 16-byte granules 16*(kk%4) + 4g' + kk/4, g' = 0..3, and lane group
     // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
     // in one aligned 32-byte piece of a row, or the LDS serves the instruction at half rate (measured: 126 against 227
     // bytes per clock and CU with eight wavefronts reading).
-    const __bf16* qn = p.q_nope + tq * p.qn_st + hq * p.qn_sh + g * 32;
-    const __bf16* qr = p.q_rope + tq * p.qr_st + hq * p.qr_sh + g * 16;
+    KernArgPtr kp = cold();
+    const __bf16* qn = kp->q_nope + tq * kp->qn_st + hq * kp->qn_sh + g * 32;
+    const __bf16* qr = kp->q_rope + tq * kp->qr_st + hq * kp->qr_sh + g * 16;
 #pragma unroll
     for (int kk = 0; kk < 16; kk++)
-      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[kk]) : "v"(qn), "i"((kk >> 2) * 256 + (kk & 3) * 16));
+      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[kk]) : "v"(qn), "i"((kk & 3) * 256 + (kk >> 2) * 16));
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[16 + kk]) : "v"(qr), "i"(kk * 16));
     __builtin_amdgcn_s_waitcnt(0x0F70);                                         // vmcnt(0)
@@ -407,8 +426,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   int top_tag = -1;              // ... and where: (block << 3) | element number
 
   // ---- per-lane LDS offsets ----
-  const uint32_t kbase = (uint32_t)(l16 * 1024 + (((g << 2) ^ swz_nope(l16)) << 4));      // ^ ((kk&3) << 4), offset kg*16384 + (kk>>2)*256
-  const uint32_t rbase = (uint32_t)(kRopeOff + l16 * 128 + (((g << 1) ^ swz_rope(l16)) << 4));   // ^ ((kk-16) << 4), offset kg*2048
+  // K-fragment reads: latent part at kbase ^ ((kk>>2) << 4), offset kg*16384 + (kk&3)*256; rope part at
+  // rbase ^ ((kk-16) << 4), offset kg*2048 (kbase, rbase: the table at kKTabOff)
   const int g16 = lane >> 4, j16 = lane & 15;
   const int v_row = 4 * (g16 >> 1) + (j16 >> 2);              // + 8*rd + 16*kb
   const int v_cl = 2 * (g16 & 1) + ((j16 & 3) >> 1);
@@ -423,7 +442,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   // (n = row % 32, h) holding keys 16kb + {4h..4h+3, 8+4h..8+4h+3}.  The QK lane (row l16 of wave w, group g) holds keys
   // 16kg + 4g + {0..3}: they are the first (g < 2) or second (g >= 2) 8 bytes of lane (n, h = g & 1).
   const uint32_t p_w_off = (uint32_t)(kPOff + (((wave >> 1) * 2) * 64 + (g & 1) * 32 + (wave & 1) * 16 + l16) * 16 + (g >> 1) * 8);   // + kg*1024 + parity*8192
-  const uint32_t p_r_off = (uint32_t)(kPOff + lane * 16);     // + (rg*2 + kb)*1024 + parity*8192
 
   // S^T for block `blk`: hand-placed K-fragment reads kAhead fragments ahead of the MFMA that consumes them, explicit
   // lgkmcnt waits, MFMAs as assembly with the scores in ordinary vector registers (the accumulation file is full of
@@ -434,18 +452,19 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     constexpr bool kIssue = kIssueMode != 0;
     // the six addresses the 36 reads use (the rest is immediate offsets)
     uint32_t na[4], ra[2];
-    na[0] = lds0 + (blk & 3) * kNopeBufB + kbase;
-    ra[0] = lds0 + rope_buf_of(blk) * kRopeBufB + rbase;
+    const u32x2 kr = *(const u32x2*)(lds + kKTabOff + lane_now() * 8);
+    na[0] = lds0 + (blk & 3) * kNopeBufB + kr[0];
+    ra[0] = lds0 + rope_buf_of(blk) * kRopeBufB + kr[1];
 #pragma unroll
     for (int b4 = 1; b4 < 4; b4++) na[b4] = na[0] ^ (uint32_t)(b4 << 4);
     ra[1] = ra[0] ^ 16u;
     IssueCtx ic;
-    if constexpr (kIssue) { ids_load(blk_issue + 1); ic = issue_begin(blk_issue); }
+    if constexpr (kIssue) { ids_dma(blk_issue + 1); ic = issue_begin(blk_issue); }
     bf16x8 ka[kAhead];
     // fragment j: contraction step kk = j >> 1, key group kg = j & 1; each statement is wait + MFMA + the read that
     // refills the fragment register (one statement, so that nothing is scheduled or padded in between)
-#define MLA_K_ADDR(j) (((j) >> 1) < 16 ? na[((j) >> 1) & 3] : ra[((j) >> 1) - 16])
-#define MLA_K_OFF(j) (((j) >> 1) < 16 ? ((j) & 1) * 16384 + ((j) >> 3) * 256 : ((j) & 1) * 2048)
+#define MLA_K_ADDR(j) (((j) >> 1) < 16 ? na[(j) >> 3] : ra[((j) >> 1) - 16])
+#define MLA_K_OFF(j) (((j) >> 1) < 16 ? ((j) & 1) * 16384 + (((j) >> 1) & 3) * 256 : ((j) & 1) * 2048)
 #if defined(ABL_QK_NOREAD)
 #define RD "; "
 #else
@@ -471,11 +490,14 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       else
         asm volatile("s_waitcnt lgkmcnt(%3)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+v"(s[j & 1]) : "v"(ka[j % D]), "v"(qf[j >> 1]), "i"(younger));
-      if constexpr (kIssue) if (j % 7 == 3) issue_piece(ic, j / 7, std::integral_constant<bool, kIssueMode == 2>{}, std::true_type{});
+      if constexpr (kIssue) if (j % 7 == 3) issue_piece(ic, j / 7, std::integral_constant<bool, kIssueMode == 2>{});
     }
 #undef MLA_K_ADDR
 #undef MLA_K_OFF
     asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s[0]), "+v"(s[1]));
+#ifdef ABL_QK_NOMFMA
+    s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0];
+#endif
   };
 
   // ---- softmax + P.V, hand-ordered ----
@@ -520,7 +542,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     const uint32_t vb = lds0 + (blk & 3) * kNopeBufB;
     const uint32_t a0 = vb + vbase[0], a1 = vb + vbase[1];    // ^ 64 for the second 32 columns, + 16384 for the second k-block
     const uint32_t a0x = a0 ^ 64u, a1x = a1 ^ 64u;
-    const uint32_t pa = lds0 + (blk & 1) * kPBufB + p_r_off;  // + (rg*2 + kb)*1024
+    const uint32_t pa = lds0 + (blk & 1) * kPBufB + kPOff + ((uint32_t)lane_now() << 4);   // + (rg*2 + kb)*1024
     bf16x4 v0l, v0h, v1l, v1h;
     bf16x8 pr0, pr1;
 #define PV_VREAD(kb)                                                                                                   \
@@ -636,7 +658,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       issue_first();
       restart = false;
     }
-    ids_load(blk_begin + kLead);                              // (older than the copies below: their wait covers it)
+    ids_dma(blk_begin + kLead);                               // (older than the copies below: their wait covers it)
     issue_next_two();
     // ---- block 0: QK, softmax, publish ----
     {
@@ -661,7 +683,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     }
     // Everything the loop keeps in registers is touched here: a value that was parked in scratch during the prologue is
     // brought back (and waited for) now, not at its first use inside the loop.
-    asm volatile("" :: "v"(kbase), "v"(rbase), "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(p_r_off), "v"(p_w_off));
+    asm volatile("" :: "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(p_w_off), "v"(dma_off));
     // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
     for (int i = 0; i + 1 < nb; i++) {
       const int blk = blk_begin + i;
@@ -669,8 +691,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
       if (i + 2 < nb) MLA_WAIT_VMCNT(5); else MLA_WAIT_VMCNT(0);
       TR_ADD(0);
-      ids_rotate();
       lds_barrier();
+      if (i + kLead < nb) ids_fetch(blk + kLead);             // (row list) the rows of the block whose copies go out now
       TR_ADD(1);
       const int fl = flags_read(blk);
       f32x4 s[2];
@@ -678,11 +700,11 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0];
       if (true) {}                                            // no QK and no copies at all (never a copy past the segment)
 #elif defined(ABL_NO_COPY)
-      if (true) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
+      if (true) { qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0); s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0]; }
 #else
       if (i + kLead >= nb) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
 #endif
-      else if (kSparse || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead);
+      else if (kSparse || !full_ok || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead);
       else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + kLead);
       TR_ADD(2);
       if (restarts_left > 0 && flags_ask_restart(fl)) { restart = true; restarts_left--; break; }
@@ -743,29 +765,33 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     // Rows whose most probable key carries more than 1/16 of the weight leave a note for the merge kernel: the rounding
     // error of that key's probability (already divided by l) and the address of its latent vector in the cache.
     float corr = 0.f;
-    const __bf16* vrow = p.nope;
+    KernArgPtr kp = cold();
+    const __bf16* nope0 = kp->nope;
+    const __bf16* vrow = nope0;
     if (e_row_ok && top_tok >= 0 && top_p * 16.f > l_tot) {
       corr = (top_p - (float)(__bf16)top_p) * inv;
       if constexpr (kSparse) {
-        int64_t slot = p.sparse_rows[(int64_t)b * p.sparse_stride + top_tok];
+        int64_t slot = kp->sparse_rows[(int64_t)b * kp->sparse_stride + top_tok];
         slot = slot < 0 ? 0 : (slot > max_row ? max_row : slot);
-        vrow = p.nope + slot * p.nope_sr;
+        vrow = nope0 + slot * kp->nope_sr;
       } else {
-        const int ctok = top_tok + ((kWindow && top_tok >= p.win_sink) ? win_skip * kBlk : 0);   // position in the cache
+        const int ctok = top_tok + ((kWindow && top_tok >= kp->win_sink) ? win_skip * kBlk : 0);   // position in the cache
         int page = ctok / kPage;
-        page = page < p.max_blocks ? page : p.max_blocks - 1;
-        int64_t pg = p.block_table[(int64_t)b * p.bt_stride + page];
-        pg = pg < 0 ? 0 : (pg >= p.num_pages ? p.num_pages - 1 : pg);
-        vrow = p.nope + pg * p.nope_sp + (int64_t)(ctok % kPage) * p.nope_sr;
+        const int mb = kp->max_blocks;
+        page = page < mb ? page : mb - 1;
+        int64_t pg = kp->block_table[(int64_t)b * kp->bt_stride + page];
+        const int64_t np_ = kp->num_pages;
+        pg = pg < 0 ? 0 : (pg >= np_ ? np_ - 1 : pg);
+        vrow = nope0 + pg * kp->nope_sp + (int64_t)(ctok % kPage) * kp->nope_sr;
       }
     }
     if (e_g == 0) {
       *(float*)(lds + kPOff + (e_rloc & 31) * 16 + (e_rloc >> 5) * 4) = inv;
       if (e_row < r_max) {
         const int64_t pr = part_base + e_rloc;
-        p.lse_part[pr] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
-        p.corr_scale[pr] = corr;
-        p.corr_row[pr] = vrow;
+        kp->lse_part[pr] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
+        kp->corr_scale[pr] = corr;
+        kp->corr_row[pr] = vrow;
       }
     }
   }
@@ -774,6 +800,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   // transpose through this wave's private 16 KiB: 128 rows x 64 columns, fp16 (128 bytes per row, 8-byte slots XORed
   // with the row so that neither the writes nor the reads collide)
   char* stage = lds + wave * 16384;
+  _Float16* o_part_c = cold()->o_part;
 #pragma unroll
   for (int rg = 0; rg < 4; rg++) {
     const int srow = rg * 32 + e_h32;
@@ -796,7 +823,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     const int srow = it * 4 + e_g;
     const u32x2 v = *(const u32x2*)(stage + srow * 128 + ((e_l16 ^ ((srow >> 1) & 15)) << 3));
     if (grp * 128 + srow < r_max)
-      *(u32x2*)(p.o_part + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
+      *(u32x2*)(o_part_c + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }  // segments

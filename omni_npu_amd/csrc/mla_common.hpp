@@ -69,6 +69,13 @@ __device__ __forceinline__ void dma16_sv(const void* gbase_uniform, uint32_t vof
                : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
                : "memory", "m0");
 }
+// the same with the LDS address given as a uniform base plus a compile-time constant (one scalar add straight into M0)
+__device__ __forceinline__ void dma16_sv_m0add(const void* gbase_uniform, uint32_t voff, uint32_t lds_base_uniform, int lds_imm) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_base_uniform), "v"(voff), "s"(gbase_uniform), "n"(lds_imm)
+               : "memory", "m0", "scc");
+}
 // source = per-lane 64-bit address
 __device__ __forceinline__ void dma16_v(const void* gaddr, uint32_t lds_addr_uniform) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
@@ -91,6 +98,16 @@ __device__ __forceinline__ void dma16_v_lo32(const void* gaddr, uint32_t lds_add
   asm volatile("s_mov_b32 %0, exec_hi\n\ts_mov_b32 exec_hi, 0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 exec_hi, %0"
                : "=&s"(save)
                : "s"(lds_addr_uniform), "v"(gaddr)
+               : "memory", "m0");
+}
+
+// Four dwords by lanes 0..3 (the rest of the execution mask is cleared around the instruction): lane i's dword lands at
+// lds_addr + 4 * i.
+__device__ __forceinline__ void dma4_sv_lanes4(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  uint64_t save;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 15\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\ts_mov_b64 exec, %0"
+               : "=&s"(save)
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
                : "memory", "m0");
 }
 
