@@ -116,6 +116,21 @@ int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h
                     void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out /* fp32 [T,N] or NULL */,
                     void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
 
+/* The same decode without a workspace argument, for callers that cannot allocate or hand one over: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  (No counterpart in the reference: its vendor op
+ * owns its scratch.)  The split-KV partials live in a device array built into the library,
+ * MLA_DECODE_STATIC_SCRATCH_BYTES per GPU, held until the process ends; a shape that needs more
+ * (mla_decode_workspace_bytes) is refused with -4.  The call allocates and frees nothing.  Calls that overlap in time
+ * on one GPU share the array and race: keep them on one stream or order them with events. */
+#define MLA_DECODE_STATIC_SCRATCH_BYTES ((size_t)48 << 20)
+int mla_decode_bf16_static(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                           int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,
+                           int64_t nope_row_stride, const void* rope_cache, int64_t rope_page_stride,
+                           int64_t rope_row_stride, int64_t num_pages, const int32_t* block_table, int64_t bt_stride,
+                           int32_t max_blocks, const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                           int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                           int64_t out_stride_h, float* lse_out, int32_t num_splits, mlahip_stream_t stream);
+
 int mla_decode_bf16_split(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
                           int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_page_stride,
                           int64_t nope_row_stride, const void* rope_cache, int64_t rope_page_stride,

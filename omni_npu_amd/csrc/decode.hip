@@ -12,6 +12,7 @@
 // normalised fp16 partials [slots, rows, 512], fp32 log-sum-exps [slots, rows], a correction record per row (fp32
 // factor + cache address of the row's dominant key) and two partial numbers per sequence.
 #include <cstdlib>
+#include <mutex>
 #include "mla_common.hpp"
 #include "decode_v2_params.hpp"
 
@@ -224,6 +225,60 @@ extern "C" int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t 
   if (rc != MLA_OK) return rc;
   return mla_splitkv_reduce(workspace, workspace_bytes, seq_lens, query_start_loc, batch, max_q_len, num_heads, num_splits,
                             out, out_stride_t, out_stride_h, lse_out, stream);
+}
+
+// The same decode for callers that cannot allocate or hand over a workspace (code under HIP graph capture, serving loops,
+// harnesses that forbid hipMalloc): the split-KV partials live in a file-scope device array of kStaticScratchBytes.
+// Every GPU the library runs on holds its own copy of the array at its own address for the life of the process; the
+// address is looked up once per device (hipGetSymbolAddress) and from then on only that pointer is used.  Calls that
+// overlap in time on one GPU share the array and race; calls on one stream, or ordered by events, do not.  Nothing has
+// to start at zero: the split phase writes every partial, log-sum-exp, correction record and segment number the merge
+// reads (the merge derives which ones exist from seq_lens, as the split does).
+namespace mlahip {
+constexpr size_t kStaticScratchBytes = (size_t)48 << 20;   // 48 MiB: the headline step (64 x 128 heads, 4 splits) needs 42.6 MB
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];                    // per device, nullptr = not looked up yet
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(MLA_ERR_LAUNCH, "mla_decode_bf16_static: no current device (hipGetDevice gave %d)", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(MLA_ERR_LAUNCH, "mla_decode_bf16_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MLA_OK;
+}
+}  // namespace mlahip
+
+extern "C" int mla_decode_bf16_static(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                      int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache,
+                                      int64_t nope_page_stride, int64_t nope_row_stride, const void* rope_cache,
+                                      int64_t rope_page_stride, int64_t rope_row_stride, int64_t num_pages,
+                                      const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                      const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                                      int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                                      int64_t out_stride_h, float* lse_out, int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1, MLA_ERR_SHAPE,
+              "mla_decode_bf16_static: batch=%d max_q_len=%d num_heads=%d num_splits=%d", batch, max_q_len, num_heads, num_splits);
+  const size_t need = mla_decode_workspace_bytes(batch, max_q_len, num_heads, num_splits);
+  MLA_REQUIRE(need <= kStaticScratchBytes, MLA_ERR_WORKSPACE,
+              "mla_decode_bf16_static: this shape needs %zu bytes of split-KV scratch, the built-in array holds %zu; "
+              "use mla_decode_bf16 with a caller-owned workspace", need, (size_t)kStaticScratchBytes);
+  void* ptr = nullptr;
+  const int rc = static_scratch(&ptr);
+  if (rc != MLA_OK) return rc;
+  return mla_decode_bf16(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache, nope_page_stride,
+                         nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages, block_table, bt_stride,
+                         max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads, scale, out, out_stride_t,
+                         out_stride_h, lse_out, ptr, kStaticScratchBytes, num_splits, stream);
 }
 
 // Sparse absorbed MLA over a per-token list of cache rows (reference: npu_sparse_flash_attention as called in
