@@ -185,6 +185,14 @@ int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_str
                      int32_t in_dtype, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
                      float* out_lse /* may be NULL */, int32_t tokens, int32_t heads, int32_t dim, mlahip_stream_t stream);
 
+/* N-way merge: replaces attention_update_torch (attention/ops.py:109-141), the torch stand-in of
+ * torch_npu.npu_attention_update: outs [n, T, D] (dtype code 0 = bf16, 1 = fp32, 2 = fp16; last dimension contiguous),
+ * lses fp32 [n, T] -> out fp32 [T, D], lse_out fp32 [T] (may be NULL).  +inf log-sum-exps read as -inf; a row whose
+ * partials all weigh nothing gives zeros and -inf.  One launch for any n. */
+int mla_merge_n_states(const void* outs, int64_t outs_stride_n, int64_t outs_stride_t, int32_t in_dtype, const float* lses,
+                       int64_t lses_stride_n, float* out, int64_t out_stride_t, float* lse_out, int32_t n, int32_t tokens,
+                       int32_t dim, mlahip_stream_t stream);
+
 /* ---- non-absorbed varlen attention for prefill -------------------------------------------
  * Replaces the prefill calls of npu_fused_infer_attention_score, attention/backends/mla.py:574-590 (suffix:
  * right-down causal, sparse_mode 3) and :415-431 (context chunk: no mask, softmax_lse_flag): q_nope [T,N,128],

@@ -49,24 +49,15 @@ def merge_attn_states(
 
 def attention_update_torch(outs, lses):
     """N-way merge (reference ops.py:109-141): outs [n, T, D] (or list), lses [n, T] -> (out fp32 [T, D], lse fp32 [T]).
-    Folded pairwise with the two-way merge kernel (the merge is associative)."""
+    One launch of the N-way merge kernel for any n."""
     if type(outs) is list:
         assert type(lses) is list and len(outs) == len(lses)
         outs = torch.stack(outs, dim=0)
         lses = torch.stack(lses, dim=0)
     assert outs.dim() == 3 and lses.dim() == 2
     assert outs.size(0) == lses.size(0) and outs.size(1) == lses.size(1)
-    n, t, d = outs.shape
-    acc = outs[0].float().contiguous().view(t, 1, d)
-    acc_lse = lses[0].float().contiguous().view(t, 1)
-    for i in range(1, n):
-        nxt, nxt_lse = torch.empty_like(acc), torch.empty_like(acc_lse)
-        K.merge_states(acc, acc_lse, outs[i].float().contiguous().view(t, 1, d), lses[i].float().contiguous().view(t, 1),
-                       nxt, nxt_lse)
-        acc, acc_lse = nxt, nxt_lse
-    if n == 1:   # same conventions as the merge: +inf reads as -inf, an empty row is zeros
-        z, zl = torch.zeros_like(acc), torch.full_like(acc_lse, float("-inf"))
-        nxt, nxt_lse = torch.empty_like(acc), torch.empty_like(acc_lse)
-        K.merge_states(acc, acc_lse, z, zl, nxt, nxt_lse)
-        acc, acc_lse = nxt, nxt_lse
-    return acc.view(t, d), acc_lse.view(t)
+    if outs.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        outs = outs.float()
+    if outs.stride(-1) != 1:
+        outs = outs.contiguous()
+    return K.merge_n_states(outs, lses)

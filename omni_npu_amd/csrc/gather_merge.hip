@@ -70,8 +70,65 @@ __global__ __launch_bounds__(256) void merge_states_kernel(const TIn* po, int64_
   if (out_lse && lane == 0) out_lse[r] = lse;
 }
 
+// N-way merge of attention partials (src/omni_npu/attention/ops.py:109-141): outs [n, T, D], lses [n, T] ->
+// out fp32 [T, D], lse fp32 [T].  +inf log-sum-exps read as -inf; a row whose partials all weigh nothing gives zeros
+// and -inf; a partial with zero weight contributes nothing even if it holds NaN / inf garbage.  One wavefront per row:
+// the weights are worked out once (lane p holds partial p, up to 64 at a time), then the lanes walk the row's columns.
+template <typename TIn>
+__global__ __launch_bounds__(256) void merge_n_states_kernel(const TIn* __restrict__ outs, int64_t o_sn, int64_t o_st,
+                                                            const float* __restrict__ lses, int64_t l_sn,
+                                                            float* __restrict__ out, int64_t out_st, float* __restrict__ lse_out,
+                                                            int32_t n, int32_t tokens, int32_t dim) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= tokens) return;
+  auto lse_of = [&](int q) -> float {
+    float l = q < n ? lses[(int64_t)q * l_sn + t] : -INFINITY;
+    return l == INFINITY ? -INFINITY : l;
+  };
+  float m = -INFINITY;
+  for (int q0 = 0; q0 < n; q0 += 64) m = fmaxf(m, lse_of(q0 + lane));
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, 64));
+  float se = 0.f;
+  if (m != -INFINITY)
+    for (int q0 = 0; q0 < n; q0 += 64) se += __expf(lse_of(q0 + lane) - m);
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) se += __shfl_xor(se, d, 64);
+  const bool valid = se > 0.f;                              // (false also for NaN)
+  for (int i = lane; i < dim; i += 64) {
+    float a = 0.f;
+    if (valid)
+      for (int q = 0; q < n; q++) {
+        const float w = __expf(lse_of(q) - m) / se;
+        if (w > 0.f) a += ld(outs + (int64_t)q * o_sn + t * o_st + i) * w;
+      }
+    out[t * out_st + i] = a;
+  }
+  if (lse_out && lane == 0) lse_out[t] = valid ? __logf(se) + m : -INFINITY;
+}
+
 }  // namespace mlahip
 using namespace mlahip;
+
+// dtype codes: 0 = bf16, 1 = fp32, 2 = fp16
+extern "C" int mla_merge_n_states(const void* outs, int64_t outs_stride_n, int64_t outs_stride_t, int32_t in_dtype,
+                                  const float* lses, int64_t lses_stride_n, float* out, int64_t out_stride_t, float* lse_out,
+                                  int32_t n, int32_t tokens, int32_t dim, hipStream_t stream) {
+  MLA_REQUIRE(outs && lses && out, MLA_ERR_NULL, "mla_merge_n_states: null pointer argument");
+  MLA_REQUIRE(n >= 1 && tokens >= 0 && dim >= 1, MLA_ERR_SHAPE, "mla_merge_n_states: n=%d tokens=%d dim=%d", n, tokens, dim);
+  MLA_REQUIRE(in_dtype >= 0 && in_dtype <= 2, MLA_ERR_UNSUPPORTED, "mla_merge_n_states: dtype codes are 0 (bf16), 1 (fp32), 2 (fp16)");
+  if (tokens == 0) return MLA_OK;
+  const dim3 grid((unsigned)(((int64_t)tokens + 3) / 4)), block(256);
+#define MLA_MERGE_N(TI)                                                                                                  \
+  hipLaunchKernelGGL((merge_n_states_kernel<TI>), grid, block, 0, stream, (const TI*)outs, outs_stride_n, outs_stride_t, \
+                     lses, lses_stride_n, out, out_stride_t, lse_out, n, tokens, dim)
+  if (in_dtype == 0) MLA_MERGE_N(__bf16);
+  else if (in_dtype == 1) MLA_MERGE_N(float);
+  else MLA_MERGE_N(_Float16);
+#undef MLA_MERGE_N
+  return check_launch("mla_merge_n_states");
+}
 
 extern "C" int mla_gather_paged(const void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride,
                                 const void* rope_cache, int64_t rope_page_stride, int64_t rope_row_stride,

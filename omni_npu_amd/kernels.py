@@ -243,6 +243,38 @@ def merge_states(prefix_out: torch.Tensor, prefix_lse: torch.Tensor, suffix_out:
     _lib.check(rc, "mla_merge_states")
 
 
+def merge_n_states(outs: torch.Tensor, lses: torch.Tensor, out: Optional[torch.Tensor] = None,
+                   lse_out: Optional[torch.Tensor] = None):
+    """N-way log-sum-exp merge in one launch (reference: attention_update_torch, src/omni_npu/attention/ops.py:109-141).
+    outs [n,T,D] bf16 / fp16 / fp32 (last dim contiguous), lses fp32 [n,T] -> (out fp32 [T,D], lse fp32 [T])."""
+    _need_cuda(outs, lses, out, lse_out)
+    if outs.dim() != 3 or lses.dim() != 2 or outs.shape[:2] != lses.shape:
+        raise ValueError("merge_n_states: outs [n,T,D] and lses [n,T] expected")
+    codes = {torch.bfloat16: 0, torch.float32: 1, torch.float16: 2}
+    if outs.dtype not in codes:
+        raise TypeError("merge_n_states: bf16 / fp16 / fp32 partials only")
+    if outs.stride(-1) != 1:
+        raise ValueError("merge_n_states: last dim must be contiguous")
+    n, t, d = outs.shape
+    lses = lses.float()
+    if lses.stride(-1) != 1:
+        lses = lses.contiguous()
+    if out is None:
+        out = torch.empty(t, d, dtype=torch.float32, device=outs.device)
+    if lse_out is None:
+        lse_out = torch.empty(t, dtype=torch.float32, device=outs.device)
+    if out.dtype != torch.float32 or out.shape != (t, d) or out.stride(-1) != 1 or lse_out.dtype != torch.float32 or \
+            lse_out.numel() != t or not lse_out.is_contiguous():
+        raise TypeError("merge_n_states: out fp32 [T,D] (rows contiguous) and lse_out fp32 [T] expected")
+    if n == 0:
+        raise ValueError("merge_n_states: at least one partial")
+    rc = _lib.load().mla_merge_n_states(outs.data_ptr(), outs.stride(0), outs.stride(1), codes[outs.dtype], lses.data_ptr(),
+                                        lses.stride(0), out.data_ptr(), out.stride(0), lse_out.data_ptr(), n, t, d,
+                                        _stream(out))
+    _lib.check(rc, "mla_merge_n_states")
+    return out, lse_out
+
+
 # ------------------------------------------------------------------------------------------------
 _workspaces: dict = {}
 

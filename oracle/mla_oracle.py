@@ -13,12 +13,16 @@ Pinning status (what checks each function beyond re-typing its formula lives in
 
 * ``cache_write``                 closed form (row scatter); slot formula from
                                   tests/integration/attention/test_npu_mla_math.py:201-223.  pinned.
-* ``gather_paged``                restates attention/ops.py:5-41; pinned by the scatter/gather round trip
-                                  and by brute-force indexing.
+* ``gather_paged``                restates attention/ops.py:5-41; pinned by the scatter/gather round trip,
+                                  by brute-force indexing, and by a vector written by the reference function
+                                  itself (tests/golden/ops_vectors.npz, tests/test_ops_golden.py).
 * ``merge_attn_states``,
   ``attention_update``            restate attention/ops.py:44-106 and :109-141; pinned by the identity
                                   "merge of chunk results == one softmax over the concatenation", by the
-                                  -inf / +inf special cases, and by fold associativity.
+                                  -inf / +inf special cases, by fold associativity, and - for the conventions
+                                  mathematics does not fix (+inf reads as -inf, rows without weight) - by
+                                  vectors written by the reference functions themselves
+                                  (tests/golden/make_ops_vectors.py imports that one file, which needs only torch).
 * ``absorbed_decode``             restates tests/integration/attention/test_npu_mla_math.py:516-539;
                                   pinned by L=1, all-equal-K, block-table permutation invariance, a
                                   float64 brute-force loop, and the absorbed == non-absorbed equivalence.
@@ -52,8 +56,10 @@ Pinning status (what checks each function beyond re-typing its formula lives in
                                   position 0 = de-interleave only, q.k depends on the position difference only)
                                   and agreement of the two output layouts up to the fixed permutation.
 * ``fp8 quantise / dequantise``   PARITY UNPINNED against the reference (it has no fp8 KV format,
-                                  attention/ops.py:11-12 ignores its scale); pinned by the round-trip error
-                                  bound of e4m3 (relative 2^-4 per element, exact for representable values).
+                                  attention/ops.py:11-12 ignores its scale); the block and the per-token
+                                  quantiser are each pinned by their closed form: scale = amax / 448 exactly
+                                  (1.0 for zeros), the extreme lands on +-448, half-ulp error bound per binade,
+                                  grid values and ties-to-even survive exactly, power-of-two scaling invariance.
 """
 from __future__ import annotations
 
