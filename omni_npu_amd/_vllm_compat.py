@@ -119,11 +119,17 @@ except Exception:  # vLLM absent: stand-ins
 
         @property
         def page_size_bytes(self) -> int:
-            return self.block_size * self.num_kv_heads * self.head_size * torch.empty((), dtype=self.dtype).element_size()
+            # keys and values: twice the row (vLLM's AttentionSpec)
+            return 2 * self.block_size * self.num_kv_heads * self.head_size * torch.empty((), dtype=self.dtype).element_size()
 
     @dataclass
     class MLAAttentionSpec(AttentionSpec):
         cache_dtype_str: Optional[str] = None
+
+        @property
+        def page_size_bytes(self) -> int:
+            # one latent row per token serves as key and value (vLLM's MLAAttentionSpec)
+            return self.block_size * self.num_kv_heads * self.head_size * torch.empty((), dtype=self.dtype).element_size()
 
     @dataclass
     class CommonAttentionMetadata:

@@ -149,6 +149,7 @@ class LightningIndexer:
         self.topk_tokens, self.n_head, self.head_dim = topk_tokens, n_head, head_dim
         self.topk_indices_buffer = torch.full((max_tokens, topk_tokens), -1, dtype=torch.int32, device=device)
         self._logits = None
+        self._logits_kept = []       # outgrown score buffers: a captured graph may still hold their address, never freed
 
     def __call__(self, q: torch.Tensor, k: torch.Tensor, weights: torch.Tensor, kv_cache, attn_metadata):
         if attn_metadata is None:                                   # profile run (patch_dsv32_indexer.py:104-112)
@@ -175,7 +176,12 @@ class LightningIndexer:
             max_len = meta.block_table.shape[1] * k8.shape[1]
             stride = K.indexer_logits_stride(max_len)
             if self._logits is None or self._logits.shape[0] < ntok or self._logits.shape[1] < stride:
-                self._logits = torch.empty(max(ntok, 1), stride, dtype=torch.float32, device=q.device)
+                if self._logits is not None:
+                    self._logits_kept.append(self._logits)
+                    ntok_a, stride_a = max(ntok, self._logits.shape[0]), max(stride, self._logits.shape[1])
+                else:
+                    ntok_a, stride_a = max(ntok, 1), stride
+                self._logits = torch.empty(ntok_a, stride_a, dtype=torch.float32, device=q.device)
             lg = self._logits[:ntok, :stride]
             sl = slice(off, off + ntok)
             K.indexer_scores(q8[sl], w[sl], k8, ks, meta.block_table, lens, lg, q_len=q_len, q_scale=qs[sl],
@@ -207,6 +213,9 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
                 "encoder/decoder cross-attention "
                 "are not implemented for "
                 "NPUDSAImpl")
+        if kv_cache_dtype in ("fp8", "fp8_e4m3"):
+            raise NotImplementedError("NPUDSAImpl writes the bf16 cache layout (latent, rope, indexer keys) only: "
+                                      "an fp8 KV cache is not supported for DSA models")
 
     def _v_up_proj(self, x: torch.Tensor, out: torch.Tensor):
         """[T,N,512] token-major -> out [T, N*V]  (reference dsa.py:233-240)."""
@@ -239,10 +248,10 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         K.build_sparse_rows(topk_indices.reshape(bs, k), meta.block_table, lens, nope.shape[1], nope.shape[0], rows, counts,
                             q_len=q_len, query_start_loc=qsl)
         if proj_out is not None:
-            K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, proj_out, w_uv=self.W_UV)
+            K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, proj_out, w_uv=self.W_UV, counts_bounded=True)
             return None
         out = torch.empty(bs, self.num_heads, self.kv_lora_rank, dtype=q_nope.dtype, device=q_nope.device)
-        K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, out)
+        K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, out, counts_bounded=True)
         return out
 
     def forward(self, layer, q: torch.Tensor, k_c_normed: torch.Tensor, k_pe: torch.Tensor,
@@ -255,6 +264,12 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         if attn_metadata is None:
             _ = torch.empty((self.chunked_prefill_workspace_size, self.num_heads,
                              self.qk_nope_head_dim + self.v_head_dim), device=k_c_normed.device, dtype=k_c_normed.dtype)
+            # the profile run sizes the KV cache: the split-KV scratch a real prefill will need (bounded by
+            # SPARSE_WORKSPACE_CAP whatever the chunk size) is allocated now, so that it is counted
+            if k_c_normed.is_cuda:
+                toks = max(int(k_c_normed.shape[0]), 1)
+                need = K._lib.load().mla_decode_workspace_bytes(min(toks, 32768), 1, self.num_heads, 1)
+                K._workspace(k_c_normed.device, min(need, K.SPARSE_WORKSPACE_CAP))
             return output.fill_(0)
 
         num_actual_toks = attn_metadata.num_actual_tokens

@@ -280,12 +280,26 @@ _workspaces: dict = {}
 
 
 def _workspace(dev: torch.device, nbytes: int, tag: str = "decode") -> torch.Tensor:
-    key = (dev.index, tag)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
-        _workspaces[key] = ws
-    return ws
+    """Scratch memory of at least ``nbytes``, kept per (device, stream, tag).
+
+    A buffer handed out once is NEVER freed: a HIP graph captured earlier holds its address, and memory returned to the
+    caching allocator would be given to other tensors while replays of that graph still write split-KV partials into it.
+    When a later call needs more, a new buffer (at least 1.5 x the old size) is allocated next to the old ones, which stay
+    alive; an earlier graph keeps using the buffer it captured.  Buffers are not shared between streams, so steps running
+    concurrently on different streams do not write into each other's partials.  Callers that want to own the lifetime pass
+    ``workspace=`` instead."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream, tag)
+    bufs = _workspaces.setdefault(key, [])
+    if bufs and bufs[-1].numel() >= nbytes:
+        return bufs[-1]
+    size = max(nbytes, 1, (bufs[-1].numel() * 3) // 2 if bufs else 0)
+    bufs.append(torch.empty(size, dtype=torch.uint8, device=dev))
+    return bufs[-1]
+
+
+# Sparse MLA over many tokens (a DSA prefill chunk) runs in launches of at most this much split-KV scratch, so the scratch
+# does not grow with the prefill chunk (128 heads, one split: about 970 tokens per launch)
+SPARSE_WORKSPACE_CAP = 256 << 20
 
 
 def default_num_splits(batch: int, max_q_len: int, num_heads: int, max_seq_len: int, num_cus: int = 256) -> int:
@@ -578,10 +592,15 @@ def build_sparse_rows(indices: torch.Tensor, block_table: torch.Tensor, seq_lens
 def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor, rope_cache: torch.Tensor,
                   rows: torch.Tensor, counts: torch.Tensor, scale: float, out: torch.Tensor,
                   lse_out: Optional[torch.Tensor] = None, num_splits: Optional[int] = None,
-                  workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None,
+                  counts_bounded: bool = False) -> torch.Tensor:
     """Absorbed MLA of token t over cache rows rows[t, :counts[t]] (reference: npu_sparse_flash_attention call,
     src/omni_npu/attention/backends/dsa.py:259-291).  out bf16 viewed as [T,N,512]; with ``w_uv`` (bf16 [N,512,128])
-    the value up-projection of dsa.py:233-240 is fused into the merge and out is [T, N*128] / [T,N,128]."""
+    the value up-projection of dsa.py:233-240 is fused into the merge and out is [T, N*128] / [T,N,128].
+
+    counts[t] must not exceed rows.shape[1]; unless the caller vouches for that (``counts_bounded``: the counts come from
+    build_sparse_rows / topk_rows) they are clamped here.  Many tokens (a prefill chunk) run as several launches so that
+    the split-KV scratch stays below SPARSE_WORKSPACE_CAP and the launch below the grid limit."""
     _need_cuda(q_nope, q_rope, nope_cache, rope_cache, rows, counts, out)
     lib = _lib.load()
     nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
@@ -598,21 +617,34 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
             raise TypeError("sparse_decode: bf16 tensors with a contiguous last dim only")
     if rows.dtype != torch.int32 or counts.dtype != torch.int32 or rows.stride(-1) != 1 or not counts.is_contiguous():
         raise TypeError("sparse_decode: int32 rows [T,K] and counts [T]")
+    if lse_out is not None and (lse_out.dtype != torch.float32 or lse_out.numel() != t * n or not lse_out.is_contiguous()):
+        raise TypeError("sparse_decode: lse_out must be contiguous fp32 [T,N]")
+    if not counts_bounded:
+        counts = counts[:t].clamp(max=rows.shape[1])
     if num_splits is None:
         num_splits = default_num_splits(t, 1, n, rows.shape[1])
-    need = lib.mla_decode_workspace_bytes(t, 1, n, num_splits)
+    per_token = lib.mla_decode_workspace_bytes(1, 1, n, num_splits)
+    cap = workspace.numel() * workspace.element_size() if workspace is not None else SPARSE_WORKSPACE_CAP
+    step = max(1, min(t, cap // max(per_token, 1), 32768))
+    need = lib.mla_decode_workspace_bytes(min(step, max(t, 1)), 1, n, num_splits)
     ws = workspace if workspace is not None else _workspace(q_nope.device, need)
-    rc = lib.dsa_sparse_decode_bf16(
-        q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1),
-        nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[0],
-        nope.shape[1], rows.data_ptr(), rows.stride(0), counts.data_ptr(), t, n, float(scale),
-        out.data_ptr() if o3 is None else None, out.stride(0) if o3 is None else 0, out.stride(1) if o3 is None else 0,
-        lse_out.data_ptr() if lse_out is not None else None, ws.data_ptr(),
-        ws.numel() * ws.element_size(), num_splits, _stream(q_nope))
-    _lib.check(rc, "dsa_sparse_decode_bf16")
-    if o3 is not None:
-        _reduce_vup(lib, (ws.data_ptr(), ws.numel() * ws.element_size()), counts, None, t, 1, n, num_splits, t, w_uv, o3,
-                    _stream(q_nope))
+    ws_args = (ws.data_ptr(), ws.numel() * ws.element_size())
+    st = _stream(q_nope)
+    lse2 = lse_out.view(t, n) if lse_out is not None else None
+    for t0 in range(0, t, step):
+        t1 = min(t, t0 + step)
+        qn, qr, rw, ct = q_nope[t0:t1], q_rope[t0:t1], rows[t0:t1], counts[t0:t1]
+        oc = out[t0:t1] if o3 is None else None
+        rc = lib.dsa_sparse_decode_bf16(
+            qn.data_ptr(), qn.stride(0), qn.stride(1), qr.data_ptr(), qr.stride(0), qr.stride(1),
+            nope.data_ptr(), nope.stride(0), nope.stride(1), rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[0],
+            nope.shape[1], rw.data_ptr(), rw.stride(0), ct.data_ptr(), t1 - t0, n, float(scale),
+            oc.data_ptr() if oc is not None else None, oc.stride(0) if oc is not None else 0,
+            oc.stride(1) if oc is not None else 0, lse2[t0:t1].data_ptr() if lse2 is not None else None, *ws_args,
+            num_splits, st)
+        _lib.check(rc, "dsa_sparse_decode_bf16")
+        if o3 is not None:
+            _reduce_vup(lib, ws_args, ct, None, t1 - t0, 1, n, num_splits, t1 - t0, w_uv, o3[t0:t1], st)
     return out
 
 
@@ -692,6 +724,15 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
             raise TypeError("decode_fp8: bf16 queries / output with a contiguous last dim")
     if block_table.dtype != torch.int32 or seq_lens.dtype != torch.int32:
         raise TypeError("decode_fp8: block_table and seq_lens must be int32")
+    if block_table.dim() != 2 or block_table.shape[0] < b or block_table.stride(-1) != 1:
+        raise ValueError(f"decode_fp8: block_table must be [>= {b}, max_blocks] with contiguous rows, got {tuple(block_table.shape)}")
+    if not seq_lens.is_contiguous():
+        seq_lens = seq_lens.contiguous()
+    if query_start_loc is not None and (query_start_loc.dtype != torch.int32 or query_start_loc.numel() < b + 1 or
+                                        not query_start_loc.is_contiguous()):
+        raise TypeError("decode_fp8: query_start_loc must be contiguous int32 [B+1]")
+    if lse_out is not None and (lse_out.dtype != torch.float32 or lse_out.numel() != t * n or not lse_out.is_contiguous()):
+        raise TypeError("decode_fp8: lse_out must be contiguous fp32 [T,N]")
     if query_start_loc is None and t != b * q_len:
         raise ValueError(f"decode_fp8: {t} query tokens != batch {b} x q_len {q_len}")
     if max_seq_len is None:

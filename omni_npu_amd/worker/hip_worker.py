@@ -17,12 +17,17 @@ from .._vllm_compat import HAVE_VLLM, AttentionSpec, MLAAttentionSpec
 INDEX_HEAD_DIM_DEFAULT = 128
 
 
-def kv_cache_dtype_and_head_size(cache_dtype: str, model_dtype: torch.dtype, head_size: int):
-    """fp8 cache: 656 bytes per token in a uint8 tensor (512 e4m3 | 4 fp32 scales | 64 bf16 rope); otherwise head_size
-    elements of the model dtype."""
+def kv_cache_dtype_and_head_size(cache_dtype: str, model_dtype: torch.dtype, head_size: int, index_head_dim: int = 0):
+    """fp8 cache: 656 bytes per token in a uint8 tensor (512 e4m3 | 4 fp32 scales | 64 bf16 rope); otherwise
+    head_size + index_head_dim elements of the model dtype (the DSA layout keeps the indexer keys in the same pages).
+    An fp8 latent cache for a DSA model is refused: the 656-byte row has no room for the indexer keys and NPUDSAImpl writes
+    the bf16 layout only."""
     if cache_dtype in ("fp8", "fp8_e4m3"):
+        if index_head_dim:
+            raise NotImplementedError("an fp8 KV cache is not supported for DSA (indexer) models: the fp8 row layout holds "
+                                      "the 512 + 64 latent only; use kv_cache_dtype='auto'")
         return torch.uint8, K.FP8_ROW_BYTES
-    return model_dtype, head_size
+    return model_dtype, head_size + index_head_dim
 
 
 class KVCacheHooksMixin:
@@ -37,7 +42,7 @@ class KVCacheHooksMixin:
         extra = getattr(mc.hf_config, "index_head_dim", INDEX_HEAD_DIM_DEFAULT) if is_dsa else 0
         specs = {}
         for layer_name, attn_module in self._attention_layers().items():
-            dtype, head = kv_cache_dtype_and_head_size(cc.cache_dtype, mc.dtype, attn_module.head_size + extra)
+            dtype, head = kv_cache_dtype_and_head_size(cc.cache_dtype, mc.dtype, attn_module.head_size, extra)
             specs[layer_name] = MLAAttentionSpec(block_size=cc.block_size, num_kv_heads=1, head_size=head, dtype=dtype,
                                                  cache_dtype_str=cc.cache_dtype)
         return specs
