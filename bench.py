@@ -24,6 +24,52 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16
 
 
+def host_cpu():
+    """Model name and logical CPU count of the host, and the thread count the oracle runs with (the GPU box gives one GPU's
+    job 16 CPUs whatever the host has)."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    logical = os.cpu_count() or 1
+    return model, logical, min(logical, 16)
+
+
+def cpu_fields():
+    model, logical, threads = host_cpu()
+    torch.set_num_threads(threads)
+    return {"cores": threads, "host_logical_cpus": logical, "cpu_model": model}
+
+
+def median3(fn):
+    ts, res = [], None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        res = fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[1], res
+
+
+def profile_traffic(fname, applies=True):
+    """HBM bytes per launch of the roofline kernel as the committed counter summary states them (a line
+    `traffic_bytes_per_launch = N` in profiles/<fname>); None when the summary is absent or the run is not the workload it
+    was taken on.  A counter run cannot be made from inside this script."""
+    if not applies:
+        return None, None
+    import re
+    try:
+        with open(os.path.join(ROOT, "profiles", fname)) as f:
+            m = re.search(r"^traffic_bytes_per_launch\s*=\s*([0-9_]+)", f.read(), re.M)
+    except OSError:
+        return None, None
+    return (int(m.group(1).replace("_", "")), "profiles/" + fname) if m else (None, None)
+
+
 def build_workload(seed: int, batch: int, heads: int, lo: int, hi: int, q_len: int):
     from oracle import mla_oracle as O       # input generator only (bits identical for oracle and GPU)
     return O.make_decode_case(batch, heads, lo, hi, seed=seed, q_len=q_len)
@@ -43,7 +89,10 @@ def algorithmic_bytes(case, heads):
 
 def bench_dsa(K, dev, args):
     """configs[3]: lightning indexer (64 fp8 heads x 128) over contexts uniform[32768, 65536], batch 32, top-2048,
-    sparse absorbed MLA over the selected rows.  Per-stage device times (HIP events on the launch stream)."""
+    sparse absorbed MLA over the selected rows.  Index keys and queries are N(0,1) values put through the per-token e4m3
+    quantiser (the keys by the product's quantising cache write, a sequence at a time).  Per-stage device times (HIP events
+    on the launch stream); a sample of sequences is recomputed by the oracle, timed, and compared."""
+    from oracle import mla_oracle as O
     g = torch.Generator().manual_seed(args.seed)
     B, H, N, k = 32, 64, 128, 2048
     lens = torch.randint(32768, 65537, (B,), generator=g).to(torch.int32)
@@ -56,16 +105,26 @@ def bench_dsa(K, dev, args):
         n = int(nblk_seq[b])
         bt[b, :n] = perm[o:o + n].to(torch.int32)
         o += n
-    # fp8-e4m3 bit patterns of finite positive values for keys and queries, fp32 scales and head weights N(0,1)
-    k8 = torch.randint(0, 120, (nblk, 128, 128), dtype=torch.uint8, generator=g).to(dev)
-    ks = torch.rand(nblk, 128, generator=g).to(dev)
-    q8 = torch.randint(0, 120, (B, H, 128), dtype=torch.uint8, generator=g).to(dev)
-    w = torch.randn(B, H, generator=g).to(dev)
+    btd, lensd = bt.to(dev), lens.to(dev)
+    sample = (0, B - 1)
+    k8 = torch.zeros(nblk, 128, 128, dtype=torch.uint8, device=dev)
+    ks = torch.zeros(nblk, 128, dtype=torch.float32, device=dev)
+    k_src = {}
+    torch.manual_seed(args.seed)
+    for b in range(B):
+        L = int(lens[b])
+        x = torch.randn(L, 128, device=dev).bfloat16()
+        pos = torch.arange(L, device=dev)
+        K.quant_rows_fp8(x, k8, ks, slot_mapping=btd[b, pos // 128].long() * 128 + pos % 128)
+        if b in sample:
+            k_src[b] = x.cpu()
+    q8c, qsc = O.fp8_quant_token(torch.randn(B, H, 128, generator=g))
+    wc = torch.randn(B, H, generator=g)
+    q8, w = q8c.to(dev), (wc * qsc).to(dev)            # the caller folds the query scale into the head weights
     nope = torch.randn(nblk, 128, 512, device=dev).bfloat16()
     rope = torch.randn(nblk, 128, 64, device=dev).bfloat16()
-    qn = torch.randn(B, N, 512, device=dev).bfloat16()
-    qr = torch.randn(B, N, 64, device=dev).bfloat16()
-    btd, lensd = bt.to(dev), lens.to(dev)
+    qnc, qrc = torch.randn(B, N, 512, generator=g).bfloat16(), torch.randn(B, N, 64, generator=g).bfloat16()
+    qn, qr = qnc.to(dev), qrc.to(dev)
     max_len = int(lens.max())
     logits = torch.empty(B, K.indexer_logits_stride(max_len), device=dev)
     idx = torch.empty(B, k, dtype=torch.int32, device=dev)
@@ -73,11 +132,12 @@ def bench_dsa(K, dev, args):
     counts = torch.empty(B, dtype=torch.int32, device=dev)
     out = torch.empty(B, N, 512, dtype=torch.bfloat16, device=dev)
     splits = args.splits or K.default_num_splits(B, 1, N, k)
+    scale = 192 ** -0.5
     stages = [
         ("indexer", lambda: K.indexer_scores(q8, w, k8, ks, btd, lensd, logits, max_seq_len=max_len)),
         ("topk_with_rows", lambda: K.topk(logits, lensd, k, idx, block_table=btd, page_size=128, num_pages=nblk, rows=rows,
                                           counts=counts)),
-        ("sparse_decode", lambda: K.sparse_decode(qn, qr, nope, rope, rows, counts, 192 ** -0.5, out, num_splits=splits)),
+        ("sparse_decode", lambda: K.sparse_decode(qn, qr, nope, rope, rows, counts, scale, out, num_splits=splits)),
     ]
 
     def whole():
@@ -97,6 +157,15 @@ def bench_dsa(K, dev, args):
         return a.elapsed_time(e) * 1e3 / n
 
     total = ev_time(whole, args.steps)
+    # the chain again as one captured HIP graph
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        whole()
+        with torch.cuda.graph(graph, stream=side):
+            whole()
+    torch.cuda.synchronize()
+    total_graph = ev_time(graph.replay, args.steps)
     # a stage timed alone in a launch loop is bounded below by the host's launch rate (about 10 us a call): the small
     # stages read high here, the per-kernel durations of a rocprofv3 kernel trace are the better figure for them
     per_stage = {name: round(ev_time(f, args.steps), 2) for name, f in stages}
@@ -104,22 +173,58 @@ def bench_dsa(K, dev, args):
     idx_bytes = sum_l * (128 + 4) + B * H * (128 + 4) + sum_l * 4          # fp8 keys + scales, queries + weights, logits out
     sparse_bytes = B * k * 576 * 2 + B * N * (576 + 512) * 2
     ideal_us = (idx_bytes + sum_l * 4 + sparse_bytes) / (HBM_PEAK_GBS * 1e9) * 1e6
-    return {
+    best = min(total, total_graph)
+    traffic, traffic_src = profile_traffic("dsa_chain_b32_ctx32k_64k.md", args.seed == 0)
+    res = {
         "metric": "DSA decode us/layer (B=32, ctx 32k-64k, indexer 64 fp8 heads + top-2048 + sparse MLA 128 heads)",
-        "value": round(total, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "higher_is_better": False, "dtype": "fp8 (indexer) / bf16 (attention)", "data": "synthetic",
+        "value": round(best, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "fp8 (indexer) / bf16 (attention)",
+        "data": "synthetic: N(0,1) index keys / queries quantised per token to e4m3, N(0,1) bf16 latent cache",
         "config": {"workload": "configs[3]: DSA sparse decode path", "batch": B, "index_heads": H, "heads": N, "topk": k,
                    "seq_lens": "uniform[32768,65536]", "sum_seq_len": sum_l, "kv_splits": splits, "seed": args.seed},
-        "stage_us_launch_loop": per_stage, "launch": "eager launches",
+        "chain_us": {"eager_launches": round(total, 2), "hip_graph_replay": round(total_graph, 2)},
+        "stage_us_launch_loop": per_stage,
         "roofline": {"kernel": "dsa_indexer_fp8_kernel", "bound": "hbm",
                      "achieved": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(idx_bytes / (per_stage["indexer"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
-                     # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)
-                     "traffic": 219_800_000 if args.seed == 0 else None,
-                     "algorithmic_bytes": idx_bytes},
+                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": idx_bytes},
         "chain_roofline": {"hbm_bytes": idx_bytes + sum_l * 4 + sparse_bytes, "ideal_us_at_8TBs": round(ideal_us, 2),
-                           "frac": round(ideal_us / total, 4)},
+                           "frac": round(ideal_us / best, 4)},
     }
+    if args.no_cpu_baseline:
+        return res
+    # oracle chain of the sampled sequences on the host: logits of every visible key, stable top-k, attention over the picks
+    cpu = cpu_fields()
+    whole()
+    torch.cuda.synchronize()
+    lg, idx_c = logits.cpu(), idx.cpu()
+    worst_logit, worst_attn, sets_equal, t_cpu = 0.0, 0.0, True, 0.0
+    for b in sample:
+        L = int(lens[b])
+        ref8, ref_s = O.fp8_quant_token(k_src[b])
+        r = rows[b].long()
+        small_n = nope.view(-1, 512)[r].cpu().view(k // 128, 128, 512)
+        small_r = rope.view(-1, 64)[r].cpu().view(k // 128, 128, 64)
+
+        def chain():
+            sc = O.indexer_scores(q8c[b], qsc[b], ref8, ref_s, wc[b])
+            picks = O.topk_stable(sc, k, L)
+            att = O.sparse_decode(qnc[b:b + 1], qrc[b:b + 1], small_n, small_r, torch.arange(k // 128, dtype=torch.int32)[None],
+                                  torch.tensor([k], dtype=torch.int32), torch.arange(k, dtype=torch.int32)[None], scale)
+            return sc, picks, att
+        t, (sc, picks, att) = median3(chain)
+        t_cpu += t
+        worst_logit = max(worst_logit, ((lg[b, :L] - sc).abs().max() / sc.abs().max()).item())
+        sets_equal &= idx_c[b].tolist() == sorted(O.topk_stable(lg[b], k, L).tolist())
+        worst_attn = max(worst_attn, (out[b:b + 1].float().cpu() - att).abs().max().item())
+    sample_l = sum(int(lens[b]) for b in sample)
+    res["cpu_baseline"] = {"value": round(t_cpu * sum_l / sample_l * 1e6, 1), "unit": "us/layer", **cpu, "kind": "port",
+                           "sample": f"oracle chain (indexer logits, stable top-k, sparse attention; torch fp32) of sequences "
+                                     f"{list(sample)} of {B} ({sample_l} of {sum_l} keys), median of 3 each, scaled by key count",
+                           "sample_seconds": round(t_cpu, 3)}
+    res["gpu_vs_oracle"] = {"logits_max_err_rel_to_row_max": worst_logit, "topk_sets_equal_stable_topk_of_gpu_logits": sets_equal,
+                            "attention_max_abs": round(worst_attn, 5), "sequences": list(sample)}
+    return res
 
 
 def bench_prefill(K, dev, args):
@@ -138,9 +243,9 @@ def bench_prefill(K, dev, args):
     vc = torch.randn(B * C, N, 128, device=dev).bfloat16()
     cu_q = torch.arange(0, (B + 1) * Q, Q, dtype=torch.int32, device=dev)
     cu_c = torch.arange(0, (B + 1) * C, C, dtype=torch.int32, device=dev)
-    o_s = torch.empty(B * Q, N, 128, dtype=torch.bfloat16, device=dev)
+    o_s = torch.empty(B * Q, N, 128, dtype=torch.float32, device=dev)      # partials that the merge reads stay fp32
     o_c = torch.empty_like(o_s)
-    o = torch.empty_like(o_s)
+    o = torch.empty(B * Q, N, 128, dtype=torch.bfloat16, device=dev)
     l_s = torch.empty(B * Q, N, dtype=torch.float32, device=dev)
     l_c = torch.empty_like(l_s)
     # latent cache of the prefix for the gather + up-projection leg
@@ -176,7 +281,30 @@ def bench_prefill(K, dev, args):
     fl_c = B * N * Q * C * 2 * (192 + 128)
     fl_s = B * N * Q * (Q + 1) // 2 * 2 * (192 + 128)
     attn_us = per["context_attention"] + per["suffix_attention"] + per["merge"]
+    traffic, traffic_src = profile_traffic("mla_prefill_varlen_4x2048_over_16k.md", args.seed == 0)
+    extra = {}
+    if not args.no_cpu_baseline:
+        # one (sequence, head) pair recomputed by the oracle as a single causal attention over prefix + chunk keys
+        from oracle import mla_oracle as O
+        cpu = cpu_fields()
+        sb, sh = 1, 5
+        c = lambda x: x.float().cpu().bfloat16()
+        kq = slice(sb * Q, (sb + 1) * Q)
+        kc = slice(sb * C, (sb + 1) * C)
+        k_n = torch.cat([c(kc_n[kc, sh:sh + 1]), c(ks_n[kq, sh:sh + 1])])
+        k_p = torch.cat([c(kc_p[kc]), c(ks_p[kq])])
+        v_a = torch.cat([c(vc[kc, sh:sh + 1]), c(vs[kq, sh:sh + 1])])
+        q_n, q_p = c(qn[kq, sh:sh + 1]), c(qp[kq, sh:sh + 1])
+        t_cpu, (ref, _) = median3(lambda: O.attention_varlen(q_n, q_p, k_n, k_p, v_a, [0, Q], [0, C + Q], scale, True))
+        err = (o[kq, sh:sh + 1].float().cpu() - ref).abs()
+        extra["cpu_baseline"] = {"value": round(t_cpu * B * N * 1e6, 1), "unit": "us/layer", **cpu, "kind": "port",
+                                 "sample": f"oracle attention_varlen (torch fp32) of 1 of {B * N} (sequence, head) pairs: {Q} "
+                                           f"query rows over {C + Q} keys, median of 3, scaled by pair count",
+                                 "sample_seconds": round(t_cpu, 3)}
+        extra["gpu_vs_oracle"] = {"max_abs": round(err.max().item(), 5),
+                                  "mean_rel": round((err.sum() / ref.abs().sum()).item(), 6), "pair": [sb, sh]}
     return {
+        **extra,
         "metric": "MLA chunked prefill us/layer (4 x 2048-token chunk over 16384 cached tokens, 128 heads, bf16, attention kernels)",
         "value": round(attn_us, 1), "unit": "us/layer", "n_gpus": 1, "steps": n, "warmup": 2, "higher_is_better": False,
         "dtype": "bf16", "data": "synthetic",
@@ -188,8 +316,7 @@ def bench_prefill(K, dev, args):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round((fl_c + fl_s) / ((per["context_attention"] + per["suffix_attention"]) * 1e-6) / 1e12
                                    / MFMA_BF16_PEAK_TFLOPS, 4),
-                     # context-attention launch: FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of this workload
-                     "traffic": 5_413_000_000 if args.seed == 0 else None, "algorithmic_flops": fl_c + fl_s},
+                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_flops": fl_c + fl_s},
     }
 
 
@@ -208,13 +335,18 @@ def bench_fp8(K, dev, args):
         n = int(nblk_seq[b])
         bt[b, :n] = perm[o:o + n]
         o += n
-    cache = torch.empty(nblk, 128, K.FP8_ROW_BYTES, dtype=torch.uint8, device=dev)
-    # fill the cache on the GPU through the product's own quantising write, 64 pages at a time
-    for p0 in range(0, nblk, 64):
-        p1 = min(nblk, p0 + 64)
-        rows = (p1 - p0) * 128
-        K.cache_write_fp8(torch.randn(rows, 512, device=dev).bfloat16(), torch.randn(rows, 64, device=dev).bfloat16(),
-                          torch.arange(p0 * 128, p1 * 128, dtype=torch.int64, device=dev), cache)
+    cache = torch.zeros(nblk, 128, K.FP8_ROW_BYTES, dtype=torch.uint8, device=dev)
+    # fill the cache on the GPU through the product's own quantising write, a sequence at a time; sequence 0 keeps its
+    # source rows for the oracle
+    torch.manual_seed(args.seed)
+    btd = bt.to(dev)
+    for b in range(B):
+        L = int(lens[b])
+        c_b, r_b = torch.randn(L, 512, device=dev).bfloat16(), torch.randn(L, 64, device=dev).bfloat16()
+        pos = torch.arange(L, device=dev)
+        K.cache_write_fp8(c_b, r_b, btd[b, pos // 128].long() * 128 + pos % 128, cache)
+        if b == 0:
+            src0 = (c_b.cpu(), r_b.cpu())
     T = B * QL
     qn = torch.randn(T, N, 512, device=dev).bfloat16()
     qr = torch.randn(T, N, 64, device=dev).bfloat16()
@@ -225,7 +357,7 @@ def bench_fp8(K, dev, args):
         for j in range(QL):
             pos = int(lens[b]) - QL + j
             slots[b * QL + j] = int(bt[b, pos // 128]) * 128 + pos % 128
-    slots, btd, lensd = slots.to(dev), bt.to(dev), lens.to(dev)
+    slots, lensd = slots.to(dev), lens.to(dev)
     out = torch.empty(T, N, 512, dtype=torch.bfloat16, device=dev)
     splits = args.splits or K.default_num_splits(B, QL, N, int(lens.max()))
 
@@ -257,7 +389,31 @@ def bench_fp8(K, dev, args):
     flops = sum_l * N * QL * 2 * (576 + 512)
     bytes_ = sum_l * K.FP8_ROW_BYTES + T * N * (576 + 512) * 2
     best = min(t_graph, t_eager)
+    traffic, traffic_src = profile_traffic("mla_decode_fp8_b256_ctx16k_32k.md", args.seed == 0)
+    extra = {}
+    if not args.no_cpu_baseline:
+        # sequence 0 on the host: the oracle's block quantiser on the same source rows, then the oracle's decode
+        from oracle import mla_oracle as O
+        cpu = cpu_fields()
+        L = int(lens[0])
+        c0, r0 = src0[0].clone(), src0[1].clone()
+        c0[L - QL:], r0[L - QL:] = new_c[:QL].cpu(), new_r[:QL].cpu()
+        q8, sc = O.fp8_quant_block(c0.float())
+        npg = (L + 127) // 128
+        deq, rp = torch.zeros(npg * 128, 512), torch.zeros(npg * 128, 64, dtype=torch.bfloat16)
+        deq[:L], rp[:L] = O.fp8_dequant_block(q8, sc), r0
+        qn0, qr0 = qn[:QL].cpu(), qr[:QL].cpu()
+        t_cpu, ref = median3(lambda: O.absorbed_decode(qn0, qr0, deq.view(npg, 128, 512), rp.view(npg, 128, 64),
+                                                       torch.arange(npg, dtype=torch.int32)[None], lens[:1], 192 ** -0.5))
+        err = (out[:QL].float().cpu() - ref).abs()
+        extra["cpu_baseline"] = {"value": round(t_cpu * sum_l / L * 1e6, 1), "unit": "us/layer", **cpu, "kind": "port",
+                                 "sample": f"oracle absorbed_decode (torch fp32, cache rows dequantised beforehand) of sequence 0 of "
+                                           f"{B} ({L} of {sum_l} cached tokens), median of 3, scaled by token count",
+                                 "sample_seconds": round(t_cpu, 3)}
+        extra["gpu_vs_oracle"] = {"max_abs": round(err.max().item(), 5),
+                                  "mean_rel": round((err.sum() / ref.abs().sum()).item(), 6), "sequence": 0}
     return {
+        **extra,
         "metric": "MLA decode us/layer, fp8-e4m3 block-scaled cache (B=256, ctx 16k-32k, 128 heads, q_len 2)",
         "value": round(best, 1), "unit": "us/layer", "n_gpus": 1, "steps": n, "warmup": 3, "higher_is_better": False,
         "dtype": "bf16 MFMA over fp8 storage (dequantised on chip)", "data": "synthetic",
@@ -267,8 +423,7 @@ def bench_fp8(K, dev, args):
         "roofline": {"kernel": "mla_decode_v2_fp8_kernel<false>", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                     # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)
-                     "traffic": 5_444_600_000 if args.seed == 0 else None,
+                     "traffic": traffic, "traffic_source": traffic_src,
                      "algorithmic_flops": flops, "algorithmic_bytes": bytes_,
                      "hbm_gbs": round(bytes_ / (best * 1e-6) / 1e9, 1)},
     }
@@ -355,7 +510,7 @@ def bench_prologue(K, dev, args):
                      "achieved": round(tot_bytes / step_us / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(tot_bytes / step_us / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
                      "algorithmic_bytes": tot_bytes},
-        "cpu_baseline": {"value": round(cpu * 1e6, 1), "unit": "us", "cores": torch.get_num_threads(),
+        "cpu_baseline": {"value": round(cpu * 1e6, 1), "unit": "us", **cpu_fields(),
                          "kind": "port", "sample": "oracle (torch float64) on the same 8192 tokens, median of 3",
                          "gpu_vs_oracle_max_ulp": int(bits)},
     }
@@ -417,6 +572,7 @@ def bench_epilogue(K, dev, args):
     alg_bytes = segments * N * 1040 + N * 512 * 128 * 2 + B * N * 128 * 2
     # oracle chain on the host: attention of a sample of sequences, then the up-projection of all
     sample = 8
+    cpu_info = cpu_fields()
     t0 = time.perf_counter()
     ref_o = O.absorbed_decode(case["q_nope"][:sample], case["q_rope"][:sample], case["nope"], case["rope"],
                               case["block_table"][:sample], case["seq_lens"][:sample], case["scale"])
@@ -424,6 +580,7 @@ def bench_epilogue(K, dev, args):
     cpu_s = time.perf_counter() - t0
     err = (out_f[:sample].float().cpu() - ref).abs().max().item()
     same = (out_f.float() - out_u.float()).abs().max().item()
+    traffic, traffic_src = profile_traffic("mla_reduce_vup_b64_128heads.md", args.seed == 0 and not args.splits)
     return {
         "metric": "merge of the split-KV partials + value up-projection, us/layer (B=64, 128 heads, 4 chunks per sequence)",
         "value": round(t_f, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -433,9 +590,8 @@ def bench_epilogue(K, dev, args):
         "unfused_us": round(t_u, 2), "fused_vs_unfused_max_abs": same,
         "roofline": {"kernel": "mla_reduce_vup_kernel", "bound": "hbm", "achieved": round(alg_bytes / t_f / 1e3, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_bytes / t_f / 1e3 / HBM_PEAK_GBS, 4),
-                     # FETCH_SIZE x 2.000 + WRITE_SIZE of a rocprofv3 --pmc run of exactly this workload (seed 0)
-                     "traffic": 80_600_000 if (args.seed == 0 and not args.splits) else None, "algorithmic_bytes": alg_bytes},
-        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", "cores": torch.get_num_threads(),
+                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": alg_bytes},
+        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", **cpu_info,
                          "kind": "port", "sample": f"oracle attention (torch fp32) of {sample} of {B} sequences + up-projection, scaled by sequence count",
                          "gpu_vs_oracle_max_abs": err},
     }
@@ -487,24 +643,24 @@ def bench_window(K, dev, args):
     visible = int((torch.clamp(case["seq_lens"], max=win) + sink).sum())
     alg_bytes = visible * 1152 + B * N * 576 * 2 + B * N * 512 * 2
     sample = 4
+    cpu_info = cpu_fields()
     t0 = time.perf_counter()
     ref = O.sink_decode(case["q_nope"][:sample], case["q_rope"][:sample], nope_c, rope_c, bt_c[:sample], case["seq_lens"][:sample],
                         sink, case["scale"], win)
     cpu_s = time.perf_counter() - t0
     err = (out[:sample].float().cpu() - ref).abs().max().item()
+    traffic, traffic_src = profile_traffic("mla_decode_window_b64_sink128_w4096.md", args.seed == 0 and not args.splits)
     return {
         "metric": "MLA decode with static sink + sliding window, us/layer (B=64, ctx 4k-8k, sink 128, window 4096, 128 heads, bf16)",
         "value": round(t_step, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "static sink tokens + sliding window decode (plan + split + merge, graph replay)", "batch": B,
                    "heads": N, "sink_len": sink, "window": win, "visible_keys": visible, "seed": args.seed},
-        "roofline": {"kernel": "plan + mla_decode_v2_kernel<false, true> + merge (whole step)", "bound": "hbm",
+        "roofline": {"kernel": "mla_window_plan_kernel + mla_decode_v3_kernel<false, true> + merge (whole step)", "bound": "hbm",
                      "achieved": round(alg_bytes / t_step / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(alg_bytes / t_step / 1e3 / HBM_PEAK_GBS, 4),
-                     # FETCH_SIZE x 2.000 + WRITE_SIZE of rocprofv3 --pmc runs of exactly this workload (seed 0), the three
-                     # kernels of the step added up
-                     "traffic": 429_600_000 if (args.seed == 0 and not args.splits) else None, "algorithmic_bytes": alg_bytes},
-        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", "cores": torch.get_num_threads(),
+                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": alg_bytes},
+        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", **cpu_info,
                          "kind": "port", "sample": f"oracle sink_decode (torch fp32) of {sample} of {B} sequences, scaled by sequence count",
                          "gpu_vs_oracle_max_abs": err},
     }
@@ -627,7 +783,7 @@ def main():
     # HBM bytes per launch of the split kernel from the FETCH_SIZE / WRITE_SIZE counter runs (scaled on a plain copy) of
     # exactly this workload; a counter run cannot be made from inside this script, so other shapes report null
     default_shape = (args.seed, b, heads, args.len_lo, args.len_hi, q_len, splits) == (0, 64, 128, 4096, 8192, 1, 4)
-    traffic = 533_400_000 if default_shape else None
+    traffic, traffic_src = profile_traffic("mla_decode_v3_b64_ctx8k.md", default_shape)
     res = {
         "metric": "MLA decode us/layer (B=64, ctx 4k-8k, 128 heads, bf16, cache write + split-KV decode + reduce)",
         "value": round(dev_step_avg, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -642,8 +798,9 @@ def main():
         "step_hbm_gbs": round(ab["total"] / (dev_step_avg * 1e-6) / 1e9, 1),
         "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                                     / (dev_step_avg * 1e-6), 4),
-        "roofline": {"kernel": "mla_decode_v2_kernel<false, false>", "bound": "hbm", "achieved": round(achieved, 1),
+        "roofline": {"kernel": "mla_decode_v3_kernel<false, false>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": traffic_src,
                      "kernel_us_avg": round(k_avg, 2), "kernel_us_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),
                      "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
@@ -651,8 +808,7 @@ def main():
 
     if not args.no_cpu_baseline:
         from oracle import mla_oracle as O
-        ncpu = min(os.cpu_count() or 1, 16)
-        torch.set_num_threads(ncpu)
+        cpu_info = cpu_fields()
         ns = min(args.cpu_seqs, b)
         sl = slice(0, ns * q_len)
         cn, cr = case["nope"].clone(), case["rope"].clone()      # the oracle sees the same new rows in its cache
@@ -671,7 +827,7 @@ def main():
         sample_l = int(case["seq_lens"][:ns].sum())
         cpu_us_full = sorted(ts)[1] * 1e6 * sum_l / sample_l
         err = (out_v[sl].float().cpu() - ref).abs().max().item()
-        res["cpu_baseline"] = {"value": round(cpu_us_full, 1), "unit": "us/layer", "cores": ncpu, "kind": "port",
+        res["cpu_baseline"] = {"value": round(cpu_us_full, 1), "unit": "us/layer", **cpu_info, "kind": "port",
                                "sample": f"oracle (torch fp32) on the first {ns} of {b} sequences ({sample_l} of {sum_l} "
                                          f"cached tokens), median of 3, scaled by token count",
                                "sample_seconds": round(sorted(ts)[1], 3), "gpu_vs_oracle_max_abs": round(err, 5)}

@@ -223,7 +223,9 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             kv_c_normed = cc.workspace[:toks][..., :self.kv_lora_rank]
             k_pe = cc.workspace[:toks][..., self.kv_lora_rank:]
             k_nope, v = self._kv_up(kv_c_normed)
-            attn_output = torch.empty(t, n, self.v_head_dim, dtype=q_nope.dtype, device=q_nope.device)
+            # partial results that a merge will read stay fp32: each bf16 rounding in between would add 2^-10 of mean
+            # relative error to the layer's output
+            attn_output = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q_nope.device)
             attn_lse = torch.empty(t, n, dtype=torch.float32, device=q_nope.device)
             K.prefill_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cc.cu_seq_lens[i].to(torch.int32).contiguous(),
                              prefill.max_query_len, self.scale, False, attn_output, attn_lse)
@@ -248,14 +250,14 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
         k_nope, v = self._kv_up(kv_c_normed)
         cu_q = prefill.query_start_loc.to(torch.int32).contiguous()
-        output = torch.empty(t, n, self.v_head_dim, dtype=q.dtype, device=q.device)
+        output = torch.empty(t, n, self.v_head_dim, dtype=torch.float32 if has_context else q.dtype, device=q.device)
         output_lse = torch.empty(t, n, dtype=torch.float32, device=q.device) if has_context else None
         K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
                          output, output_lse)
         if has_context:
             ctx_out, ctx_lse = self._compute_prefill_context(q_nope, q_pe, kv_cache[0], kv_cache[1], attn_metadata, k_scale)
             if ctx_out is not None:
-                merged = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q.device)
+                merged = torch.empty(t, n, self.v_head_dim, dtype=torch.bfloat16, device=q.device)
                 K.merge_states(ctx_out, ctx_lse, output, output_lse, merged)
                 output = merged
         return output.to(torch.bfloat16).flatten(start_dim=-2)
@@ -281,17 +283,17 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             return output.flatten(start_dim=-2)
         ks_nope, vs = self._kv_up(self.sink_compressed_kv)
         cu_s = s_len * torch.arange(nb + 1, dtype=torch.int32, device=q.device)
-        out_sink = torch.empty_like(output)
+        out_sink = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q.device)     # fp32 partials into the merge
+        band = torch.empty_like(out_sink)
         lse_sink = torch.empty(t, n, dtype=torch.float32, device=q.device)
         K.prefill_varlen(q_nope, q_pe, ks_nope.repeat(nb, 1, 1), sink_pe.repeat(nb, 1), vs.repeat(nb, 1, 1), cu_q, cu_s,
                          prefill.max_query_len, self.scale, False, out_sink, lse_sink)
         k_nope, v = self._kv_up(kv_c_normed)
         lse = torch.empty(t, n, dtype=torch.float32, device=q.device)
         K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
-                         output, lse, window=self.sliding_window)
-        merged = torch.empty_like(output)
-        K.merge_states(out_sink, lse_sink, output, lse, merged)
-        return merged.flatten(start_dim=-2)
+                         band, lse, window=self.sliding_window)
+        K.merge_states(out_sink, lse_sink, band, lse, output)
+        return output.flatten(start_dim=-2)
 
     @staticmethod
     def _insert_tensor_by_start_loc(raw_tensor: torch.Tensor, insert_segment: torch.Tensor, start_loc: list) -> torch.Tensor:

@@ -54,7 +54,10 @@ def test_prefill_varlen_matches_oracle(dev, causal, q_lens, k_lens, n):
     K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
                      torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
                      max(q_lens), scale, causal, out_bf)
-    attn_close(out_bf, ref, 2e-2, 3e-3)
+    # bf16 output: its rounding alone is 2^-10 = 1e-3 of mean relative error, and with a few dozen keys per row the bf16
+    # rounding of the probabilities (2^-9 each) does not average out; such rows measure 2.0e-3 to 2.1e-3, so rows shorter
+    # than one 64-key block get 2.5e-3, all others the 2e-3 bar
+    attn_close(out_bf, ref, 2e-2, 2e-3 if min(k for k in k_lens if k) >= 64 else 2.5e-3)
 
 
 def test_chunked_context_flow_gather_attend_merge(dev):
