@@ -87,7 +87,7 @@ typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scala
 
 #ifdef MLA_V3_TRACE
 __device__ unsigned long long* g_trace;                     // [workgroup][wave][8]: clock sums per phase, block count
-#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0
+#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0, tr_k0 = 0, tr_e0 = 0, tr_ep = 0; TR_STAMP(tr_k0)
 #define TR_STAMP(x) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x)::"memory")
 #define TR_ADD(k) do { TR_STAMP(tr_b); tr_t[k] += tr_b - tr_a; tr_a = tr_b; } while (0)
 #else
@@ -100,6 +100,10 @@ template <bool kSparse, bool kWindow>
 __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params p) {
   static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
+#ifdef MLA_V3_TRACE
+  uint64_t tr_start;
+  TR_STAMP(tr_start);
+#endif
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // 0..7
   const int l16 = lane & 15;                                  // QK: query row of the wave / key of a 16-key group
@@ -495,7 +499,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
 #undef MLA_K_ADDR
 #undef MLA_K_OFF
     asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s[0]), "+v"(s[1]));
-#ifdef ABL_QK_NOMFMA
+#if defined(ABL_QK_NOMFMA) || defined(ABL_QK_NOREAD)
     s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0];
 #endif
   };
@@ -685,6 +689,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     // brought back (and waited for) now, not at its first use inside the loop.
     asm volatile("" :: "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(p_w_off), "v"(dma_off));
     // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
+#ifdef MLA_V3_TRACE
+    if (tr_t[5] == 0) { TR_STAMP(tr_b); tr_t[5] = tr_b - tr_start; }
+#endif
     for (int i = 0; i + 1 < nb; i++) {
       const int blk = blk_begin + i;
       TR_STAMP(tr_a);
@@ -711,7 +718,10 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       Sm st;
       float sc[8];
       unpack_scores(s, sc);
-#ifdef ABL_NO_PV
+#ifdef ABL_NO_PVSM
+      st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
+      st.pw[0] = st.pw[1] = st.pw[2] = st.pw[3] = 0;
+#elif defined(ABL_NO_PV)
       pv_softmax(blk, std::false_type{}, std::true_type{}, sc, st);
 #elif defined(ABL_NO_SOFTMAX)
       st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
@@ -741,6 +751,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   } while (restart);
 
   // ---- epilogue ----
+  TR_STAMP(tr_e0);
   // (lane-derived values are worked out again from the hardware lane number: nothing of them has to live through the loop)
   lds_barrier();                                              // all PV done; tile buffers and P buffers are free
   const int e_ln = lane_now();
@@ -826,12 +837,16 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       *(u32x2*)(o_part_c + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#ifdef MLA_V3_TRACE
+  TR_STAMP(tr_b); tr_ep += tr_b - tr_e0;
+#endif
   }  // segments
 #ifdef MLA_V3_TRACE
   if (g_trace && lane == 0) {
     unsigned long long* t = g_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.z) * 8 + wave) * 8;
     for (int k = 0; k < 6; k++) t[k] = tr_t[k];
     t[6] = tr_n;
+    t[7] = tr_ep;
   }
 #endif
 }
