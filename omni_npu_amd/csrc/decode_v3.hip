@@ -44,11 +44,12 @@ constexpr int kFlagOff = kPOff + 2 * kPBufB;               // 159744: restart fl
 constexpr int kLimitOff = kFlagOff + 64;                   // per row of the group: number of visible keys (read by masking blocks only)
 constexpr int kSeenOff = kLimitOff + 512;                  // per lane: the score that raised its restart flag
 constexpr int kKTabOff = kSeenOff + 2048;                  // per lane: LDS offsets of its K-fragment reads (latent, rope)
-constexpr int kIdsOff = kKTabOff + 512;                    // row lists: 4 blocks x 8 waves x the wave's four cache rows
+constexpr int kIdsOff = kKTabOff + 512;                    // row lists: 4 blocks x 4 copying waves x the wave's eight cache rows
 constexpr int kLdsB = kIdsOff + 512;
 static_assert(kLdsB <= 160 * 1024, "LDS budget");
 constexpr int kLead = 3;                                   // block i + kLead is copied while block i is consumed
-constexpr int kCopies = 5;                                 // copy instructions per wavefront and block (4 nope rows + rope)
+constexpr int kCopyWaves = 4;                              // wavefronts 0..3 issue the copies (the older wavefront of each SIMD)
+constexpr int kCopies = 9;                                 // copy instructions per copying wavefront and block (8 nope rows + rope)
 #ifndef MLA_V3_AHEAD
 #define MLA_V3_AHEAD 4
 #endif
@@ -83,17 +84,30 @@ __device__ __forceinline__ int wave_incl_scan_i32(int v, int lane) {
   for (int d = 1; d < 64; d <<= 1) { const int t = __shfl_up(v, d, 64); v += lane >= d ? t : 0; }
   return v;
 }
+// inclusive scan over the 64 lanes with data-parallel-primitive moves (no LDS round trips): shifts inside the rows of 16,
+// then lane 15 of rows 0 and 2 into rows 1 and 3, then lane 31 into the upper half
+__device__ __forceinline__ int wave_incl_scan_dpp(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);
+  return v;
+}
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
 #ifdef MLA_V3_TRACE
 __device__ unsigned long long* g_trace;                     // [workgroup][wave][8]: clock sums per phase, block count
-#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0, tr_k0 = 0, tr_e0 = 0, tr_ep = 0; TR_STAMP(tr_k0)
+#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0, tr_k0 = 0, tr_e0 = 0, tr_ep = 0, tr_p[4] = {0, 0, 0, 0}; TR_STAMP(tr_k0)
+#define TR_PRO(k) do { if (tr_p[k] == 0) { TR_STAMP(tr_b); tr_p[k] = tr_b - tr_start; } } while (0)
 #define TR_STAMP(x) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x)::"memory")
 #define TR_ADD(k) do { TR_STAMP(tr_b); tr_t[k] += tr_b - tr_a; tr_a = tr_b; } while (0)
 #else
 #define TR_DECL
 #define TR_STAMP(x)
 #define TR_ADD(k)
+#define TR_PRO(k)
 #endif
 
 template <bool kSparse, bool kWindow>
@@ -138,36 +152,88 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   // Every non-empty sequence is kSegCost units of start-up followed by its 32-key blocks, the sequences end to end, and
   // that line is cut into gridDim.x chunks of equal length; a chunk that crosses a sequence boundary runs several
   // segments; the segment of sequence b in chunk c writes partial number c + b.
+  // With up to 64 sequences a lane holds one sequence's length and query range: everything the plan and the first
+  // segment need comes from one round of loads issued together at the start of the kernel (each dependent round trip
+  // to memory costs more than a microsecond there, with cold caches).
+#ifdef MLA_V3_TRACE
+  uint64_t tr_x0 = 0, tr_x1 = 0;
+#endif
   int seg_b;
   int64_t v_cur, v_end, v_seq;
+  int first_L = -1, first_q0 = 0, first_q1 = 0;               // the first segment's sequence, if known from the plan's loads
   {
     int tot = 0;
-    for (int i = lane; i < p.batch; i += 64) tot += work_units(p.seq_lens[i]);
-    tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
-    const int64_t cb = (int64_t)chunk * tot / gridDim.x, ce = (int64_t)(chunk + 1) * tot / gridDim.x;
+    const bool one_pass = p.batch <= 64;
+    int my_len = 0, my_q0 = 0, my_q1 = 0;
+    if (one_pass) {
+      if (lane < p.batch) {
+        my_len = p.seq_lens[lane];
+        if (p.qsl) { my_q0 = p.qsl[lane]; my_q1 = p.qsl[lane + 1]; }
+      }
+      tot = work_units(my_len);
+    } else {
+      for (int i = lane; i < p.batch; i += 64) tot += work_units(p.seq_lens[i]);
+    }
+    int pe1 = 0;
+    if (one_pass) { pe1 = wave_incl_scan_dpp(tot); tot = __builtin_amdgcn_readlane(pe1, 63); }
+    else tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
+#ifdef MLA_V3_TRACE
+    TR_STAMP(tr_x0);
+#endif
+    // chunk c covers units [floor(c * tot / G), floor((c + 1) * tot / G)); with G <= 65536 that is 32-bit arithmetic:
+    // c * tot / G = c * (tot / G) + c * (tot % G) / G exactly (a 64-bit division is a long software routine)
+    int64_t cb, ce;
+    if (gridDim.x <= 65536u) {
+      const uint32_t G = gridDim.x, q = (uint32_t)tot / G, r = (uint32_t)tot - q * G;
+      cb = (int64_t)chunk * q + (uint32_t)chunk * r / G;
+      ce = (int64_t)(chunk + 1) * q + ((uint32_t)chunk + 1u) * r / G;
+    } else {
+      cb = (int64_t)chunk * tot / gridDim.x;
+      ce = (int64_t)(chunk + 1) * tot / gridDim.x;
+    }
     if (cb == ce) return;
     int carry = 0, b0 = 0, pb0 = 0;
-    for (int base = 0; base < p.batch; base += 64) {
-      const int i = base + lane;
-      const int c = i < p.batch ? work_units(p.seq_lens[i]) : 0;
-      const int pe = wave_incl_scan_i32(c, lane) + carry;
-      const bool le = i < p.batch && pe <= cb;
-      b0 += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
-      pb0 = max(pb0, wave_max_i32(le ? pe : 0));
-      carry = __builtin_amdgcn_readlane(pe, 63);
+    if (one_pass) {
+      // the running totals do not decrease from lane to lane: the sequences that end at or before the chunk's first unit
+      // are the first b0 lanes, and the last of them holds the largest such total
+      const bool le = lane < p.batch && pe1 <= cb;
+      b0 = __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+      pb0 = b0 > 0 ? __builtin_amdgcn_readlane(pe1, b0 - 1) : 0;
+    } else {
+      for (int base = 0; base < p.batch; base += 64) {
+        const int i = base + lane;
+        const int c = i < p.batch ? work_units(p.seq_lens[i]) : 0;
+        const int pe = wave_incl_scan_i32(c, lane) + carry;
+        const bool le = i < p.batch && pe <= cb;
+        b0 += __builtin_popcountll(__builtin_amdgcn_ballot_w64(le));
+        pb0 = max(pb0, wave_max_i32(le ? pe : 0));
+        carry = __builtin_amdgcn_readlane(pe, 63);
+      }
     }
     seg_b = __builtin_amdgcn_readfirstlane(b0) - 1;
     v_seq = __builtin_amdgcn_readfirstlane(pb0);
     v_cur = cb;
     v_end = ce;
+    if (one_pass && seg_b + 1 < p.batch) {
+      first_L = __builtin_amdgcn_readlane(my_len, seg_b + 1);
+      first_q0 = __builtin_amdgcn_readlane(my_q0, seg_b + 1);
+      first_q1 = __builtin_amdgcn_readlane(my_q1, seg_b + 1);
+    }
   }
 
   TR_DECL;
+#ifdef MLA_V3_TRACE
+  TR_STAMP(tr_x1);
+  tr_p[3] = tr_x1 - tr_start;
+#endif
   while (v_cur < v_end) {
   seg_b++;
   if (seg_b >= p.batch) break;
   const int b = seg_b;
-  const int L = p.seq_lens[b];
+  const bool seg_known = first_L >= 0;                        // (only in the first pass of this loop)
+  const int L = seg_known ? first_L : p.seq_lens[b];
+  const int known_q0 = first_q0, known_q1 = first_q1;
+  first_L = -1;
   const int64_t v_b = v_seq;
   v_seq += work_units(L);
   const int64_t v_hi = v_seq < v_end ? v_seq : v_end;
@@ -190,7 +256,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     KernArgPtr kp = cold();
     const int32_t* qsl = kp->qsl;
     const int mq = kp->max_q_len;
-    if (qsl) { q0 = qsl[b]; qlen = qsl[b + 1] - q0; } else { q0 = b * mq; qlen = mq; }
+    if (qsl && seg_known) { q0 = known_q0; qlen = known_q1 - q0; }
+    else if (qsl) { q0 = qsl[b]; qlen = qsl[b + 1] - q0; }
+    else { q0 = b * mq; qlen = mq; }
     qlen = qlen < mq ? qlen : mq;
   }
   const int rows = qlen * p.num_heads;
@@ -223,20 +291,25 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     continue;
   }
 
-  // ---- global -> LDS copies: per wave and block four nope rows (1 KiB each) and four rope rows (lanes 0..31) ----
+  // ---- global -> LDS copies: wavefronts 0..3 copy eight nope rows (1 KiB each) and eight rope rows per block ----
+  // A copy instruction stalls at issue while the memory pipeline is full, and a stalled wavefront issues nothing else.
+  // The two wavefronts of a SIMD (w and w + 4) would stall at the same moments if both copied; with all copies in the
+  // older one the younger one keeps the matrix pipe busy meanwhile, and the older one is the one that otherwise waits
+  // at the barrier.
   // Row r of a block goes to nope buffer row r (granule gr at position gr ^ swz(r)) and rope buffer row r.  Wave w copies
-  // rows 4w..4w+3: swz(4w + j) = swz(4w) ^ swz(j), so one per-lane offset serves all four rows.
+  // rows 8w..8w+7: swz(8w + j) = swz(8w) ^ swz(j), so one per-lane offset serves all eight rows.
   // The per-lane offsets are worked out from the hardware lane number at every use (a handful of vector ALU
   // instructions per block, in the phase where that unit idles) instead of occupying registers through the loop.
   const uint32_t n_sr2 = (uint32_t)p.nope_sr * 2u, r_sr2 = (uint32_t)p.rope_sr * 2u;       // row strides in bytes
-  const int swz_nw = swz_nope((wave * 4) & 15), swz_rw = swz_rope((wave * 4) & 15);        // scalars
+  const bool copier = wave < kCopyWaves;
+  const int swz_nw = swz_nope((wave * 8) & 15), swz_rw = swz_rope((wave * 8) & 15);        // scalars
   // full blocks of the paged cache: the wave's row offsets ride in the per-lane offset (32 rows stay below 2^31 bytes,
   // checked where the mode is chosen), so a copy is one vector instruction, one scalar add into M0 and the load
   const bool full_ok = n_sr2 <= (1u << 25) && r_sr2 <= (1u << 25);
   const uint32_t dma_off = (uint32_t)((lane ^ swz_nw) << 4);
-  uint32_t s_rowoff[4];
+  uint32_t s_rowoff[8];
 #pragma unroll
-  for (int k = 0; k < 4; k++) s_rowoff[k] = (uint32_t)(wave * 4 + k) * n_sr2;
+  for (int k = 0; k < 8; k++) s_rowoff[k] = (uint32_t)(wave * 8 + k) * n_sr2;
 
   ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (kSparse ? 0 : (int64_t)b * p.bt_stride);
   const int64_t max_row = p.num_pages * p.page_size - 1;
@@ -248,29 +321,33 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     asm volatile("" : "+v"(ln));
     return ln;
   };
-  // Row list (kSparse): a wave copies rows 4w..4w+3 of a block and needs the cache rows of exactly those four keys.  They
-  // are fetched one block ahead by a four-lane global -> LDS copy into the wave's own slot (no register is the target of
+  // Row list (kSparse): a wave copies rows 8w..8w+7 of a block and needs the cache rows of exactly those eight keys.  They
+  // are fetched one block ahead by an eight-lane global -> LDS copy into the wave's own slot (no register is the target of
   // a load in flight, so nothing the compiler does with registers in between can lose them), issued in front of the
   // copies of the previous block so that the wait that lets those land covers it, and read back when the copies are due.
   // Keys past the end of the list name its last key (their scores are masked).
-  int32_t ids_rope = 0;                                       // cache row of this lane's rope row (lanes 0..31)
-  int32_t ids_row[4] = {0, 0, 0, 0};                          // cache rows of the wave's four keys (uniform)
+  int32_t ids_rope = 0;                                       // cache row of this lane's rope row
+  int32_t ids_row[8] = {0, 0, 0, 0, 0, 0, 0, 0};              // cache rows of the wave's eight keys (uniform)
   auto ids_dma = [&](int blk_x) {
     if constexpr (kSparse) {
-      int tok = blk_x * kBlk + wave * 4 + (lane_now() & 3);
-      tok = tok < L ? tok : L - 1;
-      tok = tok < 0 ? 0 : tok;
-      dma4_sv_lanes4(p.sparse_rows + (int64_t)b * p.sparse_stride, (uint32_t)tok * 4u, lds0 + kIdsOff + (blk_x & 3) * 128 + wave * 16);
+      if (copier) {
+        int tok = blk_x * kBlk + wave * 8 + (lane_now() & 7);
+        tok = tok < L ? tok : L - 1;
+        tok = tok < 0 ? 0 : tok;
+        dma4_sv_lanes8(p.sparse_rows + (int64_t)b * p.sparse_stride, (uint32_t)tok * 4u, lds0 + kIdsOff + (blk_x & 3) * 128 + wave * 32);
+      }
     }
   };
   auto ids_fetch = [&](int blk_x) {
     if constexpr (kSparse) {
-      const int ln = lane_now();
-      const char* slot = lds + kIdsOff + (blk_x & 3) * 128 + wave * 16;
-      const int32_t mine = *(const int32_t*)(slot + (ln & 3) * 4);
-      ids_rope = *(const int32_t*)(slot + ((ln >> 3) & 3) * 4);
+      if (copier) {
+        const int ln = lane_now();
+        const char* slot = lds + kIdsOff + (blk_x & 3) * 128 + wave * 32;
+        const int32_t mine = *(const int32_t*)(slot + (ln & 7) * 4);
+        ids_rope = *(const int32_t*)(slot + ((ln >> 3) & 7) * 4);
 #pragma unroll
-      for (int k = 0; k < 4; k++) ids_row[k] = __builtin_amdgcn_readlane(mine, k);
+        for (int k = 0; k < 8; k++) ids_row[k] = __builtin_amdgcn_readlane(mine, k);
+      }
     }
   };
   auto load_page = [&](int page) -> int64_t {
@@ -297,7 +374,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       pg_nxt = load_page(page_cur + 1);
     }
   };
-  // The five copies of a block are issued one at a time ("pieces") so that they can be spread over the MFMAs of the QK
+  // The nine copies of a block are issued one at a time ("pieces") so that they can be spread over the MFMAs of the QK
   // phase.  Rows past the end of the sequence re-read its last row (their scores are masked).
   // rope buffer of a block: (blk - blk_begin + rope_ph) % 3 without a division (rope_ph = blk_begin % 3 once per segment)
   const int rope_ph = blk_begin % 3;
@@ -335,22 +412,22 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     }
     return c;
   };
-  auto rope_lane_row = [&] { return (lane_now() >> 3) & 3; };                               // lane's row among the wave's four
+  auto rope_lane_row = [&] { return (lane_now() >> 3) & 7; };                               // lane's row among the wave's eight
   auto rope_lane_off = [&]() -> uint32_t {
-    const int ln = lane_now(), t = (ln >> 3) & 3;
-    return (uint32_t)(((ln & 7) ^ swz_rw ^ ((t & 1) << 2) ^ (t & 2)) << 4);                 // swz_rope(t) = (t0 << 2) | (t1 << 1)
+    const int ln = lane_now(), t = (ln >> 3) & 7;
+    return (uint32_t)(((ln & 7) ^ swz_rw ^ ((t & 1) << 2) ^ (t & 2) ^ (t >> 2)) << 4);      // swz_rope(t) = (t0 << 2) | (t1 << 1) | t2
   };
   // kFull: every row of the block exists and the source is the paged cache
   auto issue_piece = [&](IssueCtx& c, int k, auto full) {
     constexpr bool kFull = decltype(full)::value && !kSparse;
     auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
 
-    if (k < 4) {
-      const int r = wave * 4 + k;
+    if (k < 8) {
+      const int r = wave * 8 + k;
       if constexpr (kFull) {
         uint32_t d = dma_off;
-        asm volatile("" : "+v"(d));                           // (opaque: the four offsets are not precomputed and spilled)
-        dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + wave * 4096, k * 1024);
+        asm volatile("" : "+v"(d));                           // (opaque: the eight offsets are not precomputed and spilled)
+        dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + wave * 8192, k * 1024);
       } else {
         const uint32_t off = (uint32_t)((lane_now() ^ swz_nw ^ swz_nope(k)) << 4);
         const int re = r < c.last ? r : c.last;
@@ -358,22 +435,24 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
         else dma16_sv(c.np + (uint64_t)re * n_sr2, off, c.nbuf + r * 1024);
       }
     } else {
-      // the wave's four rope rows, 128 bytes each: half an instruction (lanes 32..63 sit out)
+      // the wave's eight rope rows, 128 bytes each: one instruction
       if constexpr (kSparse) {
-        dma16_v_lo32(c.rp + clampi(ids_rope) * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+        dma16_v(c.rp + clampi(ids_rope) * r_sr2 + rope_lane_off(), c.rbuf + wave * 1024);
       } else if constexpr (kFull) {
-        dma16_sv_lo32(c.rp, (uint32_t)(wave * 4 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+        dma16_sv(c.rp, (uint32_t)(wave * 8 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + wave * 1024);
       } else {
-        const int r = wave * 4 + rope_lane_row();
+        const int r = wave * 8 + rope_lane_row();
         const int re = r < c.last ? r : c.last;
-        dma16_sv_lo32(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + wave * 512);
+        dma16_sv(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + wave * 1024);
       }
     }
   };
   auto issue_block = [&](int blk) {
     IssueCtx c = issue_begin(blk);
+    if (copier) {
 #pragma unroll
-    for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{});
+      for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{});
+    }
   };
   // Row list: the rows of the first kLead blocks are fetched together (one round trip) before any copy goes out
   auto issue_first = [&]() {
@@ -394,28 +473,63 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     }
   };
 
-  // ---- prologue: the first block's copies go out, then the query loads; both are waited for together ----
-  issue_first();
+  // ---- prologue: the query, then the first blocks' copies ----
+  // The MFMA operand layout wants, per load instruction, 16 bytes of 64 different cache lines: read straight from
+  // memory the texture addresser needs 64 cycles per instruction and the query takes ten microseconds.  So every wave
+  // copies its own 16 rows global -> LDS whole (one row per instruction, into the tile buffers, which are free at the
+  // start of a segment) and picks its operands from there.  The copies of the first key blocks have to wait until
+  // every wave has its query in registers (one barrier).
+  TR_PRO(0);
   bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
   {
-    const int64_t tq = row_ok ? (q0 + t_local) : q0;         // rows that do not exist read row 0 of the sequence
-    const int64_t hq = row_ok ? head : 0;
     // Contraction step kk of the latent part covers the 16-byte granules 16*(kk%4) + 4g' + kk/4, g' = 0..3, and lane group
     // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
     // in one aligned 32-byte piece of a row, or the LDS serves the instruction at half rate (measured: 126 against 227
     // bytes per clock and CU with eight wavefronts reading).
     KernArgPtr kp = cold();
-    const __bf16* qn = kp->q_nope + tq * kp->qn_st + hq * kp->qn_sh + g * 32;
-    const __bf16* qr = kp->q_rope + tq * kp->qr_st + hq * kp->qr_sh + g * 16;
+    const int ln = lane_now();
+    const int nh = kp->num_heads;
+    const int r0 = grp * 128 + wave * 16;                    // the wave's first row
+    {
+      // latent part: row k of the wave is one copy instruction; lane i brings granule i ^ swz(k) (the tile swizzle)
+      int t = r0 / nh, h = r0 - t * nh;
+      const __bf16* qn0 = kp->q_nope;
+      const int64_t st = kp->qn_st, sh = kp->qn_sh;
 #pragma unroll
-    for (int kk = 0; kk < 16; kk++)
-      asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[kk]) : "v"(qn), "i"((kk & 3) * 256 + (kk >> 2) * 16));
+      for (int k = 0; k < 16; k++) {
+        const bool ok = r0 + k < rows && L > 0;              // rows that do not exist read row 0 of the sequence
+        const __bf16* src = qn0 + (ok ? (int64_t)(q0 + t) * st + (int64_t)h * sh : (int64_t)q0 * st);
+        dma16_sv(src, (uint32_t)((ln ^ swz_nope(k)) << 4), lds0 + wave * 16384 + k * 1024);
+        h++;
+        if (h == nh) { h = 0; t++; }
+      }
+    }
+    {
+      // rope part: eight rows of 128 bytes per instruction, no swizzle (two reads per lane, once per segment)
+      const __bf16* qr0 = kp->q_rope;
+      const int64_t st = kp->qr_st, sh = kp->qr_sh;
 #pragma unroll
-    for (int kk = 0; kk < 2; kk++) asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(qf[16 + kk]) : "v"(qr), "i"(kk * 16));
-    __builtin_amdgcn_s_waitcnt(0x0F70);                                         // vmcnt(0)
+      for (int j = 0; j < 2; j++) {
+        const int rw = r0 + 8 * j + (ln >> 3);
+        const bool ok = rw < rows && L > 0;
+        const int t = rw / nh, h = rw - t * nh;
+        const __bf16* src = qr0 + (ok ? (int64_t)(q0 + t) * st + (int64_t)h * sh : (int64_t)q0 * st) + (ln & 7) * 8;
+        dma16_v(src, lds0 + kPOff + wave * 2048 + j * 1024);
+      }
+    }
+    MLA_WAIT_VMCNT(0);
+    const int ql16 = ln & 15, qg = ln >> 4;
+    const uint32_t qoff = (uint32_t)(wave * 16384 + ql16 * 1024 + (((qg << 2) ^ swz_nope(ql16)) << 4));
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++) qf[kk] = *(const bf16x8*)(lds + (qoff ^ (uint32_t)((kk >> 2) << 4)) + (kk & 3) * 256);
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) qf[16 + kk] = *(const bf16x8*)(lds + kPOff + wave * 2048 + ql16 * 128 + (2 * qg + kk) * 16);
 #pragma unroll
     for (int kk = 0; kk < 18; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
   }
+  lds_barrier();                                              // every wave has read its query: the tile buffers are free
+  TR_PRO(1);
+  issue_first();
 
   f32x16 acc[2][4];                                          // [32-column block of this wave's 64][row group]
 #pragma unroll
@@ -464,6 +578,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     ra[1] = ra[0] ^ 16u;
     IssueCtx ic;
     if constexpr (kIssue) { ids_dma(blk_issue + 1); ic = issue_begin(blk_issue); }
+#ifdef MLA_V3_BURST
+    if constexpr (kIssue) if (copier) {
+#pragma unroll
+      for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::integral_constant<bool, kIssueMode == 2>{});
+    }
+#endif
     bf16x8 ka[kAhead];
     // fragment j: contraction step kk = j >> 1, key group kg = j & 1; each statement is wait + MFMA + the read that
     // refills the fragment register (one statement, so that nothing is scheduled or padded in between)
@@ -494,7 +614,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       else
         asm volatile("s_waitcnt lgkmcnt(%3)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+v"(s[j & 1]) : "v"(ka[j % D]), "v"(qf[j >> 1]), "i"(younger));
-      if constexpr (kIssue) if (j % 7 == 3) issue_piece(ic, j / 7, std::integral_constant<bool, kIssueMode == 2>{});
+#ifndef MLA_V3_BURST
+      if constexpr (kIssue) if (j % 4 == 1 && copier) issue_piece(ic, j / 4, std::integral_constant<bool, kIssueMode == 2>{});
+#endif
     }
 #undef MLA_K_ADDR
 #undef MLA_K_OFF
@@ -666,8 +788,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     issue_next_two();
     // ---- block 0: QK, softmax, publish ----
     {
-      if (nb > 2) MLA_WAIT_VMCNT(10); else if (nb > 1) MLA_WAIT_VMCNT(5); else MLA_WAIT_VMCNT(0);
+      if (nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);   // (kCopies per block in flight)
       lds_barrier();
+      TR_PRO(2);
       f32x4 s[2];
       Sm st;
       qk_block(blk_begin, s, std::integral_constant<int, 0>{}, 0);
@@ -696,7 +819,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       const int blk = blk_begin + i;
       TR_STAMP(tr_a);
       // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
-      if (i + 2 < nb) MLA_WAIT_VMCNT(5); else MLA_WAIT_VMCNT(0);
+      if (i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
       TR_ADD(0);
       lds_barrier();
       if (i + kLead < nb) ids_fetch(blk + kLead);             // (row list) the rows of the block whose copies go out now
@@ -843,10 +966,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   }  // segments
 #ifdef MLA_V3_TRACE
   if (g_trace && lane == 0) {
-    unsigned long long* t = g_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.z) * 8 + wave) * 8;
+    unsigned long long* t = g_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.z) * 8 + wave) * 16;
     for (int k = 0; k < 6; k++) t[k] = tr_t[k];
     t[6] = tr_n;
     t[7] = tr_ep;
+    for (int k = 0; k < 4; k++) t[8 + k] = tr_p[k];
+    t[12] = tr_x0 - tr_start;
   }
 #endif
 }

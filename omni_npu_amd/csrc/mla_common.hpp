@@ -110,6 +110,14 @@ __device__ __forceinline__ void dma4_sv_lanes4(const void* gbase_uniform, uint32
                : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
                : "memory", "m0");
 }
+// the same by lanes 0..7
+__device__ __forceinline__ void dma4_sv_lanes8(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  uint64_t save;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 255\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\ts_mov_b64 exec, %0"
+               : "=&s"(save)
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
+               : "memory", "m0");
+}
 
 // Transposed LDS read: within each group of 16 lanes the 16 addresses name a 4 x 16 block of
 // 16-bit elements (lane 4e+c points at row e, columns 4c..4c+3); lane j receives column j,
