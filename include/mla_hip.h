@@ -180,6 +180,16 @@ int mla_gather_paged(const void* nope_cache, int64_t nope_page_stride, int64_t n
                      int32_t max_blocks, const int32_t* cu_seq_lens, const int32_t* seq_starts /* may be NULL */,
                      int32_t batch, int64_t total_rows_hint, mlahip_stream_t stream);
 
+/* The same gather out of the fp8 block-scaled cache (rows of 656 bytes, see mla_cache_write_fp8): the latent part is
+ * dequantised to bf16 (e4m3 x block scale, rounded once), the rope part copied.  The reference's
+ * gather_and_maybe_dequant_cache (attention/ops.py:5-41) takes kv_cache_dtype and a scale for this case and ignores
+ * them; the chunked-context prefill (attention/backends/mla.py:377-450) needs the dequantised rows. */
+int mla_gather_paged_fp8(const void* cache, int64_t page_stride_bytes, int64_t row_stride_bytes, int64_t num_pages,
+                         int32_t page_size, void* dst, int64_t dst_row_stride, int64_t dst_rows,
+                         const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, const int32_t* cu_seq_lens,
+                         const int32_t* seq_starts /* may be NULL */, int32_t batch, int64_t total_rows_hint,
+                         mlahip_stream_t stream);
+
 int mla_merge_states(const void* prefix_out, int64_t po_stride_t, int64_t po_stride_h, const float* prefix_lse,
                      const void* suffix_out, int64_t so_stride_t, int64_t so_stride_h, const float* suffix_lse,
                      int32_t in_dtype, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,

@@ -30,6 +30,7 @@ SIGNATURES = {
     "mla_decode_fp8": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32, I32, I32, F32, P, I64,
                                  I64, P, P, SZ, I32, P]),
     "mla_gather_paged": (c_int32, [P, I64, I64, P, I64, I64, I64, I32, P, I64, I64, P, I64, I32, P, P, I32, I64, P]),
+    "mla_gather_paged_fp8": (c_int32, [P, I64, I64, I64, I32, P, I64, I64, P, I64, I32, P, P, I32, I64, P]),
     "mla_merge_states": (c_int32, [P, I64, I64, P, P, I64, I64, P, I32, P, I64, I64, I32, P, I32, I32, I32, P]),
     "mla_merge_n_states": (c_int32, [P, I64, I64, I32, P, I64, P, I64, P, I32, I32, I32, P]),
     "mla_decode_workspace_bytes": (SZ, [I32, I32, I32, I32]),

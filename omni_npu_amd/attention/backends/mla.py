@@ -216,7 +216,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             toks = int(cc.seq_tot[i])
             if toks == 0:
                 continue
-            ops.gather_and_maybe_dequant_cache(src_cache=(kv_c_cache, k_pe_cache), dst=cc.workspace,
+            ops.gather_and_maybe_dequant_cache(src_cache=(kv_c_cache,) if k_pe_cache is None else (kv_c_cache, k_pe_cache),
+                                               dst=cc.workspace,
                                                block_table=prefill.block_table, cu_seq_lens=cc.cu_seq_lens[i],
                                                batch_size=attn_metadata.num_prefills, kv_cache_dtype=self.kv_cache_dtype,
                                                scale=k_scale, seq_starts=cc.starts[i], total_rows=toks)
@@ -243,8 +244,6 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         assert prefill is not None
         if self.sink_len > 0:
             return self._forward_prefill_sink(q, kv_c_normed, k_pe, prefill)
-        if self.fp8_cache and prefill.chunked_context is not None:
-            raise NotImplementedError("chunked-context prefill over the fp8 cache is not implemented")
         t, n = q.shape[0], self.num_heads
         has_context = prefill.chunked_context is not None
         q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
@@ -255,7 +254,9 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
                          output, output_lse)
         if has_context:
-            ctx_out, ctx_lse = self._compute_prefill_context(q_nope, q_pe, kv_cache[0], kv_cache[1], attn_metadata, k_scale)
+            # (the fp8 cache is one tensor whose rows hold latent, scales and rope; the gather dequantises it)
+            ctx_out, ctx_lse = self._compute_prefill_context(q_nope, q_pe, kv_cache[0],
+                                                             None if self.fp8_cache else kv_cache[1], attn_metadata, k_scale)
             if ctx_out is not None:
                 merged = torch.empty(t, n, self.v_head_dim, dtype=torch.bfloat16, device=q.device)
                 K.merge_states(ctx_out, ctx_lse, output, output_lse, merged)

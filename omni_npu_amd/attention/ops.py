@@ -23,11 +23,17 @@ def gather_and_maybe_dequant_cache(
     total_rows: Optional[int] = None,
 ) -> None:
     """dst[cu[i]:cu[i+1]] = cat(nope, rope) rows of positions seq_starts[i] .. of sequence i
-    (reference ops.py:5-41).  Like the reference, ``kv_cache_dtype`` and ``scale`` are accepted and unused:
-    no dequantisation happens on this path."""
+    (reference ops.py:5-41).  Over the bf16 caches ``kv_cache_dtype`` and ``scale`` are accepted and unused, as in the
+    reference: no dequantisation happens there.  ``src_cache`` may also be this build's fp8 block-scaled cache (one
+    uint8 tensor [num_blocks, page, 656], alone or as the only member of a tuple): its rows carry their own scales and are
+    dequantised to bf16 on the way."""
     dev = dst.device
     cu = cu_seq_lens.to(device=dev, dtype=torch.int32).contiguous()
     st = None if seq_starts is None else seq_starts.to(device=dev, dtype=torch.int32).contiguous()
+    if torch.is_tensor(src_cache) or len(src_cache) == 1:
+        cache = src_cache if torch.is_tensor(src_cache) else src_cache[0]
+        K.gather_paged_fp8(cache, dst, block_table, cu, batch_size, st, total_rows)
+        return
     K.gather_paged(src_cache[0], src_cache[1], dst, block_table, cu, batch_size, st, total_rows)
 
 

@@ -33,6 +33,46 @@ __global__ __launch_bounds__(256) void gather_paged_kernel(const char* nope, int
   if (lane < 8) *(u32x4*)(d + kDNope * 2 + lane * 16) = *(const u32x4*)(rope + blk * rope_sp + off * rope_sr + lane * 16);
 }
 
+// The same gather out of the fp8 block-scaled cache (rows of 512 e4m3 | 4 fp32 scales | 64 bf16 rope, see
+// cache_write_fp8_kernel): dst row = cat(bf16(e4m3 * block scale), rope), the values the fp8 decode kernel attends over.
+__global__ __launch_bounds__(256) void gather_paged_fp8_kernel(const char* cache, int64_t page_stride_b, int64_t row_stride_b,
+                                                               char* dst, int64_t dst_stride_b, const int32_t* block_table,
+                                                               int64_t bt_stride, int32_t max_blocks,
+                                                               const int32_t* cu_seq_lens, const int32_t* seq_starts,
+                                                               int32_t batch, int32_t page_size, int64_t num_pages,
+                                                               int64_t dst_rows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t total = cu_seq_lens[batch];
+  if (row >= total || row >= dst_rows) return;
+  int lo = 0, hi = batch;                          // largest i with cu[i] <= row
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_seq_lens[mid] <= row) lo = mid; else hi = mid;
+  }
+  const int64_t pos = (seq_starts ? seq_starts[lo] : 0) + (row - cu_seq_lens[lo]);
+  int64_t pg = pos / page_size;
+  const int64_t off = pos - pg * page_size;
+  pg = pg < max_blocks ? pg : max_blocks - 1;
+  int64_t blk = block_table[(int64_t)lo * bt_stride + pg];
+  blk = blk < 0 ? 0 : (blk >= num_pages ? num_pages - 1 : blk);
+  const char* src = cache + blk * page_stride_b + off * row_stride_b;
+  char* d = dst + row * dst_stride_b;
+  const u32x2 q = *(const u32x2*)(src + lane * 8);               // eight e4m3 values
+  const float scale = *(const float*)(src + 512 + (lane >> 4) * 4);   // one scale per 128 elements = 16 lanes
+  bf16x8 o;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const f32x2 lo2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[h], false), hi2 = __builtin_amdgcn_cvt_pk_f32_fp8((int)q[h], true);
+    o[4 * h + 0] = (__bf16)(lo2[0] * scale);
+    o[4 * h + 1] = (__bf16)(lo2[1] * scale);
+    o[4 * h + 2] = (__bf16)(hi2[0] * scale);
+    o[4 * h + 3] = (__bf16)(hi2[1] * scale);
+  }
+  *(bf16x8*)(d + lane * 16) = o;
+  if (lane < 8) *(u32x4*)(d + kDNope * 2 + lane * 16) = *(const u32x4*)(src + 528 + lane * 16);
+}
+
 template <typename T> __device__ __forceinline__ float ld(const T* p) { return (float)*p; }
 template <typename T> __device__ __forceinline__ void st(T* p, float v) { *p = (T)v; }
 
@@ -152,6 +192,26 @@ extern "C" int mla_gather_paged(const void* nope_cache, int64_t nope_page_stride
                      rope_row_stride * 2, (char*)dst, dst_row_stride * 2, block_table, bt_stride, max_blocks, cu_seq_lens,
                      seq_starts, batch, page_size, num_pages, dst_rows);
   return check_launch("mla_gather_paged");
+}
+
+extern "C" int mla_gather_paged_fp8(const void* cache, int64_t page_stride_bytes, int64_t row_stride_bytes, int64_t num_pages,
+                                    int32_t page_size, void* dst, int64_t dst_row_stride, int64_t dst_rows,
+                                    const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                    const int32_t* cu_seq_lens, const int32_t* seq_starts, int32_t batch,
+                                    int64_t total_rows_hint, hipStream_t stream) {
+  MLA_REQUIRE(cache && dst && block_table && cu_seq_lens, MLA_ERR_NULL, "mla_gather_paged_fp8: null pointer argument");
+  MLA_REQUIRE(batch >= 0 && page_size >= 1 && num_pages >= 1 && max_blocks >= 1 && dst_rows >= 0 && total_rows_hint >= 0,
+              MLA_ERR_SHAPE, "mla_gather_paged_fp8: batch=%d page_size=%d num_pages=%lld max_blocks=%d", batch, page_size,
+              (long long)num_pages, max_blocks);
+  MLA_REQUIRE(row_stride_bytes >= 656 && row_stride_bytes % 16 == 0 && page_stride_bytes % 16 == 0 && dst_row_stride % 8 == 0 &&
+                  dst_row_stride >= kDNope + kDRope && (uintptr_t)cache % 16 == 0 && (uintptr_t)dst % 16 == 0,
+              MLA_ERR_SHAPE, "mla_gather_paged_fp8: cache rows are 656 bytes, 16-byte aligned; dst rows at least 576 wide");
+  const int64_t rows = total_rows_hint < dst_rows ? total_rows_hint : dst_rows;
+  if (batch == 0 || rows == 0) return MLA_OK;
+  hipLaunchKernelGGL(gather_paged_fp8_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, stream, (const char*)cache,
+                     page_stride_bytes, row_stride_bytes, (char*)dst, dst_row_stride * 2, block_table, bt_stride, max_blocks,
+                     cu_seq_lens, seq_starts, batch, page_size, num_pages, dst_rows);
+  return check_launch("mla_gather_paged_fp8");
 }
 
 // dtype codes: 0 = bf16, 1 = fp32

@@ -216,6 +216,33 @@ def gather_paged(nope_cache: torch.Tensor, rope_cache: torch.Tensor, dst: torch.
     _lib.check(rc, "mla_gather_paged")
 
 
+def gather_paged_fp8(cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor, cu_seq_lens: torch.Tensor,
+                     batch_size: int, seq_starts: Optional[torch.Tensor] = None, total_rows: Optional[int] = None) -> None:
+    """gather_paged out of the fp8 block-scaled cache (uint8 [num_blocks, page, 656], see cache_write_fp8):
+    dst[cu[i] + j] = cat(bf16(e4m3 * block scale), rope) of position seq_starts[i] + j, the values the fp8 decode attends
+    over (the chunked-context prefill of the reference, attention/backends/mla.py:377-450, over a quantised cache)."""
+    _need_cuda(cache, dst, block_table, cu_seq_lens, seq_starts)
+    lib = _lib.load()
+    if cache.dtype != torch.uint8 or cache.dim() != 3 or cache.shape[-1] != FP8_ROW_BYTES or cache.stride(-1) != 1:
+        raise ValueError(f"fp8 cache must be uint8 [num_blocks, page, {FP8_ROW_BYTES}], got {cache.dtype} {tuple(cache.shape)}")
+    if dst.dim() != 2 or dst.shape[1] < D_NOPE + D_ROPE or dst.stride(1) != 1 or dst.dtype != torch.bfloat16:
+        raise ValueError("gather_paged_fp8: dst must be bf16 [rows, >=576]")
+    if block_table.dtype != torch.int32 or cu_seq_lens.dtype != torch.int32 or not cu_seq_lens.is_contiguous():
+        raise TypeError("gather_paged_fp8: block_table and cu_seq_lens must be int32 (cu_seq_lens contiguous)")
+    if block_table.dim() != 2 or block_table.stride(1) != 1 or block_table.shape[0] < batch_size:
+        raise ValueError("gather_paged_fp8: block_table must be [>= batch, max_blocks] with contiguous rows")
+    if seq_starts is not None and (seq_starts.dtype != torch.int32 or not seq_starts.is_contiguous()):
+        raise TypeError("gather_paged_fp8: seq_starts must be contiguous int32")
+    if cu_seq_lens.numel() < batch_size + 1:
+        raise ValueError("gather_paged_fp8: cu_seq_lens needs batch_size + 1 entries")
+    rows = dst.shape[0] if total_rows is None else min(int(total_rows), dst.shape[0])
+    rc = lib.mla_gather_paged_fp8(cache.data_ptr(), cache.stride(0), cache.stride(1), cache.shape[0], cache.shape[1],
+                                  dst.data_ptr(), dst.stride(0), dst.shape[0], block_table.data_ptr(), block_table.stride(0),
+                                  block_table.shape[1], cu_seq_lens.data_ptr(),
+                                  seq_starts.data_ptr() if seq_starts is not None else None, batch_size, rows, _stream(dst))
+    _lib.check(rc, "mla_gather_paged_fp8")
+
+
 _DT = {torch.bfloat16: 0, torch.float32: 1}
 
 

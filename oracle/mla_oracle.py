@@ -330,6 +330,40 @@ def rms_norm(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> torch.Tensor:
     return (xd * inv * gamma.double()).to(x.dtype)
 
 
+def yarn_rope_tables(positions, rotary_dim: int = D_ROPE, base: float = 10000.0, scaling_factor: float = 40.0,
+                     original_max_position: int = 4096, beta_fast: float = 32, beta_slow: float = 1, mscale: float = 1.0,
+                     mscale_all_dim: float = 0.0, attn_factor: float = 1.0, dtype=torch.bfloat16):
+    """cos / sin rows cat(c, c) of the YaRN-scaled rotary embedding DeepSeek-V2/V3 use
+    (layers/rotary_embedding/deepseek_scaling_rope.py:51-87; the helper functions it imports from vLLM are not in the
+    reference tree: this is the published YaRN formulation, written as loops over the pairs in float64).
+    Pair i rotates at f_i = base^(-2i/d); pairs that turn more than beta_fast times over the original context keep f_i,
+    pairs that turn less than beta_slow times get f_i / factor, a linear ramp over the pair index lies between; the
+    values are scaled by (0.1 m ln(factor) + 1) / (0.1 m_all ln(factor) + 1) * attn_factor."""
+    import math
+    half = rotary_dim // 2
+
+    def corr(rot):
+        return rotary_dim * math.log(original_max_position / (rot * 2 * math.pi)) / (2 * math.log(base))
+
+    low, high = max(math.floor(corr(beta_fast)), 0), min(math.ceil(corr(beta_slow)), rotary_dim - 1)
+    if low == high:
+        high += 0.001
+
+    def ms(m):
+        return 1.0 if scaling_factor <= 1 else 0.1 * m * math.log(scaling_factor) + 1.0
+
+    scale = ms(mscale) / ms(mscale_all_dim) * attn_factor
+    inv = []
+    for i in range(half):
+        f = float(base) ** (-2.0 * i / rotary_dim)
+        ramp = min(max((i - low) / (high - low), 0.0), 1.0)      # 0: keep (extrapolate), 1: divide (interpolate)
+        inv.append(f * (1.0 - ramp) + f / scaling_factor * ramp)
+    inv = torch.tensor(inv, dtype=torch.float64)
+    ang = torch.outer(torch.as_tensor(positions).double(), inv)
+    c, s = ang.cos() * scale, ang.sin() * scale
+    return torch.cat((c, c), -1).to(dtype), torch.cat((s, s), -1).to(dtype)
+
+
 def interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, table: str = "half",
                     interleaved_out: bool = False) -> torch.Tensor:
     """x [T, ..., D] with pairs (2i, 2i+1); cos / sin [T, W] rows.  x1 = x[..., 0::2], x2 = x[..., 1::2],
@@ -378,6 +412,14 @@ def fp8_quant_block(x: torch.Tensor, block: int = FP8_BLOCK):
 def fp8_dequant_block(q: torch.Tensor, scale: torch.Tensor, block: int = FP8_BLOCK) -> torch.Tensor:
     xs = q.float().reshape(*q.shape[:-1], -1, block)
     return (xs * scale.unsqueeze(-1)).reshape(q.shape)
+
+
+def gather_paged_fp8(q8, scales, rope_cache, dst, block_table, cu_seq_lens, batch_size, seq_starts=None):
+    """gather_paged over a block-scaled fp8 latent cache: q8 [nblk, page, 512] e4m3 with scales [nblk, page, 4] and the bf16
+    rope cache; a destination row is cat(bf16(q8 * scale), rope) (one rounding: the fp32 product to bf16).  The chunked
+    context of attention/backends/mla.py:377-450 over a quantised cache; no reference format exists (closed form)."""
+    nope = fp8_dequant_block(q8, scales).to(torch.bfloat16)
+    gather_paged(nope, rope_cache, dst, block_table, cu_seq_lens, batch_size, seq_starts)
 
 
 def fp8_quant_token(x: torch.Tensor):

@@ -87,6 +87,53 @@ def test_mla_impl_forward_matches_reference_semantics(dev, q_lens, seq_lens, n):
     attn_close(out[:t], ref, 3e-2, 8e-3)                                                # the reference's 3e-2 bar
 
 
+def test_mla_impl_forward_fp8_cache_with_chunked_context(dev):
+    """NPUMLAImpl.forward over the fp8 block-scaled cache, mixed batch: decodes read the quantised cache (the new token
+    included), prefills attend over their own un-quantised suffix plus a chunked context gathered and dequantised from
+    the cache (two chunks of the 64-row workspace).  The oracle sees exactly those values."""
+    from omni_npu_amd import kernels as K
+    q_lens, seq_lens, n = [1, 1, 16, 16], [300, 77, 112, 64], 4
+    g = torch.Generator().manual_seed(11)
+    common = _common(q_lens, seq_lens)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    q = torch.randn(t, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(t, 512, generator=g).bfloat16(), torch.randn(t, 1, 64, generator=g).bfloat16()
+    common.slot_mapping = torch.cat([O.slots_for(common.block_table_tensor, b, s - ql, s)
+                                     for b, (ql, s) in enumerate(zip(q_lens, seq_lens))])
+    impl, w = _mk_impl(mla.NPUMLAImpl, n, dev, kv_cache_dtype="fp8")
+    builder = mla.NPUMLAMetadataBuilder(V.AttentionSpec(128, 1, 576, torch.bfloat16), ["l"], _cfg(cap=2), dev)
+    builder.chunked_prefill_workspace_size = 64
+    deq = lambda x: O.fp8_dequant_block(*O.fp8_quant_block(x.float()))
+    # oracle: what the cache holds after the write, dequantised; prefill suffixes use the raw new latents
+    nope_q, rope_c = deq(nope), rope.clone().float()
+    O.cache_write(nope_q, common.slot_mapping, deq(kvc))
+    O.cache_write(rope_c, common.slot_mapping, kpe.view(-1, 64).float())
+    qsl = common.query_start_loc_cpu.tolist()
+    ref = torch.zeros(t, n * 128)
+    for b in range(common.num_reqs):
+        L, q0, q1 = seq_lens[b], qsl[b], qsl[b + 1]
+        rows = O.slots_for(common.block_table_tensor.cpu(), b, 0, L)
+        lat, pe = nope_q.view(-1, 512)[rows].clone(), rope_c.view(-1, 64)[rows]
+        if q_lens[b] > 1:
+            lat[L - q_lens[b]:] = kvc[q0:q1].float()            # the suffix is attended before it is quantised
+        kn, vv = O.kv_up_proj(lat, w.float(), n, 128, 128)
+        o, _ = O.attention_varlen(q[q0:q1, :, :128].float(), q[q0:q1, :, 128:].float(), kn, pe, vv, [0, q1 - q0], [0, L],
+                                  impl.scale, True)
+        ref[q0:q1] = o.reshape(q1 - q0, -1)
+    meta = builder.build(0, _to(common, dev))
+    assert meta.prefill.chunked_context is not None and len(meta.prefill.chunked_context.seq_tot) >= 2
+    raw = torch.zeros(nblk * 128 * 656, dtype=torch.uint8, device=dev)
+    kv_cache = mla.NPUMLABackend.reshape_kv_cache(raw, nblk, 128, 1, 656, dtype=torch.uint8)
+    K.cache_write_fp8(nope.view(-1, 512).to(dev), rope.view(-1, 64).to(dev),
+                      torch.arange(nblk * 128, dtype=torch.int64, device=dev), kv_cache[0])
+    out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    impl.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), kv_cache, meta, output=out)
+    attn_close(out, ref, 3e-2, 8e-3)
+
+
 def test_dsa_impl_forward_with_indexer(dev):
     """Indexer (quantise, cache K, fp8 logits, top-k) -> NPUDSAImpl.forward; checked against the oracle's sparse
     attention on the index set the GPU selected, and the set against the oracle's selection on the GPU's logits."""

@@ -58,6 +58,41 @@ def test_gather_paged_matches_oracle(dev):
     assert torch.equal(dst2.cpu(), ref2)
 
 
+def test_gather_paged_fp8_matches_oracle(dev):
+    """The dequantising gather out of the fp8 cache: every row equals cat(bf16(e4m3 * block scale), rope) bit for bit."""
+    from omni_npu_amd import kernels as K
+    case = O.make_decode_case(5, 16, 200, 900, seed=22)
+    nblk = case["nope"].shape[0]
+    g = torch.Generator().manual_seed(5)
+    lat = (case["nope"].float() * (torch.rand(nblk, 128, 1, generator=g) * 6)).bfloat16()    # block scales of many sizes
+    lat[0, 3, 128:256] = 0                                                                   # an all-zero block (scale 1)
+    cache = torch.zeros(nblk, 128, 656, dtype=torch.uint8, device=dev)
+    K.cache_write_fp8(lat.view(-1, 512).to(dev), case["rope"].view(-1, 64).to(dev),
+                      torch.arange(nblk * 128, dtype=torch.int64, device=dev), cache)
+    q8, sc = O.fp8_quant_block(lat.float())                    # (the cache write is pinned bit-exact against this)
+    lens = case["seq_lens"]
+    starts = torch.tensor([0, 17, 128, 5, 300], dtype=torch.int32)
+    n = torch.minimum(lens - starts, torch.tensor([150, 0, 256, 64, 1], dtype=torch.int32))
+    cu = torch.zeros(6, dtype=torch.int32)
+    cu[1:] = torch.cumsum(n, 0)
+    tot = int(cu[-1])
+    for st in (starts, None):
+        ref = torch.zeros(tot + 3, 576, dtype=torch.bfloat16)
+        O.gather_paged_fp8(q8, sc, case["rope"], ref, case["block_table"], cu, 5, st)
+        dst = torch.zeros(tot + 3, 576, dtype=torch.bfloat16, device=dev)
+        K.gather_paged_fp8(cache, dst, case["block_table"].to(dev), cu.to(dev), 5, None if st is None else st.to(dev))
+        assert torch.equal(dst.cpu().view(torch.int16), ref.view(torch.int16))
+    # the reference-named entry takes the one-tensor cache as well
+    from omni_npu_amd.attention import ops
+    dst = torch.zeros(tot, 576, dtype=torch.bfloat16, device=dev)
+    ops.gather_and_maybe_dequant_cache((cache,), dst, case["block_table"].to(dev), cu.to(dev), 5, "fp8", None, starts.to(dev), tot)
+    ref = torch.zeros(tot, 576, dtype=torch.bfloat16)
+    O.gather_paged_fp8(q8, sc, case["rope"], ref, case["block_table"], cu, 5, starts)
+    assert torch.equal(dst.cpu().view(torch.int16), ref.view(torch.int16))
+    with pytest.raises(ValueError):
+        K.gather_paged_fp8(cache.view(nblk, 128 * 656), dst, case["block_table"].to(dev), cu.to(dev), 5)
+
+
 @pytest.mark.parametrize("in_dt,out_dt", [(torch.bfloat16, torch.float32), (torch.float32, torch.float32),
                                           (torch.bfloat16, torch.bfloat16)])
 def test_merge_states_matches_oracle(dev, in_dt, out_dt):
