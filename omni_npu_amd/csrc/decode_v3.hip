@@ -559,7 +559,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   // P^T in LDS, in the order the P.V MFMAs read it: fragment (row group rg, k-block kb) is 64 lanes x 16 B, lane
   // (n = row % 32, h) holding keys 16kb + {4h..4h+3, 8+4h..8+4h+3}.  The QK lane (row l16 of wave w, group g) holds keys
   // 16kg + 4g + {0..3}: they are the first (g < 2) or second (g >= 2) 8 bytes of lane (n, h = g & 1).
-  const uint32_t p_w_off = (uint32_t)(kPOff + (((wave >> 1) * 2) * 64 + (g & 1) * 32 + (wave & 1) * 16 + l16) * 16 + (g >> 1) * 8);   // + kg*1024 + parity*8192
+  // (worked out from the hardware lane number where it is used: a register held for it through the loop was the one the
+  // compiler chose to spill, and a scratch reload waits for every copy in flight)
+  auto p_w_off_now = [&]() -> uint32_t {
+    const int ln = lane_now(), pg = ln >> 4, pl = ln & 15;
+    return (uint32_t)(kPOff + (((wave >> 1) * 2) * 64 + (pg & 1) * 32 + (wave & 1) * 16 + pl) * 16 + (pg >> 1) * 8);   // + kg*1024 + parity*8192
+  };
 
   // S^T for block `blk`: hand-placed K-fragment reads kAhead fragments ahead of the MFMA that consumes them, explicit
   // lgkmcnt waits, MFMAs as assembly with the scores in ordinary vector registers (the accumulation file is full of
@@ -741,7 +746,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
       top_tag = nw ? (int)((uint32_t)(blk << 3) | (st.mx & 7u)) : top_tag;   // decoded in the epilogue
     }
     l_run += st.psum;
-    const uint32_t pw = lds0 + (blk & 1) * kPBufB + p_w_off;
+    const uint32_t pw = lds0 + (blk & 1) * kPBufB + p_w_off_now();
     const u32x2 w0 = {st.pw[0], st.pw[1]}, w1 = {st.pw[2], st.pw[3]};
     asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %2 offset:1024" :: "v"(pw), "v"(w0), "v"(w1) : "memory");
     const bool flag = st.t > kRestartThreshold;               // asks the workgroup to restart with better references
@@ -810,7 +815,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
     }
     // Everything the loop keeps in registers is touched here: a value that was parked in scratch during the prologue is
     // brought back (and waited for) now, not at its first use inside the loop.
-    asm volatile("" :: "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(p_w_off), "v"(dma_off));
+    asm volatile("" :: "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(dma_off));
     // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
 #ifdef MLA_V3_TRACE
     if (tr_t[5] == 0) { TR_STAMP(tr_b); tr_t[5] = tr_b - tr_start; }
