@@ -620,7 +620,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
         asm volatile("s_waitcnt lgkmcnt(%3)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+v"(s[j & 1]) : "v"(ka[j % D]), "v"(qf[j >> 1]), "i"(younger));
 #ifndef MLA_V3_BURST
-      if constexpr (kIssue) if (j % 4 == 1 && copier) issue_piece(ic, j / 4, std::integral_constant<bool, kIssueMode == 2>{});
+      if constexpr (kIssue) if (j % 4 == 1) issue_piece(ic, j / 4, std::integral_constant<bool, kIssueMode == 2>{});   // (copying waves only get here)
 #endif
     }
 #undef MLA_K_ADDR
@@ -837,7 +837,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
 #elif defined(ABL_NO_COPY)
       if (true) { qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0); s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0]; }
 #else
-      if (i + kLead >= nb) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
+      // (the wavefronts that copy nothing take the variant without copies: no branch around each copy, no page arithmetic)
+      if (i + kLead >= nb || !copier) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
 #endif
       else if (kSparse || !full_ok || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead);
       else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + kLead);
