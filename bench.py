@@ -680,8 +680,13 @@ def main():
     ap.add_argument("--splits", type=int, default=0, help="KV splits per sequence (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true",
-                    help="replay the step as a captured HIP graph instead of launching its kernels one by one (measured "
-                         "slower on this ROCm: replay adds more between kernels than the launches it saves)")
+                    help="decode workload: replay the steps from captured HIP graphs instead of launching their kernels one by "
+                         "one.  Measured slower on this part: a graph leaves no idle time between kernels, the engine clock "
+                         "drops within a millisecond, and every kernel of the graph runs 25-30 % longer than in the eager "
+                         "queue, whose few microseconds between launches keep the clock up")
+    ap.add_argument("--graph-layers", type=int, default=10,
+                    help="with --graph: steps captured into one HIP graph, as a model captures all its layers in one; the "
+                         "largest divisor of --steps up to this number is used")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
@@ -739,27 +744,40 @@ def main():
                  q_len=q_len, num_splits=splits, workspace=ws)
 
     eager_step = step
+    # The timed region is args.steps steps, queued without a host wait in between, bracketed by synchronisations on the
+    # host and by one pair of HIP events on the launch stream.  --graph replays them from captured HIP graphs (the
+    # product's decode path can: compilation/acl_graph.py), `layers` steps per graph the way a model captures its layers.
+    layers = 1
     if args.graph:
-        # the product's decode path can replay a captured HIP graph (compilation/acl_graph.py)
+        layers = max(d for d in range(1, max(1, args.graph_layers) + 1) if args.steps % d == 0)
         for _ in range(3):
             eager_step()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            eager_step()
+            for _ in range(layers):
+                eager_step()
         step = graph.replay
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    us_per_step = wall / args.steps * 1e6
+    def timed(fn, calls):
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        a.record()
+        for _ in range(calls):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, a.elapsed_time(e) * 1e-3
 
-    # device-side time of the whole step and of the dominant kernel alone (events on the launch stream)
+    for _ in range(-(-args.warmup // layers)):
+        step()
+    wall, dev_s = timed(step, args.steps // layers)
+    us_per_step = wall / args.steps * 1e6
+    dev_step_avg = dev_s / args.steps * 1e6
+
+    # per-call brackets (an event pair around every call): the time of a call that starts on an idle queue, dispatch latency
+    # included
     def event_time(fn, n):
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
         for a, e in ev:
@@ -770,10 +788,17 @@ def main():
         ts = sorted(a.elapsed_time(e) * 1e3 for a, e in ev)
         return sum(ts) / len(ts), ts[len(ts) // 2]
 
-    dev_step_avg, dev_step_med = event_time(step, args.steps)
+    eager_wall, eager_dev = timed(eager_step, args.steps)
+    eager_iso_avg, eager_iso_med = event_time(eager_step, args.steps)
+    # the dominant kernel alone: args.steps launches queued back to back between one pair of events (the launches are
+    # shorter on the host than on the GPU, so the queue never runs dry), and the per-launch brackets beside it
     split_only = lambda: K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], g["block_table"], g["seq_lens"],
                                   case["scale"], out_v, q_len=q_len, num_splits=splits, workspace=ws, phase="split")
-    k_avg, k_med = event_time(split_only, args.steps)
+    for _ in range(3):
+        split_only()
+    _, k_dev = timed(split_only, args.steps)
+    k_avg = k_dev / args.steps * 1e6
+    k_iso_avg, k_med = event_time(split_only, args.steps)
 
     ab = algorithmic_bytes(case, heads)
     sum_l = int(case["seq_lens"].sum())
@@ -793,7 +818,11 @@ def main():
                    "q_len": q_len, "seq_lens": f"uniform[{args.len_lo},{args.len_hi}]", "sum_seq_len": sum_l,
                    "page": 128, "kv_splits": splits, "seed": args.seed},
         "step_us": {"host_wall": round(us_per_step, 2), "device_avg": round(dev_step_avg, 2),
-                    "device_median": round(dev_step_med, 2), "launch": "hip graph replay" if args.graph else "eager launches"},
+                    "launch": f"hip graph replay, {layers} steps per graph" if args.graph else "eager launches, queued",
+                    "eager_host_wall": round(eager_wall / args.steps * 1e6, 2),
+                    "eager_device_queued": round(eager_dev / args.steps * 1e6, 2),
+                    "eager_device_one_step_alone_avg": round(eager_iso_avg, 2),
+                    "eager_device_one_step_alone_median": round(eager_iso_med, 2)},
         "step_tflops": round(flops / (dev_step_avg * 1e-6) / 1e12, 1),
         "step_hbm_gbs": round(ab["total"] / (dev_step_avg * 1e-6) / 1e9, 1),
         "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
@@ -801,7 +830,8 @@ def main():
         "roofline": {"kernel": "mla_decode_v3_kernel<false, false>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "traffic_source": traffic_src,
-                     "kernel_us_avg": round(k_avg, 2), "kernel_us_median": round(k_med, 2),
+                     "kernel_us_avg": round(k_avg, 2), "kernel_us_one_launch_alone_avg": round(k_iso_avg, 2),
+                     "kernel_us_one_launch_alone_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),
                      "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
     }
