@@ -4,9 +4,9 @@
 // (src/omni_npu/attention/backends/mla.py:781-804): for sequence b, head n, query token t
 //   s_j = scale * (ql[t,n] . Kc[j] + qr[t,n] . Kr[j]),  j < L_b - (q_len-1-t)   (right-down causal)
 //   o   = sum_j softmax(s)_j * Kc[j]
-// with ONE latent KV row (512 + 64) shared by all heads.  The kernels live in decode_v2.hip (bf16 cache, dense and
-// row-list sources, and the merge of the split-KV partials: the N-way merge of src/omni_npu/attention/ops.py:109-141)
-// and decode_v2_fp8.hip (fp8-e4m3 block-scaled cache).
+// with ONE latent KV row (512 + 64) shared by all heads.  The kernels live in decode_v3.hip (bf16 cache: dense, row-list
+// and sink + window sources), decode_v3_fp8.hip (fp8-e4m3 block-scaled cache) and chunk_reduce.hip (the merge of the
+// split-KV partials: the N-way merge of src/omni_npu/attention/ops.py:109-141).
 //
 // Workspace (mla_decode_workspace_bytes): batch * (num_splits + 1) partial slots of rows = max_q_len * num_heads each:
 // normalised fp16 partials [slots, rows, 512], fp32 log-sum-exps [slots, rows], a correction record per row (fp32
@@ -14,7 +14,7 @@
 #include <cstdlib>
 #include <mutex>
 #include "mla_common.hpp"
-#include "decode_v2_params.hpp"
+#include "decode_params.hpp"
 
 namespace mlahip {
 constexpr int kRowsPerWg = 128;
@@ -66,7 +66,7 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   const size_t rows = (size_t)batch * ((size_t)num_splits + 1) * r_max;
   MLA_REQUIRE((int64_t)batch * num_splits <= 0x7fffffff / 2 && nope_row_stride < (1 << 28) && rope_row_stride < (1 << 28),
               MLA_ERR_SHAPE, "mla_decode_bf16: batch * num_splits or a row stride is out of range");
-  DecodeV2Params v;
+  DecodeParams v;
   v.q_nope = (const __bf16*)q_nope; v.qn_st = qn_stride_t; v.qn_sh = qn_stride_h;
   v.q_rope = (const __bf16*)q_rope; v.qr_st = qr_stride_t; v.qr_sh = qr_stride_h;
   v.nope = (const __bf16*)nope_cache; v.nope_sp = nope_page_stride; v.nope_sr = nope_row_stride;
@@ -84,11 +84,8 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   v.win_skip = win_skip; v.win_sink = win_sink; v.win_size = win_size;
   // one workgroup per (balanced chunk, group of 128 query rows)
   const dim3 grid((unsigned)(batch * num_splits), 1, (unsigned)((r_max + kRowsPerWg - 1) / kRowsPerWg));
-  if (fp8) return launch_decode_v2_fp8(v, grid, stream);
-  static const bool use_v2 = getenv("MLA_DECODE_V2") != nullptr;
-  if (!use_v2) return launch_decode_v3(v, sparse_rows != nullptr, grid, stream);
-  if (win_skip) return launch_decode_v2_window(v, grid, stream);
-  return launch_decode_v2(v, sparse_rows != nullptr, grid, stream);
+  if (fp8) return launch_decode_v3_fp8(v, grid, stream);
+  return launch_decode_v3(v, sparse_rows != nullptr, grid, stream);
 }
 
 // Phase 1: one normalised fp16 partial + log-sum-exp per (segment of a chunk, query row) into the workspace.

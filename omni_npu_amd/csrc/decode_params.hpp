@@ -1,10 +1,11 @@
-// Parameters and launcher of the second-generation absorbed-MLA decode kernel (decode_v2.hip).
+// Parameters and launchers of the absorbed-MLA split-KV decode kernels (decode_v3.hip, decode_v3_fp8.hip), of the merge
+// of their partials (chunk_reduce.hip) and of the merge fused with the value up-projection (reduce_vup.hip).
 #pragma once
 #include "mla_common.hpp"
 
 namespace mlahip {
 
-struct DecodeV2Params {
+struct DecodeParams {
   const __bf16* q_nope; int64_t qn_st, qn_sh;
   const __bf16* q_rope; int64_t qr_st, qr_sh;
   const __bf16* nope; int64_t nope_sp, nope_sr;
@@ -48,13 +49,10 @@ __device__ __forceinline__ int plan_work_units(int len) { return len > 0 ? (len 
 int launch_reduce_vup(const ChunkReduceParams& r, const void* w_uv, int64_t w_stride_n, int64_t w_stride_k,
                       int32_t num_tokens, hipStream_t stream);
 
-// Launches mla_decode_v2_kernel<sparse> on `stream`; returns 0 or a negative error code.
-int launch_decode_v2(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
-// The dense kernel with a sink and a sliding window (p.win_skip set).
-int launch_decode_v2_window(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
-// The eight-wavefront kernel (decode_v3.hip): dense, row-list (sparse) and, with p.win_skip set, sink + window.
-int launch_decode_v3(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream);
-// Launches mla_decode_v2_fp8_kernel (decode_v2_fp8.hip) over p.cache8.
-int launch_decode_v2_fp8(const DecodeV2Params& p, dim3 grid, hipStream_t stream);
+// The eight-wavefront kernel over the bf16 cache (decode_v3.hip): dense, row-list (sparse) and, with p.win_skip set, sink +
+// window.  Returns 0 or a negative error code.
+int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream);
+// The same over the fp8 block-scaled cache p.cache8 (decode_v3_fp8.hip): dense and, with p.win_skip set, sink + window.
+int launch_decode_v3_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream);
 
 }  // namespace mlahip

@@ -27,7 +27,7 @@
 // for the row's most probable key, and combine them in the epilogue.
 // Partials: normalised fp16 through an LDS transpose, fp32 natural-log LSE, and the dominant-key correction record that
 // mla_chunk_reduce_kernel applies (the bf16 rounding of the largest probability is the biggest single error of P.V).
-#include "decode_v2_params.hpp"
+#include "decode_params.hpp"
 #include <type_traits>
 #include <cstdlib>
 
@@ -111,7 +111,7 @@ __device__ unsigned long long* g_trace;                     // [workgroup][wave]
 #endif
 
 template <bool kSparse, bool kWindow>
-__global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params p) {
+__global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p) {
   static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 #ifdef MLA_V3_TRACE
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
   // Arguments that only the start and the end of a segment need are read from the argument block where they are used
   // (through a pointer the compiler cannot see through), not held in scalar registers across the block loop: the loop
   // needs most of them itself, and scalar registers that overflow are parked in vector registers, which are short here.
-  typedef __attribute__((address_space(4))) const DecodeV2Params* KernArgPtr;
+  typedef __attribute__((address_space(4))) const DecodeParams* KernArgPtr;
   auto cold = [] {
     KernArgPtr kp = (KernArgPtr)__builtin_amdgcn_kernarg_segment_ptr();
     asm volatile("" : "+s"(kp));
@@ -984,7 +984,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeV2Params
 
 }  // namespace v3
 
-int launch_decode_v3(const DecodeV2Params& p, bool sparse, dim3 grid, hipStream_t stream) {
+int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream) {
   const void* kernel = sparse ? (const void*)v3::mla_decode_v3_kernel<true, false>
                               : (p.win_skip ? (const void*)v3::mla_decode_v3_kernel<false, true>
                                             : (const void*)v3::mla_decode_v3_kernel<false, false>);

@@ -119,6 +119,15 @@ __device__ __forceinline__ void dma4_sv_lanes8(const void* gbase_uniform, uint32
                : "memory", "m0");
 }
 
+// a 16-byte copy by lanes 0..7 only (128 bytes): lane i's bytes land at lds_addr + 16 * i
+__device__ __forceinline__ void dma16_sv_lanes8(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  uint64_t save;
+  asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, 255\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, %0"
+               : "=&s"(save)
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+
 // Transposed LDS read: within each group of 16 lanes the 16 addresses name a 4 x 16 block of
 // 16-bit elements (lane 4e+c points at row e, columns 4c..4c+3); lane j receives column j,
 // i.e. the four rows' elements at that column.

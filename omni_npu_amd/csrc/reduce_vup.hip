@@ -13,7 +13,7 @@
 // first MFMA operand (32 output columns per wavefront), read with transposed LDS reads exactly like V^T in the decode
 // kernel, the merged rows are the second operand, so a lane ends up with four consecutive output columns of one token.
 #include "mla_common.hpp"
-#include "decode_v2_params.hpp"
+#include "decode_params.hpp"
 
 namespace mlahip {
 namespace {
