@@ -51,6 +51,43 @@ def test_decode_fp8_matches_oracle(dev, batch, heads, lo, hi, q_len, splits):
         assert (out.float().cpu() - ref_full).abs().max().item() <= FP8_MAX_ABS
 
 
+@pytest.mark.parametrize("num_splits", [1, 4])
+def test_decode_fp8_scores_that_outgrow_the_first_block(dev, num_splits):
+    """The fp8 kernel fixes a row's softmax reference at its first block too and restarts the segment when a later score
+    exceeds it by more than 2^100; the scores that raised the flag are kept per row and become the new references.  Keys
+    planted late in the sequences (scores ~110 and ~220 natural units above the rest) exercise one and two restarts."""
+    from omni_npu_amd import kernels as K
+    c = O.make_decode_case(3, 128, 1500, 2500, seed=23)
+    lens = c["seq_lens"].tolist()
+
+    def plant(b, pos, head, gain):
+        page = c["block_table"][b, pos // 128].long()
+        c["nope"][page, pos % 128] = (gain * c["q_nope"][b, head].float()).bfloat16()
+    plant(0, lens[0] - 40, 3, 3.0)                             # one restart, late in the last chunk
+    plant(1, 700, 5, 3.0)
+    plant(1, 1400, 5, 6.0)                                     # two restarts for head 5 of sequence 1
+    plant(2, 7, 9, 4.0)                                        # the maximum sits in the first block: no restart
+    q8, sc = O.fp8_quant_block(c["nope"].float())
+    deq = O.fp8_dequant_block(q8, sc)
+    cache = _fill_cache(c, dev)
+    out = torch.empty(3, 128, 512, dtype=torch.bfloat16, device=dev)
+    K.decode_fp8(c["q_nope"].to(dev), c["q_rope"].to(dev), cache, c["block_table"].to(dev), c["seq_lens"].to(dev),
+                 c["scale"], out, num_splits=num_splits)
+    ref = O.absorbed_decode(c["q_nope"], c["q_rope"], deq, c["rope"], c["block_table"], c["seq_lens"], c["scale"])
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    for b, pos, head in ((0, lens[0] - 40, 3), (1, 1400, 5), (2, 7, 9)):   # these heads return the planted row
+        row = deq[c["block_table"][b, pos // 128].long(), pos % 128]
+        assert (got[b, head] - row).abs().max().item() <= 2 ** -7 * row.abs().max().item()
+    # The planted rows hold values up to ~25 and leak into other heads of their sequences; this kernel has no dominant-key
+    # correction, so the bf16 rounding of a large probability (2^-9) times such values is its largest error: the absolute bar
+    # is scaled by the magnitude of each output row, with a quarter of slack for exactly that term.
+    err = (got - ref).abs()
+    bar = 1.25 * FP8_MAX_ABS * ref.abs().amax(dim=-1, keepdim=True).clamp_min(1.0)
+    assert (err <= bar).all(), f"worst excess {(err / bar).max().item():.3f} x the bar"
+    assert (err.sum() / ref.abs().sum()).item() <= FP8_MEAN_REL
+
+
 def test_decode_step_replayed_from_a_hip_graph(dev):
     """Cache write + fp8 decode captured once; the graph is replayed with NEW sequence lengths, slots and queries
     written into the same device buffers, with eager work between replays, and every replay is checked."""
