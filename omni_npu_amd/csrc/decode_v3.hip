@@ -16,7 +16,7 @@
 //                    v_mfma_f32_32x32x16_bf16 per block, V^T fragments by transposed LDS reads of the same rows.
 // P^T (bf16) travels through LDS once per block (8 KiB, double buffered), one workgroup barrier per block.
 //
-// Pipeline:  body i = [barrier] QK(i+1) with the copies of block i+3 spread between its MFMAs | PV(i) with the softmax of
+// Pipeline:  body i = [barrier] the copies of block i+3 (wavefronts 0..3), QK(i+1) | PV(i) with the softmax of
 // block i+1 cut into steps between the MFMA groups | publish P(i+1).
 //
 // Softmax with a fixed reference (no accumulator rescaling: vector ALU instructions cannot touch the accumulation
@@ -374,8 +374,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       pg_nxt = load_page(page_cur + 1);
     }
   };
-  // The nine copies of a block are issued one at a time ("pieces") so that they can be spread over the MFMAs of the QK
-  // phase.  Rows past the end of the sequence re-read its last row (their scores are masked).
+  // The nine copies of a block ("pieces").  Rows past the end of the sequence re-read its last row (their scores are masked).
   // rope buffer of a block: (blk - blk_begin + rope_ph) % 3 without a division (rope_ph = blk_begin % 3 once per segment)
   const int rope_ph = blk_begin % 3;
   auto rope_buf_of = [&](int blk) -> int {
@@ -583,12 +582,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     ra[1] = ra[0] ^ 16u;
     IssueCtx ic;
     if constexpr (kIssue) { ids_dma(blk_issue + 1); ic = issue_begin(blk_issue); }
-#ifdef MLA_V3_BURST
-    if constexpr (kIssue) if (copier) {
+    // All nine copies go out here, in front of the wave's K reads: the copying wave then runs its S phase a few hundred
+    // clocks behind the other wave of its SIMD (which copies nothing), and the two want the LDS and the matrix pipe at
+    // different moments (measured against the copies spread between the MFMAs: 121.8 / 123.4 -> 119.5 / 121.5 us).
+    if constexpr (kIssue) {
 #pragma unroll
       for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::integral_constant<bool, kIssueMode == 2>{});
     }
-#endif
     bf16x8 ka[kAhead];
     // fragment j: contraction step kk = j >> 1, key group kg = j & 1; each statement is wait + MFMA + the read that
     // refills the fragment register (one statement, so that nothing is scheduled or padded in between)
@@ -619,9 +619,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       else
         asm volatile("s_waitcnt lgkmcnt(%3)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+v"(s[j & 1]) : "v"(ka[j % D]), "v"(qf[j >> 1]), "i"(younger));
-#ifndef MLA_V3_BURST
-      if constexpr (kIssue) if (j % 4 == 1) issue_piece(ic, j / 4, std::integral_constant<bool, kIssueMode == 2>{});   // (copying waves only get here)
-#endif
     }
 #undef MLA_K_ADDR
 #undef MLA_K_OFF
