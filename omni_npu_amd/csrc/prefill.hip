@@ -133,9 +133,14 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
   int limit = p.causal ? row + shift + 1 : sk;                // visible keys of this row
   limit = !row_ok ? 0 : (limit < 0 ? 0 : (limit > sk ? sk : limit));
   int wave_min_limit = limit;                                 // fewest keys any row of this wave can see
+  int wave_max_limit = limit;                                 // most keys any row of this wave can see
 #pragma unroll
-  for (int o = 1; o < 64; o <<= 1) { const int other = __shfl_xor(wave_min_limit, o, 64); wave_min_limit = other < wave_min_limit ? other : wave_min_limit; }
+  for (int o = 1; o < 64; o <<= 1) {
+    const int other = __shfl_xor(wave_min_limit, o, 64); wave_min_limit = other < wave_min_limit ? other : wave_min_limit;
+    const int more = __shfl_xor(wave_max_limit, o, 64); wave_max_limit = more > wave_max_limit ? more : wave_max_limit;
+  }
   wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
+  wave_max_limit = __builtin_amdgcn_readfirstlane(wave_max_limit);
   // Sliding window: a row sees keys [lo, limit).  lo grows with the row, so the first row of the workgroup gives the
   // first key any row needs, and the largest lo of a wave tells which blocks need the mask at their front.
   const int lo = (p.window > 0 && limit > p.window) ? limit - p.window : 0;
@@ -222,7 +227,7 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
       const int key_base = tile * kPfTile;
 #pragma unroll 1
       for (int tb = 0; tb < 2; tb++) {
-        if (key_base + tb * 32 >= wg_limit) break;
+        if (key_base + tb * 32 >= wave_max_limit) break;      // behind everything a row of this wavefront sees (causal diagonal)
         if (key_base + tb * 32 + 32 <= wg_lo) continue;       // in front of every row's window
         f32x16 s;
 #pragma unroll
