@@ -65,6 +65,60 @@ def clock_ramp(fn, seconds=0.3, batch=20):
         torch.cuda.synchronize()
 
 
+def _hwmon(name):
+    import glob
+    hits = sorted(glob.glob(f"/sys/class/drm/card*/device/hwmon/hwmon*/{name}"))
+    return hits[0] if hits else None
+
+
+def _read_watts(path):
+    try:
+        with open(path) as f:
+            return int(f.read()) / 1e6
+    except (OSError, ValueError):
+        return None
+
+
+def socket_power(fn, seconds=2.0, batch=20):
+    """Socket power (hwmon power1_input, sampled every 50 ms by a host thread) while `fn` is queued back to back for
+    `seconds`, the first half second left out; None where the driver exposes no such file.  Says whether the timed kernel
+    runs at the part's power cap, where fewer cycles buy a lower clock instead of less time."""
+    import threading
+    src, cap = _hwmon("power1_input"), _hwmon("power1_cap")
+    if src is None or _read_watts(src) is None:
+        return None
+    samples, stop = [], threading.Event()
+    t0 = time.perf_counter()
+
+    def sampler():
+        while not stop.is_set():
+            w = _read_watts(src)
+            if w is not None and time.perf_counter() - t0 > 0.5:
+                samples.append(w)
+            time.sleep(0.05)
+    th = threading.Thread(target=sampler)
+    th.start()
+    calls = 0
+    a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(batch):
+            fn()
+        torch.cuda.synchronize()
+        calls += batch
+    e.record()
+    torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    if not samples:
+        return None
+    us = a.elapsed_time(e) * 1e3 / calls
+    watts = sum(samples) / len(samples)
+    return {"socket_w_avg": round(watts, 1), "socket_w_max": round(max(samples), 1),
+            "cap_w": _read_watts(cap) if cap else None, "seconds": seconds, "us_per_launch": round(us, 2),
+            "mj_per_launch": round(watts * us * 1e-3, 1), "source": "hwmon power1_input, 50 ms samples"}
+
+
 def profile_traffic(fname, applies=True):
     """HBM bytes per launch of the roofline kernel as the committed counter summary states them (a line
     `traffic_bytes_per_launch = N` in profiles/<fname>); None when the summary is absent or the run is not the workload it
@@ -690,6 +744,8 @@ def main():
     ap.add_argument("--q-len", type=int, default=1)
     ap.add_argument("--splits", type=int, default=0, help="KV splits per sequence (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-power-probe", action="store_true",
+                    help="decode workload: skip the two seconds of queued split-kernel launches under the socket power reading")
     ap.add_argument("--graph", action="store_true",
                     help="decode workload: replay the steps from captured HIP graphs instead of launching their kernels one by "
                          "one.  Measured slower on this part: a graph leaves no idle time between kernels, the engine clock "
@@ -811,6 +867,7 @@ def main():
     _, k_dev = timed(split_only, args.steps)
     k_avg = k_dev / args.steps * 1e6
     k_iso_avg, k_med = event_time(split_only, args.steps)
+    power = None if args.no_power_probe else socket_power(split_only)
 
     ab = algorithmic_bytes(case, heads)
     sum_l = int(case["seq_lens"].sum())
@@ -845,7 +902,8 @@ def main():
                      "kernel_us_avg": round(k_avg, 2), "kernel_us_one_launch_alone_avg": round(k_iso_avg, 2),
                      "kernel_us_one_launch_alone_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),
-                     "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)},
+                     "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                     "socket_power": power},
     }
 
     if not args.no_cpu_baseline:

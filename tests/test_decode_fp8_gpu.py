@@ -43,12 +43,17 @@ def test_decode_fp8_matches_oracle(dev, batch, heads, lo, hi, q_len, splits):
     ref_deq = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope_deq"], c["rope"], c["block_table"], c["seq_lens"],
                                 c["scale"])
     attn_close(out, ref_deq, FP8_MAX_ABS, FP8_MEAN_REL)
+    # Against the UNQUANTISED values the e4m3 rounding of the cache itself (up to 2^-4 per element) dominates; it averages
+    # out with the context length, so the 6e-2 budget holds for long contexts.  At any length the kernel may add no more
+    # than its own bf16-path error to what the format costs (the oracle over the dequantised cache against the oracle
+    # over the original values).
+    ref_full = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"],
+                                 c["scale"])
+    err_full = (out.float().cpu() - ref_full).abs().max().item()
+    err_format = (ref_deq - ref_full).abs().max().item()
+    assert err_full <= err_format + 2e-2, (err_full, err_format)
     if lo >= 4096:
-        # against the UNQUANTISED values the e4m3 rounding noise itself (2^-4 per element) dominates; it averages out
-        # with context length, and the 6e-2 budget is stated for long contexts
-        ref_full = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"],
-                                     c["scale"])
-        assert (out.float().cpu() - ref_full).abs().max().item() <= FP8_MAX_ABS
+        assert err_full <= FP8_MAX_ABS
 
 
 @pytest.mark.parametrize("num_splits", [1, 4])
