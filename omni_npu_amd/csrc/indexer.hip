@@ -7,9 +7,12 @@
 // q8 / k8 are float8_e4m3fn (OCP), 128 wide; w already carries the per-(token, head) q scale unless a
 // separate q_scale is passed.  The selection half is dsa_topk (topk.hip).
 //
-// Pure streaming kernel, no LDS: a wavefront walks blocks of 32 keys (its equal share of all blocks of the launch).  Lane (key = l % 32, half = l / 32)
-// loads bytes [64*half, 64*half + 64) of its key row straight from the paged cache and uses them as the B
-// operand of 8 MFMA 32x32x16 fp8 steps per head block (the k order inside a step is free as long as A
+// Pure streaming kernel: a wavefront walks blocks of 32 keys (its equal share of all blocks of the launch).  A block
+// (32 rows of 128 bytes and their 32 scales) travels global -> LDS in five copy instructions that bypass the registers,
+// every one covering whole 128-byte lines (a lane that loaded its own row's bytes would touch 32 lines per instruction,
+// each of them four times over), into a ring of four slots that belongs to the wavefront alone: no barrier anywhere.
+// Lane (key = l % 32, half = l / 32) then reads bytes [64*half, 64*half + 64) of its key row from the slot and uses them
+// as the B operand of 8 MFMA 32x32x16 fp8 steps per head block (the k order inside a step is free as long as A
 // uses the same one).  A = the query's 64 heads x 128, held in 32 registers.  In the accumulator layout
 // a lane owns one key and 16 of the 32 heads of a block, so the weighted ReLU sum is 32 in-lane FMAs plus
 // one exchange between the two half-waves.
@@ -18,7 +21,10 @@
 namespace mlahip {
 
 constexpr int kIdxDim = 128;
-constexpr int kIdxAhead = 6;                          // key blocks held in registers (5 requested ahead)
+constexpr int kIdxRing = 4;                           // ring slots per wavefront (3 blocks requested ahead)
+constexpr int kIdxSlotB = 32 * kIdxDim + 32 * 4;      // 4224: 32 key rows + their 32 scales
+constexpr int kIdxLdsB = 4 * kIdxRing * kIdxSlotB;    // 67584 per workgroup of four wavefronts, two workgroups per CU
+constexpr int kIdxCopies = 5;                         // copy instructions per block
 
 struct IndexerParams {
   const uint8_t* q8; int64_t q_st, q_sh;              // bytes
@@ -47,8 +53,9 @@ __device__ __forceinline__ int idx_wave_max(int v) {
 // The 32-key blocks of all query tokens, laid end to end, are dealt out to the wavefronts of the launch in equal
 // contiguous shares (to within one block), whatever the individual context lengths; a share that crosses a token
 // boundary is processed as two (or more) segments.  Every wavefront derives its share from the sequence lengths by
-// itself (two passes: total, scan); there is no LDS and no barrier in this kernel, so wavefronts are independent.
-__global__ __launch_bounds__(256, 1) void dsa_indexer_fp8_kernel(const IndexerParams p) {
+// itself (two passes: total, scan); there is no barrier in this kernel and no LDS is shared, so wavefronts are independent.
+__global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int key_l = lane & 31, half = lane >> 5;
@@ -118,83 +125,88 @@ __global__ __launch_bounds__(256, 1) void dsa_indexer_fp8_kernel(const IndexerPa
       qa[hb][2 * j + 1] = (long)(((uint64_t)v[3] << 32) | v[2]);
     }
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int h = hb * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-      float w = p.weights[(int64_t)t * p.w_st + h];
-      if (p.q_scale) w *= p.q_scale[(int64_t)t * p.qs_st + h];
-      wr[hb][r] = w;
-    }
+    for (int r = 0; r < 16; r++) wr[hb][r] = p.weights[(int64_t)t * p.w_st + hb * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
+  }
+  if (p.q_scale) {                                      // (all 32 scales asked for together, not one round trip each)
+    float qs[2][16];
+#pragma unroll
+    for (int hb = 0; hb < 2; hb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) qs[hb][r] = p.q_scale[(int64_t)t * p.qs_st + hb * 32 + 8 * (r >> 2) + 4 * half + (r & 3)];
+#pragma unroll
+    for (int hb = 0; hb < 2; hb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) wr[hb][r] *= qs[hb][r];
   }
 
-  // Key blocks are requested kIdxAhead - 1 blocks ahead of their use: a block is 4 KiB per wavefront, and only what is in
-  // flight hides the memory latency.  When pages hold a whole number of 32-key blocks the page number of a block is a
-  // scalar (one scalar load of the block table, no dependent vector load in front of the key loads).
-  const bool block_paged = (p.page_size & 31) == 0;
-  int nxt_key0 = key_begin;                             // next block to request; its page and row offset when block_paged
-  int nxt_pg = key_begin / p.page_size;
+  // Key blocks are requested kIdxRing - 1 blocks ahead of their use: a block is 4 KiB per wavefront, and only what is in
+  // flight hides the memory latency.  Pages hold a whole number of 32-key blocks (checked on the host), so the page
+  // number of a block is a scalar (one scalar load of the block table) and the block's rows are contiguous in the page.
+  // Slot layout: row r at r * 128, its 16-byte granule g at position g ^ ((r >> 1) & 7), so that the sixteen lanes of a
+  // read phase (rows of both parities, one logical granule) hit sixteen different bank groups; the scales behind the rows.
+  // Rows of the last block past the visible keys are read too (they lie inside the page) and never used.
+  const uint32_t ring = lds_addr_of(lds) + (uint32_t)wave * (kIdxRing * kIdxSlotB);
+  const char* ring_p = lds + wave * (kIdxRing * kIdxSlotB);
+  uint32_t src_off[4];                                  // copy i, lane l: row 8 i + l / 8, granule (l % 8) ^ swizzle(row)
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int r = i * 8 + (lane >> 3);
+    src_off[i] = (uint32_t)(r * (int)p.k_sr + 16 * ((lane & 7) ^ ((r >> 1) & 7)));
+  }
+  int nxt_pg = key_begin / p.page_size;                 // page and row offset of the next block to request
   int nxt_off = key_begin - nxt_pg * p.page_size;
-  auto load_block = [&](u32x4 (&kb)[4], float& ks) {
-    const int key0 = nxt_key0;
-    int key = key0 + key_l;
-    key = key < limit ? key : limit - 1;               // tail lanes re-read the last visible key (same block)
-    const uint8_t* row;
-    const float* sc;
-    if (block_paged) {
-      const int pgc = nxt_pg < p.max_blocks ? nxt_pg : p.max_blocks - 1;
-      int64_t blk = ((const __attribute__((address_space(4))) int32_t*)p.block_table)[(int64_t)b * p.bt_stride + pgc];
-      blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
-      const int off = nxt_off + (key - key0);
-      row = p.k8 + blk * p.k_sp + (int64_t)off * p.k_sr + half * 64;
-      sc = p.k_scale + blk * p.ks_sp + off;
-      nxt_off += 32;
-      if (nxt_off >= p.page_size) { nxt_off = 0; nxt_pg++; }
-    } else {
-      int pg = key / p.page_size;
-      const int off = key - pg * p.page_size;
-      pg = pg < p.max_blocks ? pg : p.max_blocks - 1;
-      int64_t blk = p.block_table[(int64_t)b * p.bt_stride + pg];
-      blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
-      row = p.k8 + blk * p.k_sp + (int64_t)off * p.k_sr + half * 64;
-      sc = p.k_scale + blk * p.ks_sp + off;
-    }
+  auto issue_block = [&](int slot) {
+    const int pgc = nxt_pg < p.max_blocks ? nxt_pg : p.max_blocks - 1;
+    int64_t blk = ((const __attribute__((address_space(4))) int32_t*)p.block_table)[(int64_t)b * p.bt_stride + pgc];
+    blk = blk < 0 ? 0 : (blk >= p.num_pages ? p.num_pages - 1 : blk);
+    const uint8_t* rows = p.k8 + blk * p.k_sp + (int64_t)nxt_off * p.k_sr;
+    const float* sc = p.k_scale + blk * p.ks_sp + nxt_off;
+    const uint32_t dst = ring + (uint32_t)slot * kIdxSlotB;
 #pragma unroll
-    for (int j = 0; j < 4; j++) kb[j] = *(const u32x4*)(row + j * 16);
-    ks = *sc;
-    nxt_key0 += 32;
+    for (int i = 0; i < 4; i++) dma16_sv(rows, src_off[i], dst + i * 1024);
+    dma4_sv_lo32(sc, (uint32_t)lane * 4, dst + 32 * kIdxDim);
+    nxt_off += 32;
+    if (nxt_off >= p.page_size) { nxt_off = 0; nxt_pg++; }
   };
-
-  u32x4 kb[kIdxAhead][4];
-  float ks[kIdxAhead];
+  const int nblk = (key_end - key_begin + 31) >> 5;
 #pragma unroll
-  for (int i = 0; i < kIdxAhead - 1; i++)
-    if (key_begin + 32 * i < key_end) load_block(kb[i], ks[i]);
-  for (int g = 0; key_begin + 32 * g < key_end; g += kIdxAhead) {
+  for (int i = 0; i < kIdxRing - 1; i++)
+    if (i < nblk) issue_block(i);
+  const int rd_row = key_l * kIdxDim, rd_swz = (key_l >> 1) & 7;
+  for (int g = 0; g < nblk; g++) {
+    const int slot = g & (kIdxRing - 1);
+    if (g + kIdxRing - 1 < nblk) issue_block((g + kIdxRing - 1) & (kIdxRing - 1));
+    // this block has landed when at most the copies of the younger blocks are outstanding (the logits stores in between
+    // count too: at worst the wait is a little longer than needed)
+    const int younger = nblk - 1 - g;
+    if (younger >= 3) MLA_WAIT_VMCNT(15);
+    else if (younger == 2) MLA_WAIT_VMCNT(10);
+    else if (younger == 1) MLA_WAIT_VMCNT(5);
+    else MLA_WAIT_VMCNT(0);
+    const char* sp = ring_p + slot * kIdxSlotB;
+    u32x4 kb[4];
 #pragma unroll
-    for (int st = 0; st < kIdxAhead; st++) {                // ring slot = step: g is a multiple of kIdxAhead
-      const int key0 = key_begin + 32 * (g + st);
-      if (key0 >= key_end) break;
-      if (key0 + 32 * (kIdxAhead - 1) < key_end)
-        load_block(kb[(st + kIdxAhead - 1) % kIdxAhead], ks[(st + kIdxAhead - 1) % kIdxAhead]);
-      f32x16 c0, c1;
+    for (int j = 0; j < 4; j++) kb[j] = *(const u32x4*)(sp + rd_row + (((4 * half + j) ^ rd_swz) << 4));
+    const float ks = *(const float*)(sp + 32 * kIdxDim + key_l * 4);
+    f32x16 c0, c1;
 #pragma unroll
-      for (int r = 0; r < 16; r++) { c0[r] = 0.f; c1[r] = 0.f; }
+    for (int r = 0; r < 16; r++) { c0[r] = 0.f; c1[r] = 0.f; }
 #pragma unroll
-      for (int kk = 0; kk < 8; kk++) {
-        const u32x4 v = kb[st][kk >> 1];
-        const long bop = (kk & 1) ? (long)(((uint64_t)v[3] << 32) | v[2]) : (long)(((uint64_t)v[1] << 32) | v[0]);
-        c0 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[0][kk], bop, c0, 0, 0, 0);
-        c1 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[1][kk], bop, c1, 0, 0, 0);
-      }
-      float acc = 0.f;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        acc = fmaf(wr[0][r], fmaxf(c0[r], 0.f), acc);
-        acc = fmaf(wr[1][r], fmaxf(c1[r], 0.f), acc);
-      }
-      acc += xor32(acc);
-      const int key = key0 + key_l;
-      if (half == 0) p.logits[(int64_t)t * p.l_st + key] = key < limit ? acc * ks[st] : -INFINITY;
+    for (int kk = 0; kk < 8; kk++) {
+      const u32x4 v = kb[kk >> 1];
+      const long bop = (kk & 1) ? (long)(((uint64_t)v[3] << 32) | v[2]) : (long)(((uint64_t)v[1] << 32) | v[0]);
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[0][kk], bop, c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(qa[1][kk], bop, c1, 0, 0, 0);
     }
+    float acc = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      acc = fmaf(wr[0][r], fmaxf(c0[r], 0.f), acc);
+      acc = fmaf(wr[1][r], fmaxf(c1[r], 0.f), acc);
+    }
+    acc += xor32(acc);
+    const int key = key_begin + 32 * g + key_l;
+    if (half == 0) p.logits[(int64_t)t * p.l_st + key] = key < limit ? acc * ks : -INFINITY;
   }
   }  // segments
 }
@@ -259,6 +271,8 @@ extern "C" int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_
                   max_seq_len >= 1,
               MLA_ERR_SHAPE, "dsa_indexer_scores_fp8: batch=%d max_q_len=%d page_size=%d max_seq_len=%d", batch, max_q_len,
               page_size, max_seq_len);
+  MLA_REQUIRE(k_row_stride >= kIdxDim && k_row_stride <= (1 << 20), MLA_ERR_SHAPE,
+              "dsa_indexer_scores_fp8: key row stride %lld bytes", (long long)k_row_stride);
   MLA_REQUIRE(q_stride_t % 16 == 0 && q_stride_h % 16 == 0 && k_page_stride % 16 == 0 && k_row_stride % 16 == 0 &&
                   (uintptr_t)q8 % 16 == 0 && (uintptr_t)k8_cache % 16 == 0,
               MLA_ERR_SHAPE, "dsa_indexer_scores_fp8: fp8 rows must be 16-byte aligned");
@@ -276,7 +290,7 @@ extern "C" int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_
   p.seq_lens = seq_lens; p.qsl = query_start_loc;
   p.batch = batch; p.max_q_len = max_q_len; p.num_heads = num_heads; p.page_size = page_size; p.num_pages = num_pages;
   p.logits = logits; p.l_st = logits_stride;
-  // two workgroups per compute unit (what the register budget allows), never more wavefronts than 32-key blocks
+  // two workgroups per compute unit (what their LDS rings allow), never more wavefronts than 32-key blocks
   static int num_cus = 0;
   if (num_cus == 0) {
     int dev = 0;
@@ -288,6 +302,8 @@ extern "C" int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_
   int64_t wgs = 2 * (int64_t)num_cus;
   if (wgs * 4 > max_blocks_total) wgs = (max_blocks_total + 3) / 4;
   if (wgs < 1) wgs = 1;
-  hipLaunchKernelGGL(dsa_indexer_fp8_kernel, dim3((unsigned)wgs), dim3(256), 0, stream, p);
+  const int rc = ensure_dynamic_lds((const void*)dsa_indexer_fp8_kernel, kIdxLdsB, "dsa_indexer_scores_fp8");
+  if (rc != MLA_OK) return rc;
+  hipLaunchKernelGGL(dsa_indexer_fp8_kernel, dim3((unsigned)wgs), dim3(256), kIdxLdsB, stream, p);
   return check_launch("dsa_indexer_fp8_kernel");
 }

@@ -101,6 +101,15 @@ __device__ __forceinline__ void dma16_v_lo32(const void* gaddr, uint32_t lds_add
                : "memory", "m0");
 }
 
+// One dword per lane by lanes 0..31 (128 bytes): lane i's dword lands at lds_addr + 4 * i.
+__device__ __forceinline__ void dma4_sv_lo32(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  uint32_t save;
+  asm volatile("s_mov_b32 %0, exec_hi\n\ts_mov_b32 exec_hi, 0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3\n\ts_mov_b32 exec_hi, %0"
+               : "=&s"(save)
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+
 // Four dwords by lanes 0..3 (the rest of the execution mask is cleared around the instruction): lane i's dword lands at
 // lds_addr + 4 * i.
 __device__ __forceinline__ void dma4_sv_lanes4(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
