@@ -34,6 +34,15 @@ def make_indexer_case(batch, lo, hi, seed, q_len=1, heads=64, page=128):
     return dict(seq_lens=lens.to(torch.int32), block_table=bt, k8=k8, k_scale=ks, q8=q8, q_scale=qs, w=w, q_len=q_len)
 
 
+def logits_tol(c, t, ref):
+    """1e-4 of the row's largest logit, plus 1e-5 of the largest magnitude that went into a logit (the same sum with |w|):
+    with one to three visible keys every logit of a row can come out near zero by cancellation between heads, and the
+    fp32 summation error does not shrink with it."""
+    abs_c = dict(c)
+    abs_c["w"] = c["w"].abs()
+    return 1e-4 * ref.abs().max().item() + 1e-5 * oracle_logits(abs_c, t).max().item() + 1e-6
+
+
 def oracle_logits(c, t):
     q_len = c["q_len"]
     b, i = divmod(t, q_len)
@@ -58,8 +67,7 @@ def test_indexer_logits(dev, batch, lo, hi, q_len):
     for tt in range(t):
         ref = oracle_logits(c, tt)
         n = ref.numel()
-        tol = 1e-4 * ref.abs().max().item() + 1e-6
-        assert (got[tt, :n] - ref).abs().max().item() <= tol
+        assert (got[tt, :n] - ref).abs().max().item() <= logits_tol(c, tt, ref)
         pad_end = min((n + 31) // 32 * 32, got.shape[1])
         assert torch.isinf(got[tt, n:pad_end]).all() and (got[tt, n:pad_end] < 0).all()
 
@@ -221,7 +229,7 @@ def test_indexer_topk_rows_random_shapes(dev, i, batch, lo, hi, q_len, k, single
     for tt in range(t):
         ref = oracle_logits(c, tt)
         n = ref.numel()
-        assert (lg[tt, :n] - ref).abs().max().item() <= 1e-4 * ref.abs().max().item() + 1e-6
+        assert (lg[tt, :n] - ref).abs().max().item() <= logits_tol(c, tt, ref)
         want = O.topk_stable(lg[tt], k, n)
         got = [v for v in idx_c[tt].tolist() if v >= 0]
         assert got == sorted(v for v in want.tolist() if v >= 0), (tt, n, k)
