@@ -110,9 +110,15 @@ __device__ unsigned long long* g_trace;                     // [workgroup][wave]
 #define TR_PRO(k)
 #endif
 
-template <bool kSparse, bool kWindow>
+// kRG = groups of 32 query rows that can hold rows at all (4: any launch; 1 or 2: launches with at most 32 / 64 query rows
+// per request, e.g. the 16 heads a tensor-parallel rank of eight owns).  With few rows the 128-row schedule spends the same
+// MFMAs, LDS reads and watts on rows that do not exist, so the small forms leave them out: only the wavefronts that own
+// rows run the S phase and the softmax, P.V covers kRG row groups, and the copies move to wavefronts 4..7, which have
+// nothing else to do in the S phase.  The kernel is then bound by the cache stream alone.
+template <bool kSparse, bool kWindow, int kRG = 4>
 __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p) {
   static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
+  static_assert(kRG == 1 || kRG == 2 || kRG == 4, "row groups");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 #ifdef MLA_V3_TRACE
   uint64_t tr_start;
@@ -262,6 +268,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     qlen = qlen < mq ? qlen : mq;
   }
   const int rows = qlen * p.num_heads;
+  const bool has_rows = kRG == 4 || wave * 16 < rows;         // (small forms: one group of rows, grp = 0)
 
   // this lane's query row for QK / softmax; the four lanes l16 + 16*g share it
   const int rloc = wave * 16 + l16;                           // row inside the group of 128
@@ -274,6 +281,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     limit = limit < 0 ? 0 : limit;
     if (g == 0) *(int*)(lds + kLimitOff + rloc * 4) = limit;  // read back by the blocks that have to mask (the last ones)
     *(float*)(lds + kSeenOff + threadIdx.x * 4) = -INFINITY;
+    if constexpr (kRG < 4) {                                  // wavefronts without rows never write their restart flags
+      if (threadIdx.x < 16) *(int*)(lds + kFlagOff + threadIdx.x * 4) = 0;
+    }
     // the two per-lane offsets of the K-fragment reads live in LDS and are fetched at the start of every QK phase (one
     // read instead of two registers held through the P.V phase, where registers are short)
     if (wave == 0) {
@@ -301,15 +311,16 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   // The per-lane offsets are worked out from the hardware lane number at every use (a handful of vector ALU
   // instructions per block, in the phase where that unit idles) instead of occupying registers through the loop.
   const uint32_t n_sr2 = (uint32_t)p.nope_sr * 2u, r_sr2 = (uint32_t)p.rope_sr * 2u;       // row strides in bytes
-  const bool copier = wave < kCopyWaves;
-  const int swz_nw = swz_nope((wave * 8) & 15), swz_rw = swz_rope((wave * 8) & 15);        // scalars
+  const bool copier = kRG == 4 ? wave < kCopyWaves : wave >= 8 - kCopyWaves;
+  const int cw = kRG == 4 ? wave : (wave & 3);                // the copying wavefront's number among the four
+  const int swz_nw = swz_nope((cw * 8) & 15), swz_rw = swz_rope((cw * 8) & 15);            // scalars
   // full blocks of the paged cache: the wave's row offsets ride in the per-lane offset (32 rows stay below 2^31 bytes,
   // checked where the mode is chosen), so a copy is one vector instruction, one scalar add into M0 and the load
   const bool full_ok = n_sr2 <= (1u << 25) && r_sr2 <= (1u << 25);
   const uint32_t dma_off = (uint32_t)((lane ^ swz_nw) << 4);
   uint32_t s_rowoff[8];
 #pragma unroll
-  for (int k = 0; k < 8; k++) s_rowoff[k] = (uint32_t)(wave * 8 + k) * n_sr2;
+  for (int k = 0; k < 8; k++) s_rowoff[k] = (uint32_t)(cw * 8 + k) * n_sr2;
 
   ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (kSparse ? 0 : (int64_t)b * p.bt_stride);
   const int64_t max_row = p.num_pages * p.page_size - 1;
@@ -331,10 +342,10 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   auto ids_dma = [&](int blk_x) {
     if constexpr (kSparse) {
       if (copier) {
-        int tok = blk_x * kBlk + wave * 8 + (lane_now() & 7);
+        int tok = blk_x * kBlk + cw * 8 + (lane_now() & 7);
         tok = tok < L ? tok : L - 1;
         tok = tok < 0 ? 0 : tok;
-        dma4_sv_lanes8(p.sparse_rows + (int64_t)b * p.sparse_stride, (uint32_t)tok * 4u, lds0 + kIdsOff + (blk_x & 3) * 128 + wave * 32);
+        dma4_sv_lanes8(p.sparse_rows + (int64_t)b * p.sparse_stride, (uint32_t)tok * 4u, lds0 + kIdsOff + (blk_x & 3) * 128 + cw * 32);
       }
     }
   };
@@ -342,7 +353,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     if constexpr (kSparse) {
       if (copier) {
         const int ln = lane_now();
-        const char* slot = lds + kIdsOff + (blk_x & 3) * 128 + wave * 32;
+        const char* slot = lds + kIdsOff + (blk_x & 3) * 128 + cw * 32;
         const int32_t mine = *(const int32_t*)(slot + (ln & 7) * 4);
         ids_rope = *(const int32_t*)(slot + ((ln >> 3) & 7) * 4);
 #pragma unroll
@@ -422,11 +433,11 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
 
     if (k < 8) {
-      const int r = wave * 8 + k;
+      const int r = cw * 8 + k;
       if constexpr (kFull) {
         uint32_t d = dma_off;
         asm volatile("" : "+v"(d));                           // (opaque: the eight offsets are not precomputed and spilled)
-        dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + wave * 8192, k * 1024);
+        dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + cw * 8192, k * 1024);
       } else {
         const uint32_t off = (uint32_t)((lane_now() ^ swz_nw ^ swz_nope(k)) << 4);
         const int re = r < c.last ? r : c.last;
@@ -436,13 +447,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     } else {
       // the wave's eight rope rows, 128 bytes each: one instruction
       if constexpr (kSparse) {
-        dma16_v(c.rp + clampi(ids_rope) * r_sr2 + rope_lane_off(), c.rbuf + wave * 1024);
+        dma16_v(c.rp + clampi(ids_rope) * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
       } else if constexpr (kFull) {
-        dma16_sv(c.rp, (uint32_t)(wave * 8 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + wave * 1024);
+        dma16_sv(c.rp, (uint32_t)(cw * 8 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
       } else {
-        const int r = wave * 8 + rope_lane_row();
+        const int r = cw * 8 + rope_lane_row();
         const int re = r < c.last ? r : c.last;
-        dma16_sv(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + wave * 1024);
+        dma16_sv(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
       }
     }
   };
@@ -480,7 +491,10 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   // every wave has its query in registers (one barrier).
   TR_PRO(0);
   bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
-  {
+  if (!has_rows) {
+#pragma unroll
+    for (int kk = 0; kk < 18; kk++) qf[kk] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  } else {
     // Contraction step kk of the latent part covers the 16-byte granules 16*(kk%4) + 4g' + kk/4, g' = 0..3, and lane group
     // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
     // in one aligned 32-byte piece of a row, or the LDS serves the instruction at half rate (measured: 126 against 227
@@ -665,7 +679,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   // O^T += V^T P^T for block `blk` (this wave's 64 output columns, all four row groups; kPv) with the softmax of the next
   // block's scores sc riding along (kSm).  Per k-block the two V^T fragments are held while the four P^T fragments go by
   // (two registers quads, each refilled as soon as its MFMAs are issued), every fragment feeding two MFMAs.
-  auto pv_softmax = [&](int blk, auto with_pv, auto with_sm, float (&sc)[8], Sm& st) {
+  // (small forms: sm_on tells whether this wavefront owns rows; one call site serves both kinds of wavefront, so that the
+  // accumulators stay in the same registers - a copy the compiler puts behind an MFMA it cannot see would read them early)
+  auto pv_softmax = [&](int blk, auto with_pv, auto with_sm, float (&sc)[8], Sm& st, bool sm_on) {
     constexpr bool kPv = decltype(with_pv)::value, kSm = decltype(with_sm)::value;
     const uint32_t vb = lds0 + (blk & 3) * kNopeBufB;
     const uint32_t a0 = vb + vbase[0], a1 = vb + vbase[1];    // ^ 64 for the second 32 columns, + 16384 for the second k-block
@@ -685,6 +701,30 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_f32_32x32x16_bf16 %0, %2, %4, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %3, %4, %1" \
                    : "+a"(acc[0][rg]), "+a"(acc[1][rg]) : "v"(va0), "v"(va1), "v"(pr), "i"(cnt));                      \
     } while (0)
+    // (small forms only, where the matrix pipe has time to spare: the block's last MFMAs have written their accumulators
+    // before anything the compiler may place behind this statement reads them)
+#define PV_SETTLE(rg) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[0][rg]), "+a"(acc[1][rg]))
+    if constexpr (kRG == 1) {
+      // one row group: two MFMAs per k-block, the softmax steps in the shadow of the LDS reads
+      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); }
+      if constexpr (kSm) { if (sm_on) { sm_head(sc, st); SM_EXP2(0, 1); SM_EXP2(2, 3); } }
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); }
+      if constexpr (kSm) { if (sm_on) { SM_EXP2(4, 5); SM_EXP2(6, 7); sm_pm(st); } }
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 0); PV_SETTLE(0); }
+      if constexpr (kSm) { if (sm_on) { sm_sum_lo(sc, st); sm_sum_hi(sc, st); } }
+    } else if constexpr (kRG == 2) {
+      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 1, 0); }
+      if constexpr (kSm) { if (sm_on) { sm_head(sc, st); SM_EXP2(0, 1); } }
+      if constexpr (kPv) PV_MFMA2(0, pr0, 1);
+      if constexpr (kSm) { if (sm_on) SM_EXP2(2, 3); }
+      if constexpr (kPv) { PV_MFMA2(1, pr1, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); PV_PREAD(pr1, 1, 1); }
+      if constexpr (kSm) { if (sm_on) { SM_EXP2(4, 5); SM_EXP2(6, 7); sm_pm(st); } }
+      if constexpr (kPv) PV_MFMA2(0, pr0, 1);
+      if constexpr (kSm) { if (sm_on) sm_sum_lo(sc, st); }
+      if constexpr (kPv) { PV_MFMA2(1, pr1, 0); PV_SETTLE(0); PV_SETTLE(1); }
+      if constexpr (kSm) { if (sm_on) sm_sum_hi(sc, st); }
+    } else {
+    (void)sm_on;
     if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 1, 0); }
     if constexpr (kSm) sm_head(sc, st);
     if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_PREAD(pr0, 2, 0); }
@@ -700,6 +740,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     if constexpr (kPv) { PV_MFMA2(1, pr1, 1); PV_PREAD(pr1, 3, 1); }
     if constexpr (kSm) sm_sum_hi(sc, st);
     if constexpr (kPv) { PV_MFMA2(2, pr0, 1); PV_MFMA2(3, pr1, 0); }
+    }
+#undef PV_SETTLE
 #undef PV_VREAD
 #undef PV_PREAD
 #undef PV_MFMA2
@@ -763,6 +805,16 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     for (int r = 0; r < 8; r++) sc[r] = s[r >> 2][r & 3];
   };
 
+  if constexpr (kRG < 4) {
+    // a wavefront without rows publishes no probabilities: its slots of both P buffers hold zeros for the whole segment
+    // (row groups are read whole by the P.V phase; nobody else writes these slots)
+    if (!has_rows) {
+      const u32x2 z = {0u, 0u};
+      const uint32_t pw = lds0 + p_w_off_now();
+      asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %1 offset:1024\n\tds_write_b64 %0, %1 offset:8192\n\tds_write_b64 %0, %1 offset:9216"
+                   :: "v"(pw), "v"(z) : "memory");
+    }
+  }
   bool restart = false;
   int restarts_left = 4;         // every restart raises a reference by more than 2^100: fp32 has room for three
   do {
@@ -795,6 +847,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       TR_PRO(2);
       f32x4 s[2];
       Sm st;
+      if (has_rows) {
       qk_block(blk_begin, s, std::integral_constant<int, 0>{}, 0);
       if (m_ref == -INFINITY) {
         // the first block fixes the reference: the row's largest score over all 32 keys (visible or not: any finite
@@ -807,8 +860,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       }
       float sc[8];
       unpack_scores(s, sc);
-      pv_softmax(blk_begin, std::false_type{}, std::true_type{}, sc, st);
+      pv_softmax(blk_begin, std::false_type{}, std::true_type{}, sc, st, true);
       softmax_finish(blk_begin, sc, st);
+      }
     }
     // Everything the loop keeps in registers is touched here: a value that was parked in scratch during the prologue is
     // brought back (and waited for) now, not at its first use inside the loop.
@@ -834,6 +888,24 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
 #elif defined(ABL_NO_COPY)
       if (true) { qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0); s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0]; }
 #else
+      if constexpr (kRG < 4) {
+        // small forms: wavefronts 4..7 only copy, the wavefronts that own rows only compute
+        if (copier) {
+          if (i + kLead < nb) {
+            ids_dma(blk + kLead + 1);
+            IssueCtx ic = issue_begin(blk + kLead);
+            if (kSparse || !full_ok || L - 1 - (blk + kLead) * kBlk < kBlk - 1) {
+#pragma unroll
+              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::false_type{});
+            } else {
+#pragma unroll
+              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::true_type{});
+            }
+          }
+        } else if (has_rows) {
+          qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
+        }
+      } else
       // (the wavefronts that copy nothing take the variant without copies: no branch around each copy, no page arithmetic)
       if (i + kLead >= nb || !copier) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
 #endif
@@ -848,17 +920,17 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
       st.pw[0] = st.pw[1] = st.pw[2] = st.pw[3] = 0;
 #elif defined(ABL_NO_PV)
-      pv_softmax(blk, std::false_type{}, std::true_type{}, sc, st);
+      pv_softmax(blk, std::false_type{}, std::true_type{}, sc, st, true);
 #elif defined(ABL_NO_SOFTMAX)
       st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
       st.pw[0] = st.pw[1] = st.pw[2] = st.pw[3] = 0;
-      pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st);
+      pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st, true);
 #else
-      pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st);
+      pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st, has_rows);
 #endif
       TR_ADD(3);
 #ifndef ABL_NO_FINISH
-      softmax_finish(blk + 1, sc, st);
+      if (has_rows) softmax_finish(blk + 1, sc, st);
 #else
       l_run += st.psum + (float)st.pw[0];
 #endif
@@ -872,7 +944,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       MLA_WAIT_VMCNT(0);
       lds_barrier();
       if (restarts_left > 0 && flags_ask_restart(flags_read(blk))) { restart = true; restarts_left--; }
-      else { float sc[8]; Sm st; pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st); }
+      else { float sc[8]; Sm st; pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st, true); }
     }
   } while (restart);
 
@@ -939,7 +1011,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   char* stage = lds + wave * 16384;
   _Float16* o_part_c = cold()->o_part;
 #pragma unroll
-  for (int rg = 0; rg < 4; rg++) {
+  for (int rg = 0; rg < kRG; rg++) {
     const int srow = rg * 32 + e_h32;
 #pragma unroll
     for (int db = 0; db < 2; db++)
@@ -956,7 +1028,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   // read back: 16 lanes read one row (128 B), four rows per instruction
 #pragma unroll 4
-  for (int it = 0; it < 32; it++) {
+  for (int it = 0; it < 8 * kRG; it++) {
     const int srow = it * 4 + e_g;
     const u32x2 v = *(const u32x2*)(stage + srow * 128 + ((e_l16 ^ ((srow >> 1) & 15)) << 3));
     if (grp * 128 + srow < r_max)
@@ -981,12 +1053,23 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
 
 }  // namespace v3
 
-int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream) {
-  const void* kernel = sparse ? (const void*)v3::mla_decode_v3_kernel<true, false>
-                              : (p.win_skip ? (const void*)v3::mla_decode_v3_kernel<false, true>
-                                            : (const void*)v3::mla_decode_v3_kernel<false, false>);
-  const int rc = ensure_dynamic_lds(kernel, v3::kLdsB, "mla_decode_v3_kernel");
+template <bool kSparse, bool kWindow, int kRG>
+static int launch_form(const DecodeParams& p, dim3 grid, hipStream_t stream) {
+  const int rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<kSparse, kWindow, kRG>, v3::kLdsB, "mla_decode_v3_kernel");
   if (rc != MLA_OK) return rc;
+  hipLaunchKernelGGL((v3::mla_decode_v3_kernel<kSparse, kWindow, kRG>), grid, dim3(512), v3::kLdsB, stream, p);
+  return check_launch("mla_decode_v3_kernel");
+}
+template <bool kSparse, bool kWindow>
+static int launch_rows(const DecodeParams& p, dim3 grid, hipStream_t stream) {
+  // requests with at most 32 / 64 query rows (tokens x heads) take the forms that leave the missing rows out
+  const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
+  if (r_max <= 32) return launch_form<kSparse, kWindow, 1>(p, grid, stream);
+  if (r_max <= 64) return launch_form<kSparse, kWindow, 2>(p, grid, stream);
+  return launch_form<kSparse, kWindow, 4>(p, grid, stream);
+}
+
+int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream) {
 #ifdef MLA_V3_TRACE
   {
     const char* e = getenv("MLA_V3_TRACE_PTR");
@@ -994,10 +1077,9 @@ int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t 
     hipMemcpyToSymbol(HIP_SYMBOL(v3::g_trace), &ptr, sizeof(ptr));
   }
 #endif
-  if (sparse) hipLaunchKernelGGL((v3::mla_decode_v3_kernel<true, false>), grid, dim3(512), v3::kLdsB, stream, p);
-  else if (p.win_skip) hipLaunchKernelGGL((v3::mla_decode_v3_kernel<false, true>), grid, dim3(512), v3::kLdsB, stream, p);
-  else hipLaunchKernelGGL((v3::mla_decode_v3_kernel<false, false>), grid, dim3(512), v3::kLdsB, stream, p);
-  return check_launch("mla_decode_v3_kernel");
+  if (sparse) return launch_rows<true, false>(p, grid, stream);
+  if (p.win_skip) return launch_rows<false, true>(p, grid, stream);
+  return launch_rows<false, false>(p, grid, stream);
 }
 
 }  // namespace mlahip

@@ -154,13 +154,15 @@ def _plant(case, b, pos, head, gain):
     case["nope"][page, pos % 128] = (gain * case["q_nope"][b * case["q_len"], head].float()).bfloat16()
 
 
+@pytest.mark.parametrize("heads", [128, 16, 48])
 @pytest.mark.parametrize("num_splits", [1, 4])
-def test_decode_scores_that_outgrow_the_first_block(dev, num_splits):
+def test_decode_scores_that_outgrow_the_first_block(dev, num_splits, heads):
     """The kernel fixes each row's softmax reference at its first block and restarts a segment when a later score exceeds
     it by more than 2^100: keys planted late in the sequences with scores ~110 and ~220 (natural units) above the
     rest exercise one and two restarts, a planted key in the very first block exercises a reference that is already
-    the maximum, and a moderately dominant key (weight ~0.5) exercises the correction of the dominant probability."""
-    case = O.make_decode_case(4, 128, 1500, 2500, seed=21)
+    the maximum, and a moderately dominant key (weight ~0.5) exercises the correction of the dominant probability.
+    16 and 48 heads take the kernel forms for at most 32 / 64 query rows, where some wavefronts own no rows."""
+    case = O.make_decode_case(4, heads, 1500, 2500, seed=21)
     lens = case["seq_lens"].tolist()
     _plant(case, 0, lens[0] - 40, 3, 3.0)                      # one restart, late in the last chunk
     _plant(case, 1, 700, 5, 3.0)
