@@ -99,8 +99,12 @@ __device__ unsigned long long* g_trace;                     // [workgroup][wave]
 #define TR_PRO(k)
 #endif
 
-template <bool kWindow>
+// kRG = groups of 32 query rows that can hold rows at all (4: any launch; 1 or 2: at most 32 / 64 query rows per request, as
+// in the bf16 kernel): only the wavefronts that own rows run the S phase and the softmax, P.V covers kRG row groups, the
+// copies move to wavefronts 4..7; all 512 threads still turn the raw block into its bf16 tile.
+template <bool kWindow, int kRG = 4>
 __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodeParams p) {
+  static_assert(kRG == 1 || kRG == 2 || kRG == 4, "row groups");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 #ifdef MLA_V3_TRACE
   uint64_t tr_start;
@@ -250,6 +254,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     qlen = qlen < mq ? qlen : mq;
   }
   const int rows = qlen * p.num_heads;
+  const bool has_rows = kRG == 4 || wave * 16 < rows;         // (small forms: one group of rows, grp = 0)
 
   // this lane's query row for QK / softmax; the four lanes l16 + 16*g share it
   const int rloc = wave * 16 + l16;                           // row inside the group of 128
@@ -262,6 +267,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     limit = limit < 0 ? 0 : limit;
     if (g == 0) *(int*)(lds + kLimitOff + rloc * 4) = limit;  // read back by the blocks that have to mask (the last ones)
     if (g == 0) *(float*)(lds + kSeenOff + rloc * 4) = -INFINITY;
+    if constexpr (kRG < 4) {                                  // wavefronts without rows never write their restart flags
+      if (threadIdx.x < 16) *(int*)(lds + kFlagOff + threadIdx.x * 4) = 0;
+    }
     // the two per-lane offsets of the K-fragment reads live in LDS and are fetched at the start of every QK phase (one
     // read instead of two registers held through the P.V phase, where registers are short)
     if (wave == 0) {
@@ -286,7 +294,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   //   1 x the eight rows' 16 scale bytes (lanes 0..7)                                           -> behind the 32 rows
   //   1 x the eight rows' 128 rope bytes (lane i: row i/8, granule i%8, swizzled by the lane)   -> rope buffer
   // Rows past the end of the sequence re-read its last row (their scores are masked; their bytes must be finite).
-  const bool copier = wave < kCopyWaves;
+  const bool copier = kRG == 4 ? wave < kCopyWaves : wave >= 8 - kCopyWaves;
+  const int cw = kRG == 4 ? wave : (wave & 3);                // the copying wavefront's number among the four
   // The hardware lane number behind an opaque (and volatile) statement: what is derived from it inside the loop is
   // computed inside the loop.  Left alone the compiler hoists every loop-invariant LDS address out of the block loop, a
   // dozen registers of them, and then spills them - and a scratch reload waits for every copy in flight.
@@ -295,7 +304,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     asm volatile("" : "+v"(ln));
     return ln;
   };
-  const int swz_rw = swz_rope((wave * 8) & 15);                // scalar
+  const int swz_rw = swz_rope((cw * 8) & 15);                  // scalar
   ConstI32Ptr bt = (ConstI32Ptr)(p.block_table) + (int64_t)b * p.bt_stride;
   auto load_page = [&](int page) -> int64_t {
     page = page < p.max_blocks ? page : p.max_blocks - 1;
@@ -331,14 +340,14 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     auto row_of = [&](int r) { return r < last ? r : last; };  // (a full block: last >= 31, nothing is clamped)
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-      const int r = wave * 8 + 2 * k + (ln >> 5);
-      dma16_sv(src, (uint32_t)(row_of(r) * kFp8RowBytes + (ln & 31) * 16), raw + (wave * 8 + 2 * k) * 512);
+      const int r = cw * 8 + 2 * k + (ln >> 5);
+      dma16_sv(src, (uint32_t)(row_of(r) * kFp8RowBytes + (ln & 31) * 16), raw + (cw * 8 + 2 * k) * 512);
     }
-    dma16_sv_lanes8(src, (uint32_t)(row_of(wave * 8 + (ln & 7)) * kFp8RowBytes + kFp8ScaleOffB), raw + kRawScaleOff + wave * 128);
+    dma16_sv_lanes8(src, (uint32_t)(row_of(cw * 8 + (ln & 7)) * kFp8RowBytes + kFp8ScaleOffB), raw + kRawScaleOff + cw * 128);
     {
       const int t = (ln >> 3) & 7;
       const uint32_t off = (uint32_t)(((ln & 7) ^ swz_rw ^ ((t & 1) << 2) ^ (t & 2) ^ (t >> 2)) << 4);   // swz_rope(t) = (t0 << 2) | (t1 << 1) | t2
-      dma16_sv(src, (uint32_t)(row_of(wave * 8 + t) * kFp8RowBytes + kFp8RopeOffB) + off, rbuf + wave * 1024);
+      dma16_sv(src, (uint32_t)(row_of(cw * 8 + t) * kFp8RowBytes + kFp8RopeOffB) + off, rbuf + cw * 1024);
     }
   };
   // raw block `blk` -> bf16 tile of that block, all 512 threads: thread (row r = t / 16, c = t % 16) turns the 32 e4m3 values
@@ -379,7 +388,10 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   // every wave has its query in registers (one barrier).
   TR_PRO(0);
   bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
-  {
+  if (!has_rows) {
+#pragma unroll
+    for (int kk = 0; kk < 18; kk++) qf[kk] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+  } else {
     // Contraction step kk of the latent part covers the 16-byte granules 16*(kk%4) + 4g' + kk/4, g' = 0..3, and lane group
     // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
     // in one aligned 32-byte piece of a row, or the LDS serves the instruction at half rate (measured: 126 against 227
@@ -534,7 +546,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   // O^T += V^T P^T for block `blk` (this wave's 64 output columns, all four row groups; kPv) with the softmax of the next
   // block's scores sc riding along (kSm).  Per k-block the two V^T fragments are held while the four P^T fragments go by
   // (two registers quads, each refilled as soon as its MFMAs are issued), every fragment feeding two MFMAs.
-  auto pv_softmax = [&](int blk, auto with_pv, auto with_sm, float (&sc)[8], Sm& st) {
+  // (small forms: sm_on tells whether this wavefront owns rows; one call site serves both kinds of wavefront, so that the
+  // accumulators stay in the same registers - a copy the compiler puts behind an MFMA it cannot see would read them early)
+  auto pv_softmax = [&](int blk, auto with_pv, auto with_sm, float (&sc)[8], Sm& st, bool sm_on) {
     constexpr bool kPv = decltype(with_pv)::value, kSm = decltype(with_sm)::value;
     const uint32_t vb = lds0 + rope_buf_of(blk) * kNopeBufB;
     const uint32_t a0 = vb + vbase[0], a1 = vb + vbase[1];    // ^ 64 for the second 32 columns, + 16384 for the second k-block
@@ -554,6 +568,29 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_f32_32x32x16_bf16 %0, %2, %4, %0\n\tv_mfma_f32_32x32x16_bf16 %1, %3, %4, %1" \
                    : "+a"(acc[0][rg]), "+a"(acc[1][rg]) : "v"(va0), "v"(va1), "v"(pr), "i"(cnt));                      \
     } while (0)
+    // (small forms only, where the matrix pipe has time to spare: the block's last MFMAs have written their accumulators
+    // before anything the compiler may place behind this statement reads them)
+#define PV_SETTLE(rg) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[0][rg]), "+a"(acc[1][rg]))
+    if constexpr (kRG == 1) {
+      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); }
+      if constexpr (kSm) { if (sm_on) { sm_head(sc, st); SM_EXP2(0, 1); SM_EXP2(2, 3); } }
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); }
+      if constexpr (kSm) { if (sm_on) { SM_EXP2(4, 5); SM_EXP2(6, 7); sm_pm(st); } }
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 0); PV_SETTLE(0); }
+      if constexpr (kSm) { if (sm_on) { sm_sum_lo(sc, st); sm_sum_hi(sc, st); } }
+    } else if constexpr (kRG == 2) {
+      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 1, 0); }
+      if constexpr (kSm) { if (sm_on) { sm_head(sc, st); SM_EXP2(0, 1); } }
+      if constexpr (kPv) PV_MFMA2(0, pr0, 1);
+      if constexpr (kSm) { if (sm_on) SM_EXP2(2, 3); }
+      if constexpr (kPv) { PV_MFMA2(1, pr1, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); PV_PREAD(pr1, 1, 1); }
+      if constexpr (kSm) { if (sm_on) { SM_EXP2(4, 5); SM_EXP2(6, 7); sm_pm(st); } }
+      if constexpr (kPv) PV_MFMA2(0, pr0, 1);
+      if constexpr (kSm) { if (sm_on) sm_sum_lo(sc, st); }
+      if constexpr (kPv) { PV_MFMA2(1, pr1, 0); PV_SETTLE(0); PV_SETTLE(1); }
+      if constexpr (kSm) { if (sm_on) sm_sum_hi(sc, st); }
+    } else {
+    (void)sm_on;
     if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 1, 0); }
     if constexpr (kSm) sm_head(sc, st);
     if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_PREAD(pr0, 2, 0); }
@@ -569,6 +606,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     if constexpr (kPv) { PV_MFMA2(1, pr1, 1); PV_PREAD(pr1, 3, 1); }
     if constexpr (kSm) sm_sum_hi(sc, st);
     if constexpr (kPv) { PV_MFMA2(2, pr0, 1); PV_MFMA2(3, pr1, 0); }
+    }
+#undef PV_SETTLE
 #undef PV_VREAD
 #undef PV_PREAD
 #undef PV_MFMA2
@@ -622,6 +661,15 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     for (int r = 0; r < 8; r++) sc[r] = s[r >> 2][r & 3];
   };
 
+  if constexpr (kRG < 4) {
+    // a wavefront without rows publishes no probabilities: its slots of both P buffers hold zeros for the whole segment
+    if (!has_rows) {
+      const u32x2 z = {0u, 0u};
+      const uint32_t pw = lds0 + p_w_off_now();
+      asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %1 offset:1024\n\tds_write_b64 %0, %1 offset:8192\n\tds_write_b64 %0, %1 offset:9216"
+                   :: "v"(pw), "v"(z) : "memory");
+    }
+  }
   bool restart = false;
   int restarts_left = 4;         // every restart raises a reference by more than 2^100: fp32 has room for three
   do {
@@ -654,6 +702,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       TR_PRO(2);
       f32x4 s[2];
       Sm st;
+      if (has_rows) {
       qk_block(blk_begin, s);
       if (m_ref == -INFINITY) {
         // the first block fixes the reference: the row's largest score over all 32 keys (visible or not: any finite
@@ -666,8 +715,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       }
       float sc[8];
       unpack_scores(s, sc);
-      pv_softmax(blk_begin, std::false_type{}, std::true_type{}, sc, st);
+      pv_softmax(blk_begin, std::false_type{}, std::true_type{}, sc, st, true);
       softmax_finish(blk_begin, sc, st);
+      }
     }
     // Everything the loop keeps in registers is touched here: a value that was parked in scratch during the prologue is
     // brought back (and waited for) now, not at its first use inside the loop.
@@ -694,15 +744,15 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       if (copier && i + 2 < nb) dequant_block(blk + 2);
       if (i + 3 < nb) issue_block(blk + 3);
       f32x4 s[2];
-      qk_block(blk + 1, s);
+      if (has_rows) qk_block(blk + 1, s);
       TR_ADD(2);
       if (restarts_left > 0 && flags_ask_restart(fl)) { restart = true; restarts_left--; break; }
       Sm st;
       float sc[8];
       unpack_scores(s, sc);
-      pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st);
+      pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st, has_rows);
       TR_ADD(3);
-      softmax_finish(blk + 1, sc, st);
+      if (has_rows) softmax_finish(blk + 1, sc, st);
       if (!copier && i + 2 < nb) dequant_block(blk + 2);
       TR_ADD(4);
 #ifdef MLA_V3_TRACE
@@ -714,7 +764,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       MLA_WAIT_VMCNT(0);
       lds_barrier();
       if (restarts_left > 0 && flags_ask_restart(flags_read(blk))) { restart = true; restarts_left--; }
-      else { float sc[8]; Sm st; pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st); }
+      else { float sc[8]; Sm st; pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st, true); }
     }
   } while (restart);
 
@@ -751,7 +801,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   char* stage = lds + wave * 16384;
   _Float16* o_part_c = cold()->o_part;
 #pragma unroll
-  for (int rg = 0; rg < 4; rg++) {
+  for (int rg = 0; rg < kRG; rg++) {
     const int srow = rg * 32 + e_h32;
 #pragma unroll
     for (int db = 0; db < 2; db++)
@@ -768,7 +818,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   // read back: 16 lanes read one row (128 B), four rows per instruction
 #pragma unroll 4
-  for (int it = 0; it < 32; it++) {
+  for (int it = 0; it < 8 * kRG; it++) {
     const int srow = it * 4 + e_g;
     const u32x2 v = *(const u32x2*)(stage + srow * 128 + ((e_l16 ^ ((srow >> 1) & 15)) << 3));
     if (grp * 128 + srow < r_max)
@@ -793,10 +843,23 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
 
 }  // namespace f8v3
 
-int launch_decode_v3_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
-  const void* kernel = p.win_skip ? (const void*)f8v3::mla_decode_v3_fp8_kernel<true> : (const void*)f8v3::mla_decode_v3_fp8_kernel<false>;
-  const int rc = ensure_dynamic_lds(kernel, f8v3::kLdsB, "mla_decode_v3_fp8_kernel");
+template <bool kWindow, int kRG>
+static int launch_form_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
+  const int rc = ensure_dynamic_lds((const void*)f8v3::mla_decode_v3_fp8_kernel<kWindow, kRG>, f8v3::kLdsB, "mla_decode_v3_fp8_kernel");
   if (rc != MLA_OK) return rc;
+  hipLaunchKernelGGL((f8v3::mla_decode_v3_fp8_kernel<kWindow, kRG>), grid, dim3(512), f8v3::kLdsB, stream, p);
+  return check_launch("mla_decode_v3_fp8_kernel");
+}
+template <bool kWindow>
+static int launch_rows_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
+  // requests with at most 32 / 64 query rows (tokens x heads) take the forms that leave the missing rows out
+  const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
+  if (r_max <= 32) return launch_form_fp8<kWindow, 1>(p, grid, stream);
+  if (r_max <= 64) return launch_form_fp8<kWindow, 2>(p, grid, stream);
+  return launch_form_fp8<kWindow, 4>(p, grid, stream);
+}
+
+int launch_decode_v3_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
 #ifdef MLA_V3_TRACE
   {
     const char* e = getenv("MLA_V3_TRACE_PTR");
@@ -804,9 +867,8 @@ int launch_decode_v3_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
     hipMemcpyToSymbol(HIP_SYMBOL(f8v3::g_trace), &ptr, sizeof(ptr));
   }
 #endif
-  if (p.win_skip) hipLaunchKernelGGL(f8v3::mla_decode_v3_fp8_kernel<true>, grid, dim3(512), f8v3::kLdsB, stream, p);
-  else hipLaunchKernelGGL(f8v3::mla_decode_v3_fp8_kernel<false>, grid, dim3(512), f8v3::kLdsB, stream, p);
-  return check_launch("mla_decode_v3_fp8_kernel");
+  if (p.win_skip) return launch_rows_fp8<true>(p, grid, stream);
+  return launch_rows_fp8<false>(p, grid, stream);
 }
 
 }  // namespace mlahip
