@@ -485,7 +485,7 @@ def bench_fp8(K, dev, args):
         "config": {"workload": "configs[4]: fp8 cache, high-batch MTP decode", "batch": B, "heads": N, "q_len": QL,
                    "seq_lens": "uniform[16384,32768]", "sum_seq_len": sum_l, "kv_splits": splits, "seed": args.seed},
         "step_us": {"hip_graph_replay": round(t_graph, 1), "eager_launches": round(t_eager, 1)},
-        "roofline": {"kernel": "mla_decode_v3_fp8_kernel<false>", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
+        "roofline": {"kernel": "mla_decode_v3_fp8_kernel<false, 4>", "bound": "mfma", "achieved": round(flops / (best * 1e-6) / 1e12, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": traffic, "traffic_source": traffic_src,
@@ -721,7 +721,7 @@ def bench_window(K, dev, args):
         "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "static sink tokens + sliding window decode (plan + split + merge, graph replay)", "batch": B,
                    "heads": N, "sink_len": sink, "window": win, "visible_keys": visible, "seed": args.seed},
-        "roofline": {"kernel": "mla_window_plan_kernel + mla_decode_v3_kernel<false, true> + merge (whole step)", "bound": "hbm",
+        "roofline": {"kernel": "mla_window_plan_kernel + mla_decode_v3_kernel<false, true, 4> + merge (whole step)", "bound": "hbm",
                      "achieved": round(alg_bytes / t_step / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(alg_bytes / t_step / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": traffic, "traffic_source": traffic_src, "algorithmic_bytes": alg_bytes},
@@ -876,10 +876,12 @@ def main():
     achieved = kern_bytes / (k_avg * 1e-6) / 1e9
     # HBM bytes per launch of the split kernel from the FETCH_SIZE / WRITE_SIZE counter runs (scaled on a plain copy) of
     # exactly this workload; a counter run cannot be made from inside this script, so other shapes report null
-    default_shape = (args.seed, b, heads, args.len_lo, args.len_hi, q_len, splits) == (0, 64, 128, 4096, 8192, 1, 4)
-    traffic, traffic_src = profile_traffic("mla_decode_v3_b64_ctx8k.md", default_shape)
+    default_shape = (args.seed, b, args.len_lo, args.len_hi, q_len, splits) == (0, 64, 4096, 8192, 1, 4)
+    profile_of = {128: "mla_decode_v3_b64_ctx8k.md", 16: "mla_decode_v3_b64_ctx8k_16heads.md"}
+    traffic, traffic_src = profile_traffic(profile_of.get(heads, ""), default_shape and heads in profile_of)
+    row_groups = 1 if heads * q_len <= 32 else (2 if heads * q_len <= 64 else 4)   # the kernel form the library picks
     res = {
-        "metric": "MLA decode us/layer (B=64, ctx 4k-8k, 128 heads, bf16, cache write + split-KV decode + reduce)",
+        "metric": f"MLA decode us/layer (B={b}, ctx {args.len_lo // 1024}k-{args.len_hi // 1024}k, {heads} heads, bf16, cache write + split-KV decode + reduce)",
         "value": round(dev_step_avg, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(us_per_step / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
@@ -896,7 +898,7 @@ def main():
         "step_hbm_gbs": round(ab["total"] / (dev_step_avg * 1e-6) / 1e9, 1),
         "step_roofline_frac": round(max(ab["total"] / (HBM_PEAK_GBS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
                                     / (dev_step_avg * 1e-6), 4),
-        "roofline": {"kernel": "mla_decode_v3_kernel<false, false>", "bound": "hbm", "achieved": round(achieved, 1),
+        "roofline": {"kernel": f"mla_decode_v3_kernel<false, false, {row_groups}>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "traffic_source": traffic_src,
                      "kernel_us_avg": round(k_avg, 2), "kernel_us_one_launch_alone_avg": round(k_iso_avg, 2),
