@@ -491,9 +491,18 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   // every wave has its query in registers (one barrier).
   TR_PRO(0);
   bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
+  // One row group: the two wavefronts that can own rows stage their query in the tile buffer of the segment's FOURTH block,
+  // which is not requested before the block loop runs, so the copying wavefronts ask for the first three blocks now and
+  // the query's round trip to memory hides under theirs.
+  const uint32_t q_stage = kRG == 1 ? (uint32_t)(((blk_begin + 3) & 3) * kNopeBufB) : 0u;
   if (!has_rows) {
 #pragma unroll
     for (int kk = 0; kk < 18; kk++) qf[kk] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (kRG == 1) {
+      issue_first();
+      ids_dma(blk_begin + kLead);
+      issue_next_two();
+    }
   } else {
     // Contraction step kk of the latent part covers the 16-byte granules 16*(kk%4) + 4g' + kk/4, g' = 0..3, and lane group
     // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
@@ -512,7 +521,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       for (int k = 0; k < 16; k++) {
         const bool ok = r0 + k < rows && L > 0;              // rows that do not exist read row 0 of the sequence
         const __bf16* src = qn0 + (ok ? (int64_t)(q0 + t) * st + (int64_t)h * sh : (int64_t)q0 * st);
-        dma16_sv(src, (uint32_t)((ln ^ swz_nope(k)) << 4), lds0 + wave * 16384 + k * 1024);
+        dma16_sv(src, (uint32_t)((ln ^ swz_nope(k)) << 4), lds0 + q_stage + wave * 16384 + k * 1024);
         h++;
         if (h == nh) { h = 0; t++; }
       }
@@ -534,7 +543,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     const int ql16 = ln & 15, qg = ln >> 4;
     const uint32_t qoff = (uint32_t)(wave * 16384 + ql16 * 1024 + (((qg << 2) ^ swz_nope(ql16)) << 4));
 #pragma unroll
-    for (int kk = 0; kk < 16; kk++) qf[kk] = *(const bf16x8*)(lds + (qoff ^ (uint32_t)((kk >> 2) << 4)) + (kk & 3) * 256);
+    for (int kk = 0; kk < 16; kk++) qf[kk] = *(const bf16x8*)(lds + q_stage + (qoff ^ (uint32_t)((kk >> 2) << 4)) + (kk & 3) * 256);
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) qf[16 + kk] = *(const bf16x8*)(lds + kPOff + wave * 2048 + ql16 * 128 + (2 * qg + kk) * 16);
 #pragma unroll
@@ -542,7 +551,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   }
   lds_barrier();                                              // every wave has read its query: the tile buffers are free
   TR_PRO(1);
-  issue_first();
+  if constexpr (kRG != 1) issue_first();
 
   f32x16 acc[2][4];                                          // [32-column block of this wave's 64][row group]
 #pragma unroll
@@ -816,6 +825,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     }
   }
   bool restart = false;
+  bool early_issued = kRG == 1;  // (one row group: the first three blocks were requested beside the query)
   int restarts_left = 4;         // every restart raises a reference by more than 2^100: fp32 has room for three
   do {
     if (restart) {
@@ -837,9 +847,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
           for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
       issue_first();
       restart = false;
+      early_issued = false;
     }
-    ids_dma(blk_begin + kLead);                               // (older than the copies below: their wait covers it)
-    issue_next_two();
+    if (!early_issued) {
+      ids_dma(blk_begin + kLead);                             // (older than the copies below: their wait covers it)
+      issue_next_two();
+    }
+    early_issued = false;
     // ---- block 0: QK, softmax, publish ----
     {
       if (nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);   // (kCopies per block in flight)

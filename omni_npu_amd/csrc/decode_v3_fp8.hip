@@ -391,6 +391,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   if (!has_rows) {
 #pragma unroll
     for (int kk = 0; kk < 18; kk++) qf[kk] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (kRG < 4) {
+      // small forms: the query is staged in the first 64 KiB (tiles) by wavefronts 0..3, the raw stages and rope buffers lie
+      // behind them, so the copying wavefronts ask for the first two raw blocks now, beside the query's round trip
+      issue_block(blk_begin);
+      if (nb > 1) issue_block(blk_begin + 1);
+    }
   } else {
     // Contraction step kk of the latent part covers the 16-byte granules 16*(kk%4) + 4g' + kk/4, g' = 0..3, and lane group
     // g takes granule g' = g (rope: granules 2g' + c for step c): the K-fragment read of two lanes 16 apart must not land
@@ -671,6 +677,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     }
   }
   bool restart = false;
+  bool early_issued = kRG < 4;   // (small forms: the first two raw blocks were requested beside the query)
   int restarts_left = 4;         // every restart raises a reference by more than 2^100: fp32 has room for three
   do {
     if (restart) {
@@ -689,8 +696,11 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       restart = false;
     }
     // ---- start-up: the first two raw blocks, dequantised into their tiles; then the third goes out ----
-    issue_block(blk_begin);                                   // raw stage of its parity, rope buffer 0
-    if (nb > 1) issue_block(blk_begin + 1);
+    if (!early_issued) {
+      issue_block(blk_begin);                                 // raw stage of its parity, rope buffer 0
+      if (nb > 1) issue_block(blk_begin + 1);
+    }
+    early_issued = false;
     MLA_WAIT_VMCNT(0);
     lds_barrier();                                            // both raw blocks have landed
     dequant_block(blk_begin);

@@ -24,7 +24,7 @@ int check_launch(const char* what) {
 // Kernels that use more dynamic LDS than the default limit must raise the limit once per device (the attribute belongs
 // to the device's copy of the function).  Remembered per (kernel, device); callers may come from several threads.
 int ensure_dynamic_lds(const void* kernel, int bytes, const char* what) {
-  constexpr int kMaxDev = 64, kMaxFn = 16;
+  constexpr int kMaxDev = 64, kMaxFn = 64;   // (the library has about twenty kernels that need the raised limit)
   static std::mutex mu;
   static const void* fns[kMaxFn];
   static bool done[kMaxFn][kMaxDev];
