@@ -38,17 +38,18 @@ typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scala
 // chain of dependent memory round trips, and this keeps the vector part of the chain at one.  (One row per wave keeps it
 // at four waves per SIMD; the gathers of the dominant keys' vectors are a third of its time.)
 // With many partials per sequence (few sequences, long contexts: up to 257 partials of one row) a single wavefront would
-// walk them in dozens of dependent round trips, so the kWide form gives a row to a whole workgroup: wavefront w merges
-// every fourth partial, sixteen per pass, and the four running states are merged through LDS at the end.
+// walk them in dozens of dependent round trips, so the kWide form gives a row to a whole workgroup of kWideWaves wavefronts
+// (eight while one workgroup per compute unit holds all rows, else four): wavefront w merges every kWideWaves-th partial,
+// sixteen per pass, and the running states are merged through LDS at the end.
 // With one chunk per sequence (large batches) a row has one partial, or two where a chunk border falls inside its
 // sequence: the kFew form then gives a wavefront four rows of two partials, a quarter of the wavefronts and rounds.
 constexpr int kRedPartsNarrow = 6, kRedPartsWide = 16, kRedPartsFew = 2, kRedRowsFew = 4;
-template <bool kWide, bool kFew>
-__global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
+template <bool kWide, bool kFew, int kWideWaves = 4>
+__global__ __launch_bounds__(kWide ? 64 * kWideWaves : 256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
   constexpr int kRedParts = kWide ? kRedPartsWide : (kFew ? kRedPartsFew : kRedPartsNarrow);
   constexpr int kRedRows = kFew ? kRedRowsFew : 1;
-  __shared__ float comb_ml[kWide ? 8 : 1];                  // wide: running maximum and sum of wavefronts 0..3
-  __shared__ float comb_a[kWide ? 4 * 64 * 8 : 1];          //       and their unnormalised rows
+  __shared__ float comb_ml[kWide ? 2 * kWideWaves : 1];            // wide: running maximum and sum of every wavefront
+  __shared__ float comb_a[kWide ? kWideWaves * 64 * 8 : 1];        //       and their unnormalised rows
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int r_max = p.max_q_len * p.num_heads;
@@ -111,11 +112,11 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
       c = (int)((((int64_t)before + 1) * G - 1) / T);
       c_last = (int)((((int64_t)before + mine) * G - 1) / T);
     }
-    // wide: wavefront w takes the chunks c + w, c + w + 4, ...; where chunks have to be tested one by one (tiny
+    // wide: wavefront w takes the chunks c + w, c + w + 8, ...; where chunks have to be tested one by one (tiny
     // workloads, a handful of partials) wavefront 0 takes them all
     int c_step = 1;
     if constexpr (kWide) {
-      if (dense_chunks) { c += wave; c_step = 4; }
+      if (dense_chunks) { c += wave; c_step = kWideWaves; }
       else if (wave != 0) c = c_last + 1;
     }
     while (c <= c_last) {
@@ -193,10 +194,10 @@ __global__ __launch_bounds__(256) void mla_chunk_reduce_kernel(const ChunkReduce
     if (wave == 0) {
       float mm = -INFINITY;
 #pragma unroll
-      for (int w = 0; w < 4; w++) mm = fmaxf(mm, comb_ml[w * 2]);
+      for (int w = 0; w < kWideWaves; w++) mm = fmaxf(mm, comb_ml[w * 2]);
       float tt = 0.f, aa[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int w = 0; w < 4; w++) {
+      for (int w = 0; w < kWideWaves; w++) {
         const float mw = comb_ml[w * 2];
         const float f = mw == -INFINITY ? 0.f : __expf(mw - mm);          // a wavefront without partials weighs nothing
         tt += comb_ml[w * 2 + 1] * f;
@@ -240,7 +241,10 @@ int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
   if (wide) {
     const int64_t row_groups = (int64_t)p.batch * r_max;
     const int64_t wgs = row_groups < (1ll << 30) ? row_groups : (1ll << 30);
-    hipLaunchKernelGGL((mla_chunk_reduce_kernel<true, false>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
+    // (measured, 128 heads: one sequence of 128k keys 25.5 -> 18.8 us with eight wavefronts per row; four sequences, i.e. two
+    // rounds of such workgroups, 16.0 us with four wavefronts against 19.2 with eight)
+    if (row_groups <= 256) hipLaunchKernelGGL((mla_chunk_reduce_kernel<true, false, 8>), dim3((unsigned)wgs), dim3(512), 0, stream, p);
+    else hipLaunchKernelGGL((mla_chunk_reduce_kernel<true, false, 4>), dim3((unsigned)wgs), dim3(256), 0, stream, p);
   } else if (few) {
     const int64_t row_groups = (int64_t)p.batch * ((r_max + kRedRowsFew - 1) / kRedRowsFew);
     hipLaunchKernelGGL((mla_chunk_reduce_kernel<false, true>), dim3((unsigned)((row_groups + 3) / 4)), dim3(256), 0, stream, p);
