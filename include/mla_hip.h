@@ -222,7 +222,8 @@ int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_strid
  * Replaces torch.ops.custom.npu_lightning_indexer, v1/layers/attention/npu_dsa.py:92-103 and
  * vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:133-146, in two steps:
  * dsa_indexer_scores_fp8: logits[t,s] = k_scale[s] * sum_h w[t,h] (* q_scale[t,h]) * relu(q8[t,h,:] . k8[s,:])
- * for the visible keys s of token t (64 heads, 128-wide float8_e4m3fn rows, fp32 scales);
+ * for the visible keys s of token t (64 heads, 128-wide float8_e4m3fn rows, fp32 scales; pages hold a multiple of 32 keys,
+ * key rows lie 128 .. 2^20 bytes apart, the scales of a page are contiguous);
  * dsa_topk: positions of the k largest logits, ties to the lower position, ascending order, -1 padding
  * (int32 [T,k], the reference's [T,1,topk] buffer). */
 int dsa_indexer_scores_fp8(const void* q8, int64_t q_stride_t, int64_t q_stride_h, const float* weights,
