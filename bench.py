@@ -865,8 +865,24 @@ def main():
     for _ in range(3):
         split_only()
     _, k_dev = timed(split_only, args.steps)
-    k_avg = k_dev / args.steps * 1e6
+    k_back_to_back = k_dev / args.steps * 1e6
     k_iso_avg, k_med = event_time(split_only, args.steps)
+    # ... and where it runs: args.steps whole steps queued as in the timed region above, the split phase of each bracketed
+    # by its own pair of events (the two phases as two calls); this is the duration a kernel trace of this command shows
+    reduce_only = lambda: K.decode(g["q_nope"], g["q_rope"], g["nope"], g["rope"], g["block_table"], g["seq_lens"],
+                                   case["scale"], out_v, q_len=q_len, num_splits=splits, workspace=ws, phase="reduce")
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for _ in range(args.warmup):
+        eager_step()
+    torch.cuda.synchronize()
+    for a, e in ev:
+        K.cache_write(g["new_c"], g["new_r"], g["slot_mapping"], g["nope"], g["rope"])
+        a.record()
+        split_only()
+        e.record()
+        reduce_only()
+    torch.cuda.synchronize()
+    k_avg = sum(a.elapsed_time(e) for a, e in ev) / len(ev) * 1e3
     power = None if args.no_power_probe else socket_power(split_only)
 
     ab = algorithmic_bytes(case, heads)
@@ -901,7 +917,8 @@ def main():
         "roofline": {"kernel": f"mla_decode_v3_kernel<false, false, {row_groups}>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "traffic_source": traffic_src,
-                     "kernel_us_avg": round(k_avg, 2), "kernel_us_one_launch_alone_avg": round(k_iso_avg, 2),
+                     "kernel_us_avg": round(k_avg, 2), "kernel_us_back_to_back_avg": round(k_back_to_back, 2),
+                     "kernel_us_one_launch_alone_avg": round(k_iso_avg, 2),
                      "kernel_us_one_launch_alone_median": round(k_med, 2),
                      "algorithmic_bytes": kern_bytes, "kernel_tflops": round(flops / (k_avg * 1e-6) / 1e12, 1),
                      "mfma_frac": round(flops / (k_avg * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
