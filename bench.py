@@ -381,7 +381,8 @@ def bench_prefill(K, dev, args):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round((fl_c + fl_s) / ((per["context_attention"] + per["suffix_attention"]) * 1e-6) / 1e12
                                    / MFMA_BF16_PEAK_TFLOPS, 4),
-                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_flops": fl_c + fl_s},
+                     "traffic": traffic, "traffic_source": traffic_src, "algorithmic_flops": fl_c + fl_s,
+                     "socket_power": None if args.no_power_probe else socket_power(stages[0][1], batch=4)},
     }
 
 
@@ -490,7 +491,8 @@ def bench_fp8(K, dev, args):
                      "frac": round(flops / (best * 1e-6) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                      "traffic": traffic, "traffic_source": traffic_src,
                      "algorithmic_flops": flops, "algorithmic_bytes": bytes_,
-                     "hbm_gbs": round(bytes_ / (best * 1e-6) / 1e9, 1)},
+                     "hbm_gbs": round(bytes_ / (best * 1e-6) / 1e9, 1),
+                     "socket_power": None if args.no_power_probe else socket_power(step, batch=4)},
     }
 
 
@@ -745,7 +747,7 @@ def main():
     ap.add_argument("--splits", type=int, default=0, help="KV splits per sequence (0 = library default)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-power-probe", action="store_true",
-                    help="decode workload: skip the two seconds of queued split-kernel launches under the socket power reading")
+                    help="decode, fp8 and prefill workloads: skip the two seconds of queued launches under the socket power reading")
     ap.add_argument("--graph", action="store_true",
                     help="decode workload: replay the steps from captured HIP graphs instead of launching their kernels one by "
                          "one.  Measured slower on this part: a graph leaves no idle time between kernels, the engine clock "
