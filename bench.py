@@ -294,8 +294,9 @@ def bench_dsa(K, dev, args):
 
 def bench_prefill(K, dev, args):
     """configs[2]: non-absorbed chunked prefill, 4 sequences, a 2048-token query chunk each over 16384 cached tokens,
-    128 heads (qk 128 + 64 rope, v 128).  Times the attention kernels (context part, causal suffix, merge) and, beside
-    them, the latent gather and the torch GEMM that up-projects the latent to K/V."""
+    128 heads (qk 128 + 64 rope, v 128).  Times the attention kernels (context part, then the causal suffix continuing
+    from the context's result: no merge launch) and, beside them, the separate merge the reference's flow has, the latent
+    gather and the torch GEMM that up-projects the latent to K/V."""
     g = torch.Generator().manual_seed(args.seed)
     B, N, Q, C = 4, 128, 2048, 16384
     scale = 192 ** -0.5
@@ -311,6 +312,7 @@ def bench_prefill(K, dev, args):
     o_s = torch.empty(B * Q, N, 128, dtype=torch.float32, device=dev)      # partials that the merge reads stay fp32
     o_c = torch.empty_like(o_s)
     o = torch.empty(B * Q, N, 128, dtype=torch.bfloat16, device=dev)
+    o_m = torch.empty_like(o)
     l_s = torch.empty(B * Q, N, dtype=torch.float32, device=dev)
     l_c = torch.empty_like(l_s)
     # latent cache of the prefix for the gather + up-projection leg
@@ -323,8 +325,10 @@ def bench_prefill(K, dev, args):
 
     stages = [
         ("context_attention", lambda: K.prefill_varlen(qn, qp, kc_n, kc_p, vc, cu_q, cu_c, Q, scale, False, o_c, l_c)),
-        ("suffix_attention", lambda: K.prefill_varlen(qn, qp, ks_n, ks_p, vs, cu_q, cu_q, Q, scale, True, o_s, l_s)),
-        ("merge", lambda: K.merge_states(o_c, l_c, o_s, l_s, o)),
+        ("suffix_attention", lambda: K.prefill_varlen(qn, qp, ks_n, ks_p, vs, cu_q, cu_q, Q, scale, True, o, prev_out=o_c,
+                                                      prev_lse=l_c)),
+        ("suffix_attention_alone", lambda: K.prefill_varlen(qn, qp, ks_n, ks_p, vs, cu_q, cu_q, Q, scale, True, o_s, l_s)),
+        ("merge_as_a_launch_of_its_own", lambda: K.merge_states(o_c, l_c, o_s, l_s, o_m)),
         ("gather_latent", lambda: K.gather_paged(nope, rope, gathered, bt, cu_c, B)),
         ("kv_up_proj_torch_gemm", lambda: torch.matmul(gathered[:, :512], w_up)),
     ]
@@ -345,7 +349,7 @@ def bench_prefill(K, dev, args):
     per = {name: round(ev_time(f, n), 1) for name, f in stages}
     fl_c = B * N * Q * C * 2 * (192 + 128)
     fl_s = B * N * Q * (Q + 1) // 2 * 2 * (192 + 128)
-    attn_us = per["context_attention"] + per["suffix_attention"] + per["merge"]
+    attn_us = per["context_attention"] + per["suffix_attention"]
     traffic, traffic_src = profile_traffic("mla_prefill_varlen_4x2048_over_16k.md", args.seed == 0)
     extra = {}
     if not args.no_cpu_baseline:

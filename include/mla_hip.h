@@ -218,6 +218,21 @@ int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_strid
                        int32_t max_q_len, int32_t causal, int32_t window, float scale, void* out, int64_t out_stride_t,
                        int64_t out_stride_h, int32_t out_dtype, float* lse_out, mlahip_stream_t stream);
 
+/* The same attention continued from an earlier result over OTHER keys of the same rows: prev_out fp32 [T,N,128] (strides
+ * in elements) and prev_lse fp32 [T,N] contiguous are what an earlier call returned (out_dtype 1, lse_out); the call returns
+ * the attention over the union of both key sets.  Replaces the pair "FIA over a context chunk, then merge_attn_states"
+ * of the reference's chunked-context loop (attention/backends/mla.py:415-447 with attention/ops.py:5-42) and the final
+ * merge of context and suffix (mla.py:594-606) by one launch each.  Rows whose prev_lse is -inf or +inf start empty, as
+ * the reference's merge treats them.  out may be prev_out and lse_out may be prev_lse. */
+int mla_prefill_varlen_continue(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
+                                int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
+                                int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v,
+                                int64_t v_stride_t, int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k,
+                                int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, int32_t window,
+                                float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
+                                float* lse_out, const float* prev_out, int64_t prev_stride_t, int64_t prev_stride_h,
+                                const float* prev_lse, mlahip_stream_t stream);
+
 /* ---- DSA lightning indexer --------------------------------------------------------------------
  * Replaces torch.ops.custom.npu_lightning_indexer, v1/layers/attention/npu_dsa.py:92-103 and
  * vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:133-146, in two steps:

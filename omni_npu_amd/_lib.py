@@ -49,6 +49,8 @@ SIGNATURES = {
                                          I32, I32, F32, P, I64, I64, P, I32, P]),
     "mla_prefill_varlen": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, P, I64, I64, P, P, I32, I32, I32, I32,
                                      I32, F32, P, I64, I64, I32, P, P]),
+    "mla_prefill_varlen_continue": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, P, I64, I64, P, P, I32, I32, I32,
+                                              I32, I32, F32, P, I64, I64, I32, P, P, I64, I64, P, P]),
     "dsa_indexer_scores_fp8": (c_int32, [P, I64, I64, P, I64, P, I64, P, I64, I64, P, I64, I64, I32, P, I64, I32, P, P, I32,
                                          I32, I32, I32, P, I64, P]),
     "dsa_quant_rows_fp8": (c_int32, [P, I64, I64, P, P, I64, I64, P, I64, I32, I64, P]),

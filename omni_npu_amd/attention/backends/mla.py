@@ -205,7 +205,9 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
 
     # ---- prefill ----
     def _compute_prefill_context(self, q_nope, q_pe, kv_c_cache, k_pe_cache, attn_metadata, k_scale):
-        """Chunked context: gather -> up-project -> unmasked attention with LSE -> running merge (reference mla.py:377-450)."""
+        """Chunked context: gather -> up-project -> unmasked attention with LSE (reference mla.py:377-450).  The reference
+        merges every chunk's result into a running one (merge_attn_states); here a chunk's launch continues from the
+        running result, so the merge is part of the attention kernel and there is no merge launch."""
         prefill = attn_metadata.prefill
         cc = prefill.chunked_context
         assert cc is not None
@@ -224,22 +226,21 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             kv_c_normed = cc.workspace[:toks][..., :self.kv_lora_rank]
             k_pe = cc.workspace[:toks][..., self.kv_lora_rank:]
             k_nope, v = self._kv_up(kv_c_normed)
-            # partial results that a merge will read stay fp32: each bf16 rounding in between would add 2^-10 of mean
-            # relative error to the layer's output
-            attn_output = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q_nope.device)
-            attn_lse = torch.empty(t, n, dtype=torch.float32, device=q_nope.device)
+            # running results stay fp32: each bf16 rounding in between would add 2^-10 of mean relative error to the
+            # layer's output
+            first = output is None
+            if first:
+                output = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q_nope.device)
+                output_lse = torch.empty(t, n, dtype=torch.float32, device=q_nope.device)
             K.prefill_varlen(q_nope, q_pe, k_nope, k_pe, v, cu_q, cc.cu_seq_lens[i].to(torch.int32).contiguous(),
-                             prefill.max_query_len, self.scale, False, attn_output, attn_lse)
-            if output is None:
-                output, output_lse = attn_output, attn_lse
-            else:
-                out_tmp, lse_tmp = torch.empty_like(output), torch.empty_like(output_lse)
-                K.merge_states(output, output_lse, attn_output, attn_lse, out_tmp, lse_tmp)
-                output, output_lse = out_tmp, lse_tmp
+                             prefill.max_query_len, self.scale, False, output, output_lse,
+                             prev_out=None if first else output, prev_lse=None if first else output_lse)
         return output, output_lse
 
     def _forward_prefill(self, q, kv_c_normed, k_pe, kv_cache, attn_metadata, k_scale) -> torch.Tensor:
-        """Causal suffix attention merged with the chunked context (reference mla.py:452-483, 573-616)."""
+        """Causal suffix attention merged with the chunked context (reference mla.py:452-483, 573-616): the context chunks
+        first, then the suffix launch continues from their result (the reference's final merge_attn_states, inside the
+        kernel)."""
         prefill = attn_metadata.prefill
         assert prefill is not None
         if self.sink_len > 0:
@@ -249,25 +250,21 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
         k_nope, v = self._kv_up(kv_c_normed)
         cu_q = prefill.query_start_loc.to(torch.int32).contiguous()
-        output = torch.empty(t, n, self.v_head_dim, dtype=torch.float32 if has_context else q.dtype, device=q.device)
-        output_lse = torch.empty(t, n, dtype=torch.float32, device=q.device) if has_context else None
-        K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
-                         output, output_lse)
+        ctx_out = ctx_lse = None
         if has_context:
             # (the fp8 cache is one tensor whose rows hold latent, scales and rope; the gather dequantises it)
             ctx_out, ctx_lse = self._compute_prefill_context(q_nope, q_pe, kv_cache[0],
                                                              None if self.fp8_cache else kv_cache[1], attn_metadata, k_scale)
-            if ctx_out is not None:
-                merged = torch.empty(t, n, self.v_head_dim, dtype=torch.bfloat16, device=q.device)
-                K.merge_states(ctx_out, ctx_lse, output, output_lse, merged)
-                output = merged
-        return output.to(torch.bfloat16).flatten(start_dim=-2)
+        output = torch.empty(t, n, self.v_head_dim, dtype=torch.bfloat16, device=q.device)
+        K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
+                         output, prev_out=ctx_out, prev_lse=ctx_lse)
+        return output.flatten(start_dim=-2)
 
     def _forward_prefill_sink(self, q, kv_c_normed, k_pe, prefill) -> torch.Tensor:
         """Prefill with static sink tokens (reference mla.py:463-560): the cached context is not read (mla.py:497).
         Without a window the sink latents go in front of every sequence's new latents and one right-down causal attention
         runs over sink_len + s_b keys.  With a window the reference runs a sink attention and a banded attention and merges
-        them by LSE; that is the same softmax over sink keys + band, computed here by the same two kernels calls."""
+        them by LSE; that is the same softmax over sink keys + band: here the banded launch continues from the sink result."""
         t, n, s_len = q.shape[0], self.num_heads, self.sink_len
         q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
         starts = prefill.query_start_loc_list
@@ -284,16 +281,14 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             return output.flatten(start_dim=-2)
         ks_nope, vs = self._kv_up(self.sink_compressed_kv)
         cu_s = s_len * torch.arange(nb + 1, dtype=torch.int32, device=q.device)
-        out_sink = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q.device)     # fp32 partials into the merge
-        band = torch.empty_like(out_sink)
+        out_sink = torch.empty(t, n, self.v_head_dim, dtype=torch.float32, device=q.device)     # the running result stays fp32
         lse_sink = torch.empty(t, n, dtype=torch.float32, device=q.device)
         K.prefill_varlen(q_nope, q_pe, ks_nope.repeat(nb, 1, 1), sink_pe.repeat(nb, 1), vs.repeat(nb, 1, 1), cu_q, cu_s,
                          prefill.max_query_len, self.scale, False, out_sink, lse_sink)
         k_nope, v = self._kv_up(kv_c_normed)
-        lse = torch.empty(t, n, dtype=torch.float32, device=q.device)
+        # the banded launch continues from the sink result: the reference's merge of the two, inside the kernel
         K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
-                         band, lse, window=self.sliding_window)
-        K.merge_states(out_sink, lse_sink, band, lse, output)
+                         output, window=self.sliding_window, prev_out=out_sink, prev_lse=lse_sink)
         return output.flatten(start_dim=-2)
 
     @staticmethod

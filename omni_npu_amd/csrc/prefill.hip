@@ -44,6 +44,10 @@ struct PrefillParams {
   float scale_log2;
   void* out; int64_t o_st, o_sh; int32_t out_fp32;
   float* lse; // [T, N]
+  // optional state to continue from: the normalised result and log-sum-exp of an attention over OTHER keys of the same rows
+  // (an earlier context chunk); the launch then returns the attention over the union, as a merge of the two would
+  const float* prev_out; int64_t po_st, po_sh;
+  const float* prev_lse;  // [T, N]
 };
 
 // copy one 64-key tile (keys k0 .. k0+63 of the flat key axis, clamped to klast) of head `head`
@@ -172,6 +176,25 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
+  if (p.prev_out != nullptr && row_ok) {
+    // Continue from (out, lse) over other keys: running maximum = lse (as a base-2 exponent), running sum = 1, accumulator
+    // = out.  A row without earlier keys comes with lse = -inf (+inf is read the same way, as the two-way merge does) and
+    // starts empty.  The sum lives in the row's lower half-wave lane; the halves are added at the end.
+    const float lse_prev = p.prev_lse[tq * p.num_heads + head];
+    if (lse_prev != INFINITY && lse_prev != -INFINITY) {
+      m_run = lse_prev * kLog2e;
+      l_run = half == 0 ? 1.f : 0.f;
+      const float* po = p.prev_out + tq * p.po_st + (int64_t)head * p.po_sh + 4 * half;
+#pragma unroll
+      for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          const f32x4 v = *(const f32x4*)(po + db * 32 + rg * 8);
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[db][rg * 4 + e] = v[e];
+        }
+    }
+  }
 
   if (tiles > 0) {
     const uint32_t lds0 = lds_addr_of(lds);
@@ -322,26 +345,28 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 using namespace mlahip;
 
 // out_dtype: 0 = bf16, 1 = fp32; window: 0 = every visible key, w = the newest w of them.  q_nope [T,N,128], q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64], v [Tk,N,128].
-extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
-                                  int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
-                                  int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v,
-                                  int64_t v_stride_t, int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k,
-                                  int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, int32_t window,
-                                  float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
-                                  float* lse_out, hipStream_t stream) {
-  MLA_REQUIRE(q_nope && q_pe && k_nope && k_pe && v && cu_q && cu_k && out, MLA_ERR_NULL,
-              "mla_prefill_varlen: null pointer argument");
+static int prefill_varlen_impl(const char* what, const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
+                               int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
+                               int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v,
+                               int64_t v_stride_t, int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k,
+                               int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, int32_t window,
+                               float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
+                               float* lse_out, const float* prev_out, int64_t prev_stride_t, int64_t prev_stride_h,
+                               const float* prev_lse, hipStream_t stream) {
+  MLA_REQUIRE(q_nope && q_pe && k_nope && k_pe && v && cu_q && cu_k && out, MLA_ERR_NULL, "%s: null pointer argument", what);
   MLA_REQUIRE(batch >= 0 && num_heads >= 1 && max_q_len >= 0 && batch <= 65535 && num_heads <= 65535 && window >= 0,
-              MLA_ERR_SHAPE, "mla_prefill_varlen: batch=%d num_heads=%d max_q_len=%d window=%d", batch, num_heads, max_q_len,
-              window);
-  MLA_REQUIRE(out_dtype == 0 || out_dtype == 1, MLA_ERR_UNSUPPORTED, "mla_prefill_varlen: out dtype code %d", out_dtype);
-  MLA_REQUIRE(scale > 0.f, MLA_ERR_UNSUPPORTED, "mla_prefill_varlen: the softmax scale must be positive (got %g)", (double)scale);
+              MLA_ERR_SHAPE, "%s: batch=%d num_heads=%d max_q_len=%d window=%d", what, batch, num_heads, max_q_len, window);
+  MLA_REQUIRE(out_dtype == 0 || out_dtype == 1, MLA_ERR_UNSUPPORTED, "%s: out dtype code %d", what, out_dtype);
+  MLA_REQUIRE(scale > 0.f, MLA_ERR_UNSUPPORTED, "%s: the softmax scale must be positive (got %g)", what, (double)scale);
   MLA_REQUIRE(qn_stride_t % 8 == 0 && qn_stride_h % 8 == 0 && qp_stride_t % 8 == 0 && qp_stride_h % 8 == 0 &&
                   kn_stride_t % 8 == 0 && kn_stride_h % 8 == 0 && kp_stride_t % 8 == 0 && v_stride_t % 8 == 0 &&
                   v_stride_h % 8 == 0 && out_stride_t % 4 == 0 && out_stride_h % 4 == 0 && (uintptr_t)q_nope % 16 == 0 &&
                   (uintptr_t)q_pe % 16 == 0 && (uintptr_t)k_nope % 16 == 0 && (uintptr_t)k_pe % 16 == 0 &&
                   (uintptr_t)v % 16 == 0 && (uintptr_t)out % 16 == 0,
-              MLA_ERR_SHAPE, "mla_prefill_varlen: rows must be 16-byte aligned");
+              MLA_ERR_SHAPE, "%s: rows must be 16-byte aligned", what);
+  MLA_REQUIRE((prev_out == nullptr) == (prev_lse == nullptr), MLA_ERR_NULL, "%s: the earlier result and its log-sum-exp go together", what);
+  MLA_REQUIRE(prev_out == nullptr || (prev_stride_t % 4 == 0 && prev_stride_h % 4 == 0 && (uintptr_t)prev_out % 16 == 0),
+              MLA_ERR_SHAPE, "%s: rows of the earlier result must be 16-byte aligned", what);
   if (batch == 0 || max_q_len == 0) return MLA_OK;
   PrefillParams p;
   p.q_nope = (const __bf16*)q_nope; p.qn_st = qn_stride_t; p.qn_sh = qn_stride_h;
@@ -353,9 +378,41 @@ extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64
   p.scale_log2 = scale * kLog2e;
   p.out = out; p.o_st = out_stride_t; p.o_sh = out_stride_h; p.out_fp32 = out_dtype;
   p.lse = lse_out;
-  const int rc = ensure_dynamic_lds((const void*)mla_prefill_varlen_kernel, kPfLdsB, "mla_prefill_varlen");
+  p.prev_out = prev_out; p.po_st = prev_stride_t; p.po_sh = prev_stride_h; p.prev_lse = prev_lse;
+  const int rc = ensure_dynamic_lds((const void*)mla_prefill_varlen_kernel, kPfLdsB, what);
   if (rc != MLA_OK) return rc;
   dim3 grid((max_q_len + kPfRows - 1) / kPfRows, num_heads, batch);
   hipLaunchKernelGGL(mla_prefill_varlen_kernel, grid, dim3(256), kPfLdsB, stream, p);
   return check_launch("mla_prefill_varlen_kernel");
+}
+
+extern "C" int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
+                                  int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
+                                  int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v,
+                                  int64_t v_stride_t, int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k,
+                                  int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, int32_t window,
+                                  float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, int32_t out_dtype,
+                                  float* lse_out, hipStream_t stream) {
+  return prefill_varlen_impl("mla_prefill_varlen", q_nope, qn_stride_t, qn_stride_h, q_pe, qp_stride_t, qp_stride_h, k_nope,
+                             kn_stride_t, kn_stride_h, k_pe, kp_stride_t, v, v_stride_t, v_stride_h, cu_q, cu_k, batch,
+                             num_heads, max_q_len, causal, window, scale, out, out_stride_t, out_stride_h, out_dtype, lse_out,
+                             nullptr, 0, 0, nullptr, stream);
+}
+
+// The same attention continued from an earlier result over other keys of the same rows (prev_out fp32 [T,N,128] with its
+// strides, prev_lse fp32 [T,N] contiguous): what the attention followed by the two-way merge returns, in one launch.
+// out may be prev_out and lse_out may be prev_lse (every row reads its own state before it writes it).
+extern "C" int mla_prefill_varlen_continue(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
+                                           int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
+                                           int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v,
+                                           int64_t v_stride_t, int64_t v_stride_h, const int32_t* cu_q, const int32_t* cu_k,
+                                           int32_t batch, int32_t num_heads, int32_t max_q_len, int32_t causal, int32_t window,
+                                           float scale, void* out, int64_t out_stride_t, int64_t out_stride_h,
+                                           int32_t out_dtype, float* lse_out, const float* prev_out, int64_t prev_stride_t,
+                                           int64_t prev_stride_h, const float* prev_lse, hipStream_t stream) {
+  MLA_REQUIRE(prev_out && prev_lse, MLA_ERR_NULL, "mla_prefill_varlen_continue: null pointer argument");
+  return prefill_varlen_impl("mla_prefill_varlen_continue", q_nope, qn_stride_t, qn_stride_h, q_pe, qp_stride_t, qp_stride_h,
+                             k_nope, kn_stride_t, kn_stride_h, k_pe, kp_stride_t, v, v_stride_t, v_stride_h, cu_q, cu_k, batch,
+                             num_heads, max_q_len, causal, window, scale, out, out_stride_t, out_stride_h, out_dtype, lse_out,
+                             prev_out, prev_stride_t, prev_stride_h, prev_lse, stream);
 }

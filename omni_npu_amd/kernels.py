@@ -678,11 +678,15 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
 # ------------------------------------------------------------------------------------------------
 def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tensor, k_pe: torch.Tensor, v: torch.Tensor,
                    cu_q: torch.Tensor, cu_k: torch.Tensor, max_q_len: int, scale: float, causal: bool,
-                   out: torch.Tensor, lse_out: Optional[torch.Tensor] = None, window: Optional[int] = None) -> torch.Tensor:
+                   out: torch.Tensor, lse_out: Optional[torch.Tensor] = None, window: Optional[int] = None,
+                   prev_out: Optional[torch.Tensor] = None, prev_lse: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Varlen non-absorbed MLA attention (reference: the prefill FIA calls, src/omni_npu/attention/backends/mla.py:574-590
     and :415-431).  q_nope [T,N,128], q_pe [T,N,64], k_nope [Tk,N,128], k_pe [Tk,64] (shared by the heads), v [Tk,N,128],
     cu_q / cu_k int32 [B+1] device tensors, out [T,N,128] bf16 or fp32, lse_out fp32 [T,N].  ``window`` keeps only the
-    newest ``window`` visible keys of each row (the sliding-window band of mla.py:525-541)."""
+    newest ``window`` visible keys of each row (the sliding-window band of mla.py:525-541).
+    ``prev_out`` (fp32 [T,N,128]) / ``prev_lse`` (fp32 [T,N]): the result of an earlier call over OTHER keys of the same
+    rows; the call then returns the attention over the union, i.e. what this attention followed by merge_attn_states
+    (src/omni_npu/attention/ops.py:5-42) gives, in one launch.  ``out`` may be ``prev_out``."""
     if window is not None and window < 1:
         raise ValueError(f"prefill_varlen: window must be positive (got {window})")
     _need_cuda(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, out, lse_out)
@@ -702,12 +706,35 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
         raise TypeError("prefill_varlen: cu_q / cu_k must be contiguous int32 [B+1]")
     if lse_out is not None and (lse_out.dtype != torch.float32 or lse_out.numel() != t * n or not lse_out.is_contiguous()):
         raise TypeError("prefill_varlen: lse_out must be contiguous fp32 [T,N]")
+    if (prev_out is None) != (prev_lse is None):
+        raise ValueError("prefill_varlen: prev_out and prev_lse go together")
+    if prev_out is not None:
+        _need_cuda(prev_out, prev_lse)
+        if prev_out.dtype != torch.float32 or prev_out.shape != (t, n, 128) or prev_out.stride(-1) != 1 or \
+                prev_lse.dtype != torch.float32 or prev_lse.numel() != t * n or not prev_lse.is_contiguous():
+            raise TypeError("prefill_varlen: prev_out must be fp32 [T,N,128], prev_lse contiguous fp32 [T,N]")
     if k_nope.shape[0] == 0 or t == 0:
         # no keys at all (a context chunk in which every sequence is empty): zeros and lse = -inf, as the kernel gives for
-        # an empty key range; empty tensors have no address to hand to the library
+        # an empty key range (the earlier result itself when there is one); empty tensors have no address to hand over
+        if prev_out is not None:
+            if out.data_ptr() != prev_out.data_ptr():
+                out.copy_(prev_out)
+            if lse_out is not None and lse_out.data_ptr() != prev_lse.data_ptr():
+                lse_out.copy_(prev_lse.view_as(lse_out))
+            return out
         out.zero_()
         if lse_out is not None:
             lse_out.fill_(float("-inf"))
+        return out
+    if prev_out is not None:
+        rc = lib.mla_prefill_varlen_continue(
+            q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_pe.data_ptr(), q_pe.stride(0), q_pe.stride(1),
+            k_nope.data_ptr(), k_nope.stride(0), k_nope.stride(1), k_pe.data_ptr(), k_pe.stride(0), v.data_ptr(), v.stride(0),
+            v.stride(1), cu_q.data_ptr(), cu_k.data_ptr(), cu_q.numel() - 1, n, int(max_q_len), 1 if causal else 0,
+            int(window or 0), float(scale), out.data_ptr(), out.stride(0), out.stride(1), _DT[out.dtype],
+            lse_out.data_ptr() if lse_out is not None else None, prev_out.data_ptr(), prev_out.stride(0), prev_out.stride(1),
+            prev_lse.data_ptr(), _stream(q_nope))
+        _lib.check(rc, "mla_prefill_varlen_continue")
         return out
     rc = lib.mla_prefill_varlen(q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_pe.data_ptr(), q_pe.stride(0),
                                 q_pe.stride(1), k_nope.data_ptr(), k_nope.stride(0), k_nope.stride(1), k_pe.data_ptr(),

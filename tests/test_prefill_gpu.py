@@ -109,6 +109,97 @@ def test_chunked_context_flow_gather_attend_merge(dev):
     attn_close(merged.view(t, -1), ref, 3e-2, 6e-3)
 
 
+def test_chunked_context_flow_with_continued_launches(dev):
+    """The same schedule with no merge launch: every context chunk's attention continues from the running result, and the
+    causal suffix continues from the context's (mla_prefill_varlen_continue); in place (out is the earlier result)."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(5)
+    bsz, ctx, suf, n = 2, 48, 16, 4
+    w = (torch.randn(512, n * 256, generator=g) * 0.02).bfloat16()
+    nope = torch.randn(bsz, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(bsz, 128, 64, generator=g).bfloat16()
+    bt = torch.tensor([[1], [0]], dtype=torch.int32)
+    q = torch.randn(bsz * suf, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(bsz * suf, 512, generator=g).bfloat16(), torch.randn(bsz * suf, 64, generator=g).bfloat16()
+    cu_q = torch.tensor([0, suf, 2 * suf], dtype=torch.int32)
+    chunks = [(torch.tensor([0, 32, 64], dtype=torch.int32), torch.tensor([0, 0], dtype=torch.int32)),
+              (torch.tensor([0, 16, 32], dtype=torch.int32), torch.tensor([32, 32], dtype=torch.int32))]
+    scale = 192 ** -0.5
+    ref = O.chunked_prefill(q, kvc, kpe, w, nope, rope, bt, cu_q.tolist(), chunks, scale)
+    d = lambda x: x.to(dev)
+    dq, dw = d(q), d(w)
+    t = bsz * suf
+    run_o = torch.empty(t, n, 128, dtype=torch.float32, device=dev)
+    run_l = torch.empty(t, n, dtype=torch.float32, device=dev)
+    ws = torch.empty(64, 576, dtype=torch.bfloat16, device=dev)
+    for i, (cu_k, starts) in enumerate(chunks):
+        toks = int(cu_k[-1])
+        K.gather_paged(d(nope), d(rope), ws, d(bt), d(cu_k), bsz, d(starts), total_rows=toks)
+        kv_c = (ws[:toks, :512] @ dw).view(toks, n, 256)
+        K.prefill_varlen(dq[..., :128], dq[..., 128:], kv_c[..., :128], ws[:toks, 512:], kv_c[..., 128:], d(cu_q), d(cu_k),
+                         suf, scale, False, run_o, run_l, prev_out=run_o if i else None, prev_lse=run_l if i else None)
+    kv_s = (d(kvc) @ dw).view(t, n, 256)
+    out = torch.empty(t, n, 128, dtype=torch.bfloat16, device=dev)
+    K.prefill_varlen(dq[..., :128], dq[..., 128:], kv_s[..., :128], d(kpe), kv_s[..., 128:], d(cu_q), d(cu_q), suf, scale,
+                     True, out, prev_out=run_o, prev_lse=run_l)
+    attn_close(out.view(t, -1), ref, 3e-2, 6e-3)
+
+
+@pytest.mark.parametrize("n,q_lens,k1,k2,causal2", [(4, [5, 130, 64], [40, 0, 300], [7, 200, 0], False),
+                                                    (16, [33, 1], [100, 64], [33, 1], True),
+                                                    (2, [257], [0], [257], True)])
+def test_prefill_continued_equals_attention_over_all_keys(dev, n, q_lens, k1, k2, causal2):
+    """Two launches, the second continuing from the first, against ONE oracle attention over the concatenated keys: the
+    first unmasked over k1 keys per sequence (some sequences have none: lse = -inf, the row starts empty), the second over
+    k2 keys (causal: the sequence's own tokens, right-down aligned).  fp32 and bf16 output, log-sum-exp included; a launch
+    without keys of its own returns the earlier result."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(n + len(q_lens))
+    bf = lambda *sh: torch.randn(*sh, generator=g).bfloat16()
+    t = sum(q_lens)
+    cu_q = [0]
+    for x in q_lens:
+        cu_q.append(cu_q[-1] + x)
+    cu1, cu2 = [0], [0]
+    for a, b in zip(k1, k2):
+        cu1.append(cu1[-1] + a)
+        cu2.append(cu2[-1] + b)
+    qn, qp = bf(t, n, 128), bf(t, n, 64)
+    kn1, kp1, v1 = bf(cu1[-1], n, 128), bf(cu1[-1], 64), bf(cu1[-1], n, 128)
+    kn2, kp2, v2 = bf(cu2[-1], n, 128), bf(cu2[-1], 64), bf(cu2[-1], n, 128)
+    scale = 192 ** -0.5
+    # the oracle over the union: keys of part 1 in front of the keys of part 2 (a causal part 2 is right-down aligned, so
+    # part 1 is visible to every row)
+    kn = torch.cat([torch.cat([kn1[cu1[i]:cu1[i + 1]], kn2[cu2[i]:cu2[i + 1]]]) for i in range(len(q_lens))])
+    kp = torch.cat([torch.cat([kp1[cu1[i]:cu1[i + 1]], kp2[cu2[i]:cu2[i + 1]]]) for i in range(len(q_lens))])
+    vv = torch.cat([torch.cat([v1[cu1[i]:cu1[i + 1]], v2[cu2[i]:cu2[i + 1]]]) for i in range(len(q_lens))])
+    cu_all = [a + b for a, b in zip(cu1, cu2)]
+    ref, ref_lse = O.attention_varlen(qn, qp, kn, kp, vv, cu_q, cu_all, scale, causal2)
+    d = lambda x: x.to(dev)
+    ti = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    o1 = torch.empty(t, n, 128, dtype=torch.float32, device=dev)
+    l1 = torch.empty(t, n, dtype=torch.float32, device=dev)
+    K.prefill_varlen(d(qn), d(qp), d(kn1), d(kp1), d(v1), ti(cu_q), ti(cu1), max(q_lens), scale, False, o1, l1)
+    for dt in (torch.float32, torch.bfloat16):
+        o2 = torch.full((t, n, 128), float("nan"), dtype=dt, device=dev)
+        l2 = torch.empty(t, n, dtype=torch.float32, device=dev)
+        K.prefill_varlen(d(qn), d(qp), d(kn2), d(kp2), d(v2), ti(cu_q), ti(cu2), max(q_lens), scale, causal2, o2, l2,
+                         prev_out=o1, prev_lse=l1)
+        attn_close(o2, ref, 2e-2, 2e-3 if dt == torch.float32 else 2.5e-3)
+        fin = torch.isfinite(ref_lse)
+        assert torch.equal(torch.isfinite(l2.cpu()), fin)
+        assert torch.allclose(l2.cpu()[fin], ref_lse[fin], atol=2e-2, rtol=0)
+    # nothing new to attend to: the earlier result comes back (through the kernel: cu_k all zero but keys present)
+    o3 = torch.empty_like(o1)
+    l3 = torch.empty_like(l1)
+    K.prefill_varlen(d(qn), d(qp), d(kn2[:1] if cu2[-1] else kn1[:1]), d(kp2[:1] if cu2[-1] else kp1[:1]),
+                     d(v2[:1] if cu2[-1] else v1[:1]), ti(cu_q), ti([0] * len(cu_q)), max(q_lens), scale, False, o3, l3,
+                     prev_out=o1, prev_lse=l1)
+    keep = torch.isfinite(l1)
+    assert torch.equal(o3[keep], o1[keep]) and torch.equal(l3[keep], l1[keep])
+    assert (o3[~keep] == 0).all() and torch.isinf(l3[~keep]).all()
+
+
 def _random_prefill_cases(n_cases, seed):
     import random
     rng = random.Random(seed)
