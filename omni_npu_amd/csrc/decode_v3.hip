@@ -50,10 +50,7 @@ static_assert(kLdsB <= 160 * 1024, "LDS budget");
 constexpr int kLead = 3;                                   // block i + kLead is copied while block i is consumed
 constexpr int kCopyWaves = 4;                              // wavefronts 0..3 issue the copies (the older wavefront of each SIMD)
 constexpr int kCopies = 9;                                 // copy instructions per copying wavefront and block (8 nope rows + rope)
-#ifndef MLA_V3_AHEAD
-#define MLA_V3_AHEAD 4
-#endif
-constexpr int kAhead = MLA_V3_AHEAD;                                  // K fragments read ahead of the MFMA that consumes them
+constexpr int kAhead = 4;                                  // K fragments read ahead of the MFMA that consumes them (2 and 6 measured the same)
 constexpr float kRestartThreshold = 100.f;                 // log2 units above a row's reference
 constexpr int kSegCost = kPlanSegCost;
 static_assert(kBlk == kPlanBlk, "the merge kernels recompute the chunk plan with these constants");
@@ -617,38 +614,25 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     // refills the fragment register (one statement, so that nothing is scheduled or padded in between)
 #define MLA_K_ADDR(j) (((j) >> 1) < 16 ? na[(j) >> 3] : ra[((j) >> 1) - 16])
 #define MLA_K_OFF(j) (((j) >> 1) < 16 ? ((j) & 1) * 16384 + (((j) >> 1) & 3) * 256 : ((j) & 1) * 2048)
-#if defined(ABL_QK_NOREAD)
-#define RD "; "
-#else
-#define RD
-#endif
-#if defined(ABL_QK_NOMFMA)
-#define MF "; "
-#else
-#define MF
-#endif
 #pragma unroll
-    for (int i = 0; i < kAhead; i++) asm volatile(RD "ds_read_b128 %0, %1 offset:%2" : "=v"(ka[i]) : "v"(MLA_K_ADDR(i)), "i"(MLA_K_OFF(i)));
+    for (int i = 0; i < kAhead; i++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(ka[i]) : "v"(MLA_K_ADDR(i)), "i"(MLA_K_OFF(i)));
 #pragma unroll
     for (int j = 0; j < 36; j++) {
       constexpr int D = kAhead;
       const int younger = (36 - 1 - j) < (D - 1) ? (36 - 1 - j) : (D - 1);
       if (j < 2)
-        asm volatile("s_waitcnt lgkmcnt(%5)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0\n\t" RD "ds_read_b128 %1, %3 offset:%4"
+        asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, 0\n\tds_read_b128 %1, %3 offset:%4"
                      : "=&v"(s[j & 1]), "+v"(ka[j % D]) : "v"(qf[j >> 1]), "v"(MLA_K_ADDR(j + D)), "i"(MLA_K_OFF(j + D)), "i"(younger));
       else if (j + D < 36)
-        asm volatile("s_waitcnt lgkmcnt(%5)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\t" RD "ds_read_b128 %1, %3 offset:%4"
+        asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\tds_read_b128 %1, %3 offset:%4"
                      : "+v"(s[j & 1]), "+v"(ka[j % D]) : "v"(qf[j >> 1]), "v"(MLA_K_ADDR(j + D)), "i"(MLA_K_OFF(j + D)), "i"(younger));
       else
-        asm volatile("s_waitcnt lgkmcnt(%3)\n\t" MF "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+        asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                      : "+v"(s[j & 1]) : "v"(ka[j % D]), "v"(qf[j >> 1]), "i"(younger));
     }
 #undef MLA_K_ADDR
 #undef MLA_K_OFF
     asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s[0]), "+v"(s[1]));
-#if defined(ABL_QK_NOMFMA) || defined(ABL_QK_NOREAD)
-    s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0];
-#endif
   };
 
   // ---- softmax + P.V, hand-ordered ----
@@ -896,12 +880,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       TR_ADD(1);
       const int fl = flags_read(blk);
       f32x4 s[2];
-#ifdef ABL_NO_QK
-      s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0];
-      if (true) {}                                            // no QK and no copies at all (never a copy past the segment)
-#elif defined(ABL_NO_COPY)
-      if (true) { qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0); s[0] = f32x4{0.f, 0.f, 0.f, 0.f}; s[1] = s[0]; }
-#else
       if constexpr (kRG < 4) {
         // small forms: wavefronts 4..7 only copy, the wavefronts that own rows only compute
         if (copier) {
@@ -922,7 +900,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       } else
       // (the wavefronts that copy nothing take the variant without copies: no branch around each copy, no page arithmetic)
       if (i + kLead >= nb || !copier) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
-#endif
       else if (kSparse || !full_ok || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead);
       else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + kLead);
       TR_ADD(2);
@@ -930,24 +907,9 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       Sm st;
       float sc[8];
       unpack_scores(s, sc);
-#ifdef ABL_NO_PVSM
-      st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
-      st.pw[0] = st.pw[1] = st.pw[2] = st.pw[3] = 0;
-#elif defined(ABL_NO_PV)
-      pv_softmax(blk, std::false_type{}, std::true_type{}, sc, st, true);
-#elif defined(ABL_NO_SOFTMAX)
-      st.pm = 0.f; st.t = 0.f; st.mx = 0; st.psum = sc[0] + sc[5];
-      st.pw[0] = st.pw[1] = st.pw[2] = st.pw[3] = 0;
-      pv_softmax(blk, std::true_type{}, std::false_type{}, sc, st, true);
-#else
       pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st, has_rows);
-#endif
       TR_ADD(3);
-#ifndef ABL_NO_FINISH
       if (has_rows) softmax_finish(blk + 1, sc, st);
-#else
-      l_run += st.psum + (float)st.pw[0];
-#endif
       TR_ADD(4);
 #ifdef MLA_V3_TRACE
       tr_n++;

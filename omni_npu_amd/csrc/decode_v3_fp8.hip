@@ -39,10 +39,7 @@ static_assert(8 * 16384 <= kPOff, "the query staging area ends in front of the P
 constexpr int kFp8RowBytes = 656, kFp8ScaleOffB = 512, kFp8RopeOffB = 528;
 constexpr int kCopyWaves = 4;                              // wavefronts 0..3 issue the copies (the older wavefront of each SIMD)
 constexpr int kCopies = 6;                                 // per copying wavefront and block: 4 x two latent rows, 8 scale sets, 8 rope rows
-#ifndef MLA_V3_AHEAD
-#define MLA_V3_AHEAD 4
-#endif
-constexpr int kAhead = MLA_V3_AHEAD;                                  // K fragments read ahead of the MFMA that consumes them
+constexpr int kAhead = 4;                                  // K fragments read ahead of the MFMA that consumes them (2 and 6 measured the same)
 constexpr float kRestartThreshold = 100.f;                 // log2 units above a row's reference
 constexpr int kSegCost = kPlanSegCost;
 static_assert(kBlk == kPlanBlk, "the merge kernels recompute the chunk plan with these constants");
