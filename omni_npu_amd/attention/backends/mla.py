@@ -82,17 +82,26 @@ class NPUMLAPrefillMetadata(MLACommonPrefillMetadata):
 @dataclass
 class NPUMLADecodeMetadata(MLACommonDecodeMetadata):
     # Unlike the reference (host lists, mla.py:137-138) the lengths stay on the device so that a captured HIP graph
-    # reads fresh values on every replay; the host copies are kept for callers that want them.
+    # reads fresh values on every replay.  Nothing on the GPU path reads host lists; a caller that wants the
+    # reference's gets them from seq_lens_list / query_cumlens_list, which are only built when asked for.
     query_cumlens: torch.Tensor = None
     query_start_loc: torch.Tensor = None
-    seq_lens_list: list = None
-    query_cumlens_list: list = None
+    seq_lens_cpu: torch.Tensor = None
+    query_start_loc_cpu: torch.Tensor = None
     q_len: int = 1
     max_seq_len: int = 0
     mc2_mask: torch.Tensor = None
     # static sink tokens (reference mla.py:152-153): the sink keys sit in the first pages of every block-table row and
     # ``seq_lens`` counts the keys behind them (the reference passes it next to block_table[:, num_sink_blocks:]).
     seq_sink_len: list = None
+
+    @property
+    def seq_lens_list(self) -> list:
+        return self.seq_lens_cpu.tolist()
+
+    @property
+    def query_cumlens_list(self) -> list:
+        return self.query_start_loc_cpu[1:].tolist()
 
 
 @dataclass
@@ -134,8 +143,8 @@ class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
             dcp_tot_seq_lens=dcp_tot_seq_lens_device,
             query_cumlens=query_start_loc_device[1:],
             query_start_loc=None if uniform else query_start_loc_device.to(torch.int32).contiguous(),
-            seq_lens_list=seq_lens_cpu.tolist(),
-            query_cumlens_list=query_start_loc_cpu[1:].tolist(),
+            seq_lens_cpu=seq_lens_cpu,
+            query_start_loc_cpu=query_start_loc_cpu,
             q_len=max_q,
             max_seq_len=int(seq_lens_cpu.max()) if num_decodes else 0,
         )
