@@ -43,7 +43,9 @@ typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scala
 // sixteen per pass, and the running states are merged through LDS at the end.
 // With one chunk per sequence (large batches) a row has one partial, or two where a chunk border falls inside its
 // sequence: the kFew form then gives a wavefront four rows of two partials, a quarter of the wavefronts and rounds.
-constexpr int kRedPartsNarrow = 6, kRedPartsWide = 16, kRedPartsFew = 2, kRedRowsFew = 4;
+// (eight partials per pass in the one-wavefront form: the eight segments of a sparse-attention token in one pass, 121
+// registers, still four wavefronts per SIMD; six measured 1 us slower there and on four to five partials per row)
+constexpr int kRedPartsNarrow = 8, kRedPartsWide = 16, kRedPartsFew = 2, kRedRowsFew = 4;
 template <bool kWide, bool kFew, int kWideWaves = 4>
 __global__ __launch_bounds__(kWide ? 64 * kWideWaves : 256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
   constexpr int kRedParts = kWide ? kRedPartsWide : (kFew ? kRedPartsFew : kRedPartsNarrow);
@@ -233,9 +235,9 @@ __global__ __launch_bounds__(kWide ? 64 * kWideWaves : 256) void mla_chunk_reduc
 int launch_chunk_reduce(const ChunkReduceParams& p, hipStream_t stream) {
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
   const int64_t per_seq = p.batch > 0 ? p.num_chunks / p.batch + 1 : 0;     // about that many partials per sequence
-  // many partials: past two passes of the one-wavefront form the wide form wins, as long as all rows' workgroups are
-  // resident at once (two per CU at its register use)
-  const bool wide = per_seq > 2 * kRedPartsNarrow && (int64_t)p.batch * r_max <= 512;
+  // many partials: past a dozen per row the wide form wins, as long as all rows' workgroups are resident at once (two
+  // per CU at its register use)
+  const bool wide = per_seq > 12 && (int64_t)p.batch * r_max <= 512;
   // one or two partials and rows for more than one round of resident wavefronts: four rows per wavefront
   const bool few = !wide && per_seq <= kRedPartsFew && (int64_t)p.batch * r_max > 16384;
   if (wide) {
