@@ -24,13 +24,25 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(ScatterSrc s0, Scatte
   const int64_t t = w / NSRC;
   if (t >= num_tokens) return;
   const ScatterSrc& s = (NSRC == 2 && (w % NSRC) == 1) ? s1 : s0;
+  // the slot and the first 1 KiB of the row are asked for together (one memory round trip in front of the store, not two)
+  const char* src = s.src + t * s.src_stride_b;
+  const int i0 = lane * 16;
+  u32x4 first = {0u, 0u, 0u, 0u};
+  if (i0 < s.row_bytes) first = *(const u32x4*)(src + i0);
   const int64_t slot = slots[t];
   if (slot < 0 || slot >= num_pages * page_size) return;
-  const int64_t pg = slot / page_size;
-  const int64_t off = slot - pg * page_size;
-  const char* src = s.src + t * s.src_stride_b;
+  int64_t pg, off;
+  if (slot < (1ll << 31)) {                                  // 32-bit division where it is enough (64-bit is a long routine)
+    const uint32_t pg32 = (uint32_t)slot / (uint32_t)page_size;
+    pg = pg32;
+    off = (uint32_t)slot - pg32 * (uint32_t)page_size;
+  } else {
+    pg = slot / page_size;
+    off = slot - pg * page_size;
+  }
   char* dst = s.cache + pg * s.page_stride_b + off * s.row_stride_b;
-  for (int i = lane * 16; i < s.row_bytes; i += 64 * 16) *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
+  if (i0 < s.row_bytes) *(u32x4*)(dst + i0) = first;
+  for (int i = i0 + 64 * 16; i < s.row_bytes; i += 64 * 16) *(u32x4*)(dst + i) = *(const u32x4*)(src + i);
 }
 
 }  // namespace mlahip
