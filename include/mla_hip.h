@@ -92,6 +92,14 @@ int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_stride_h, i
                         const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, int32_t interleaved_out,
                         void* out, int64_t out_stride_t, int64_t out_stride_h, mlahip_stream_t stream);
 
+/* Replaces torch_npu.npu_rotary_mul as the indexer calls it (v1/layers/attention/npu_dsa.py:120, 130): the
+ * half-rotation pairing, element i with element i + 32, out = cat(x1*c - x2*s, x2*c + x1*s) with x = cat(x1, x2)
+ * (the neox branch of layers/rotary_embedding/rotary_embedding_torch_npu.py:146-163).  x [T, N, 64] through its
+ * strides -> out [T, N, 64]; entry i*cos_step of a table row belongs to pair i; rows 8-byte aligned; in place is fine. */
+int mla_rotary_mul(const void* x, int64_t x_stride_t, int64_t x_stride_h, int64_t num_tokens, int32_t num_heads,
+                   const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, void* out,
+                   int64_t out_stride_t, int64_t out_stride_h, mlahip_stream_t stream);
+
 /* ---- absorbed-MLA paged decode ----------------------------------------------------------
  * Replaces the decode call of torch.ops.npu.npu_fused_infer_attention_score, attention/backends/mla.py:781-804
  * (input_layout "TND_NTD", block_size 128, sparse_mode 3): sequence b owns query tokens

@@ -159,6 +159,27 @@ __global__ __launch_bounds__(256) void interleave_rope_kernel(RopeParams p) {
   }
 }
 
+// Half-rotation ("neox") pairing: element i pairs with element i + 32, the result keeps the input's layout, so the
+// rotation may run in place.  One thread per (token, head, group of four pairs).
+__global__ __launch_bounds__(256) void rotary_mul_kernel(RopeParams p) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int j = (int)(i & 7);
+  const int64_t th = i >> 3;
+  const int64_t t = th / p.num_heads;
+  const int h = (int)(th - t * p.num_heads);
+  if (t >= p.num_tokens) return;
+  const __bf16* src = p.x + t * p.x_st + (int64_t)h * p.x_sh;
+  const bf16x4 a = *(const bf16x4*)(src + j * 4), b = *(const bf16x4*)(src + 32 + j * 4);
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 4; e++) { r[2 * e] = a[e]; r[2 * e + 1] = b[e]; }
+  bf16x4 o1, o2;
+  rope4(r, p.cos + t * p.cs_stride, p.sin + t * p.cs_stride, j * 4, p.cos_step, o1, o2);
+  char* dst = (char*)(p.out + t * p.o_st + (int64_t)h * p.o_sh);
+  *(bf16x4*)(dst + j * 8) = o1;
+  *(bf16x4*)(dst + 64 + j * 8) = o2;
+}
+
 static int check_tables(const char* who, const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step) {
   MLA_REQUIRE(cos && sin, MLA_ERR_NULL, "%s: null cos / sin table", who);
   MLA_REQUIRE((cos_step == 1 || cos_step == 2) && cs_stride >= 31 * (int64_t)cos_step + 1, MLA_ERR_SHAPE,
@@ -258,4 +279,24 @@ extern "C" int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_
   const int64_t threads = num_tokens * num_heads * 8;
   hipLaunchKernelGGL(interleave_rope_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, p);
   return check_launch("mla_interleave_rope");
+}
+
+extern "C" int mla_rotary_mul(const void* x, int64_t x_stride_t, int64_t x_stride_h, int64_t num_tokens, int32_t num_heads,
+                              const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, void* out,
+                              int64_t out_stride_t, int64_t out_stride_h, hipStream_t stream) {
+  MLA_REQUIRE(x && out, MLA_ERR_NULL, "mla_rotary_mul: null pointer argument");
+  if (int rc = check_tables("mla_rotary_mul", cos, sin, cs_stride, cos_step)) return rc;
+  MLA_REQUIRE(num_tokens >= 0 && num_heads >= 1 && num_tokens * num_heads < (1ll << 40), MLA_ERR_SHAPE,
+              "mla_rotary_mul: num_tokens=%lld num_heads=%d", (long long)num_tokens, num_heads);
+  MLA_REQUIRE(x_stride_t % 4 == 0 && x_stride_h % 4 == 0 && out_stride_t % 4 == 0 && out_stride_h % 4 == 0 &&
+                  (uintptr_t)x % 8 == 0 && (uintptr_t)out % 8 == 0,
+              MLA_ERR_SHAPE, "mla_rotary_mul: rows must be 8-byte aligned");
+  if (num_tokens == 0) return MLA_OK;
+  RopeParams p;
+  p.x = (const __bf16*)x; p.x_st = x_stride_t; p.x_sh = x_stride_h; p.out = (__bf16*)out; p.o_st = out_stride_t;
+  p.o_sh = out_stride_h; p.cos = (const __bf16*)cos; p.sin = (const __bf16*)sin; p.cs_stride = cs_stride;
+  p.cos_step = cos_step; p.num_tokens = num_tokens; p.num_heads = num_heads; p.interleaved_out = 0;
+  const int64_t threads = num_tokens * num_heads * 8;
+  hipLaunchKernelGGL(rotary_mul_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, p);
+  return check_launch("mla_rotary_mul");
 }

@@ -191,6 +191,26 @@ def interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, out: 
     return out
 
 
+def rotary_mul(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, out: Optional[torch.Tensor] = None,
+               table: str = "half") -> torch.Tensor:
+    """Rotary embedding of x [T, N, 64] with the half-rotation pairing (element i with i + 32), result in the input's
+    layout, like torch_npu.npu_rotary_mul in the indexer (src/omni_npu/v1/layers/attention/npu_dsa.py:120, 130).
+    ``out`` may be ``x`` (in place); returns ``out`` (a new tensor unless given)."""
+    _need_cuda(x, cos, sin)
+    lib = _lib.load()
+    if x.dim() != 3 or x.shape[-1] != D_ROPE or x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+        raise ValueError(f"x must be bf16 [T, N, 64] with a contiguous last dim, got {x.dtype} {tuple(x.shape)}")
+    if out is None:
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+    if out.shape != x.shape or out.dtype != x.dtype or out.stride(-1) != 1 or not out.is_cuda:
+        raise ValueError("out must match x")
+    cos, sin, step = _table_step(cos, sin, x.shape[0], table)
+    rc = lib.mla_rotary_mul(x.data_ptr(), x.stride(0), x.stride(1), x.shape[0], x.shape[1], cos.data_ptr(), sin.data_ptr(),
+                            cos.stride(0), step, out.data_ptr(), out.stride(0), out.stride(1), _stream(x))
+    _lib.check(rc, "mla_rotary_mul")
+    return out
+
+
 def gather_paged(nope_cache: torch.Tensor, rope_cache: torch.Tensor, dst: torch.Tensor, block_table: torch.Tensor,
                  cu_seq_lens: torch.Tensor, batch_size: int, seq_starts: Optional[torch.Tensor] = None,
                  total_rows: Optional[int] = None) -> None:

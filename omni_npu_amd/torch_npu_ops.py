@@ -1,6 +1,7 @@
 """The vendor ops of the step in front of the attention path, under the names and argument order the reference calls
 them with (``torch_npu.npu_kv_rmsnorm_rope_cache`` at src/omni_npu/v1/layers/attention/npu_mla.py:196-206, 296-309 and
-npu_dsa.py:410-424, 517-527; ``torch_npu.npu_interleave_rope`` at npu_mla.py:210, 316), backed by the HIP kernels.
+npu_dsa.py:410-424, 517-527; ``torch_npu.npu_interleave_rope`` at npu_mla.py:210, 316; ``torch_npu.npu_rotary_mul`` at
+npu_dsa.py:120, 130; ``torch_npu.npu_attention_update`` at attention/backends/mla.py:683-687), backed by the HIP kernels.
 
 Differences a caller must know: the cache layout is the plain paged one (``cache_mode="PA"``); the Ascend fractal layout
 ("PA_NZ") has no meaning for these kernels and is rejected.  Quantisation scales / offsets are rejected (the reference
@@ -50,3 +51,27 @@ def npu_interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -
     else:
         x3 = x
     return K.interleave_rope(x3, cos, sin, table="half").view(shape)
+
+
+def npu_rotary_mul(x: torch.Tensor, r1: torch.Tensor, r2: torch.Tensor) -> torch.Tensor:
+    """x * r1 + rotate_half(x) * r2 for x [B, N, S, 64] (or [T, N, 64]) and cos / sin rows r1 / r2 [B, 1, S, 64] whose two
+    halves are equal (cat(c, c), as the reference builds them): the half-rotation rotary embedding of the indexer
+    (npu_dsa.py:116-131).  Same shape as x."""
+    shape = x.shape
+    if x.dim() == 4:
+        if x.shape[2] != 1:
+            raise NotImplementedError("npu_rotary_mul: one position per (batch, head) row (S = 1)")
+        x3 = x.squeeze(2)
+    else:
+        x3 = x
+    return K.rotary_mul(x3, r1, r2, table="half").view(shape)
+
+
+def npu_attention_update(lse, local_out, update_type: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """N-way log-sum-exp merge of partial attention results: ``lse`` a list of n fp32 [R] vectors, ``local_out`` a list
+    of n [R, D] matrices -> (merged fp32 [R, D], merged lse fp32 [R]) (attention/backends/mla.py:683-687; the same
+    formula as attention/ops.py:109-141).  One launch for any n."""
+    if update_type != 0:
+        raise NotImplementedError(f"npu_attention_update: update_type {update_type}")
+    from .attention.ops import attention_update_torch
+    return attention_update_torch(list(local_out), [v.reshape(-1) for v in lse])

@@ -383,6 +383,21 @@ def interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, table
     return torch.cat((o1, o2), -1).to(x.dtype)
 
 
+def rotary_mul(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, table: str = "half") -> torch.Tensor:
+    """Half-rotation pairing: x = cat(x1, x2) on the last dim, o1 = x1*cos - x2*sin, o2 = x2*cos + x1*sin, result
+    cat(o1, o2) (layers/rotary_embedding/rotary_embedding_torch_npu.py:146-163, neox branch; what
+    torch_npu.npu_rotary_mul computes at v1/layers/attention/npu_dsa.py:120, 130 with rows cat(c, c)).  float64, rounded
+    once."""
+    d = x.shape[-1]
+    step = {"half": 1, "repeat": 2}[table]
+    c = cos.reshape(cos.shape[0], -1)[:, 0:(d // 2) * step:step].double()
+    s = sin.reshape(sin.shape[0], -1)[:, 0:(d // 2) * step:step].double()
+    while c.dim() < x.dim():
+        c, s = c.unsqueeze(1), s.unsqueeze(1)
+    x1, x2 = x[..., : d // 2].double(), x[..., d // 2:].double()
+    return torch.cat((x1 * c - x2 * s, x2 * c + x1 * s), -1).to(x.dtype)
+
+
 def kv_rmsnorm_rope_cache(kv, gamma, cos, sin, slot_mapping, nope_cache, rope_cache, eps, table="half",
                           interleaved_out=False):
     """The fused vendor op torch_npu.npu_kv_rmsnorm_rope_cache (v1/layers/attention/npu_mla.py:196-206) as the

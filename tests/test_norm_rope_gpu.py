@@ -138,6 +138,23 @@ def test_query_rope_strided_and_in_place(dev, layout, interleaved):
             K.interleave_rope(qd[..., 128:], cos.to(dev), sin.to(dev), out=qd[..., 128:], table=layout)
 
 
+@pytest.mark.parametrize("layout", ["half", "repeat"])
+def test_rotary_mul_strided_and_in_place(dev, layout):
+    """The half-rotation pairing of the indexer's rope dims (npu_dsa.py:116-131) on a strided view, then in place."""
+    from omni_npu_amd import kernels as K
+    t, n = 41, 64
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(t, n, 128, generator=g).bfloat16()
+    pos = torch.randint(0, 8192, (t,), generator=g)
+    cos, sin = O.rope_tables(pos, layout=layout)
+    want = O.rotary_mul(q[..., :64], cos, sin, table=layout)
+    qd = q.to(dev)
+    got = K.rotary_mul(qd[..., :64], cos.to(dev), sin.to(dev), table=layout)
+    _ulp_close(got, want)
+    K.rotary_mul(qd[..., :64], cos.to(dev), sin.to(dev), out=qd[..., :64], table=layout)
+    assert torch.equal(qd[..., :64], got) and torch.equal(qd[..., 64:].cpu(), q[..., 64:])
+
+
 def test_reference_named_ops(dev):
     """The call shapes of src/omni_npu/v1/layers/attention/npu_mla.py:296-316."""
     from omni_npu_amd import torch_npu_ops as T
@@ -161,3 +178,19 @@ def test_reference_named_ops(dev):
     got = T.npu_interleave_rope(q_pe.to(dev), cos.to(dev).view(-1, 1, 1, 64), sin.to(dev).view(-1, 1, 1, 64))
     assert got.shape == q_pe.shape
     _ulp_close(got.view(t, n, 64), O.interleave_rope(q_pe.view(t, n, 64), cos, sin))
+    # the indexer's call (npu_dsa.py:116-131): [T, N, 1, 64] with full-width rows
+    got = T.npu_rotary_mul(q_pe.to(dev), cos.to(dev).view(-1, 1, 1, 64), sin.to(dev).view(-1, 1, 1, 64))
+    assert got.shape == q_pe.shape
+    _ulp_close(got.view(t, n, 64), O.rotary_mul(q_pe.view(t, n, 64), cos, sin))
+    # the merge of partial results under the vendor op's name and argument layout (mla.py:683-687)
+    parts, rows, d = 3, 40, 512
+    outs = [torch.randn(rows, d, generator=g) for _ in range(parts)]
+    lses = [torch.randn(rows, generator=g) * 3 for _ in range(parts)]
+    lses[1][5] = float("-inf")
+    merged, lse = T.npu_attention_update(lse=[v.to(dev) for v in lses], local_out=[o.to(dev) for o in outs], update_type=0)
+    want_o, want_l = O.attention_update(torch.stack(outs), torch.stack(lses))
+    assert merged.shape == (rows, d) and lse.shape == (rows,)
+    assert torch.allclose(merged.cpu(), want_o.float(), rtol=1e-5, atol=1e-5)
+    assert torch.allclose(lse.cpu(), want_l.float(), rtol=1e-5, atol=1e-5)
+    with pytest.raises(NotImplementedError):
+        T.npu_attention_update(lse=[v.to(dev) for v in lses], local_out=[o.to(dev) for o in outs], update_type=1)

@@ -93,3 +93,30 @@ def test_fused_oracle_is_the_composition_and_skips_pad_slots():
     untouched = torch.ones(256, dtype=torch.bool)
     untouched[[5, 130, 255, 0]] = False
     assert (flat_n[untouched] == 0).all() and (flat_r[untouched] == 0).all()
+
+
+def test_rotary_mul_float64_loop_library_rotate_half_and_the_interleaved_form():
+    """The half-rotation pairing (torch_npu.npu_rotary_mul in the indexer, npu_dsa.py:120, 130): entry by entry in
+    float64, against the transformers library's rotate_half formulation, and as the interleaved form on permuted input."""
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(6, 3, 64, generator=g).bfloat16()
+    pos = torch.tensor([0, 1, 17, 300, 4095, 9999])
+    cos, sin = O.rope_tables(pos)
+    out = O.rotary_mul(x, cos, sin)
+    for t in (0, 2, 5):
+        for i in (0, 13, 31):
+            c, s = float(cos[t, i]), float(sin[t, i])
+            a, b = float(x[t, 1, i]), float(x[t, 1, 32 + i])
+            assert out[t, 1, i] == torch.tensor(a * c - b * s, dtype=torch.float64).bfloat16()
+            assert out[t, 1, 32 + i] == torch.tensor(b * c + a * s, dtype=torch.float64).bfloat16()
+    # library routine: q * cos + rotate_half(q) * sin with full-width rows cat(c, c)
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    xd = x.double().transpose(0, 1).unsqueeze(0)                        # [1, heads, tokens, 64]
+    lib, _ = apply_rotary_pos_emb(xd, xd, cos.double().unsqueeze(0), sin.double().unsqueeze(0))
+    assert torch.equal(lib.squeeze(0).transpose(0, 1).bfloat16(), out)
+    # the same rotation as the interleaved pairing applied to the interleaved arrangement of the same numbers
+    inter = torch.stack((x[..., :32], x[..., 32:]), -1).reshape(x.shape)
+    assert torch.equal(O.interleave_rope(inter, cos, sin), out)
+    # the 'repeat' table layout carries the same numbers
+    cr, sr = O.rope_tables(pos, layout="repeat")
+    assert torch.equal(O.rotary_mul(x, cr, sr, "repeat"), out)
