@@ -3,13 +3,16 @@ selection (fp8 quantisation, key cache write, score GEMM, exact top-k).
 
 Mirrors the patched ``Indexer.__init__`` / ``forward`` of
 src/omni_npu/vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:24-146; the linear layers are plain
-``torch.nn.Linear`` (library GEMMs; the reference uses replicated, i.e. unsharded, linears too, :50-67)."""
+``torch.nn.Linear`` (library GEMMs; the reference uses replicated, i.e. unsharded, linears too, :50-67).
+``forward_tables`` is the custom-model variant of src/omni_npu/v1/layers/attention/npu_dsa.py:105-142, which gets the
+cos / sin rows of its tokens instead of positions and rotates with the half-rotation pairing (``npu_rotary_mul``)."""
 from __future__ import annotations
 
 from typing import Optional
 
 import torch
 
+from ... import kernels as K
 from ...attention.backends.dsa import LightningIndexer
 
 
@@ -41,3 +44,15 @@ class DSV32Indexer(torch.nn.Module):
         k = torch.cat([k_pe.squeeze(1), k_nope], dim=-1)
         weights = self.weights_proj(hidden_states)
         return self.select(q, k, weights, kv_cache, attn_metadata)
+
+    def forward_tables(self, hidden_states: torch.Tensor, qr: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                       attn_metadata=None, kv_cache=None):
+        """Argument order and return value of npu_dsa.py:105-142: (top-k indices, the rotated index key [T, 1, 128]).
+        The rope dims sit in front of the others in q and k already, so the rotation runs in place on strided views and
+        no concatenation is needed."""
+        q = self.wq_b(qr).view(-1, self.n_head, self.head_dim)
+        k = self.k_norm(self.wk(hidden_states)).unsqueeze(1)
+        K.rotary_mul(q[..., :self.rope_dim], cos, sin, out=q[..., :self.rope_dim])
+        K.rotary_mul(k[..., :self.rope_dim], cos, sin, out=k[..., :self.rope_dim])
+        weights = self.weights_proj(hidden_states)
+        return self.select(q, k.squeeze(1), weights, kv_cache, attn_metadata), k

@@ -104,7 +104,10 @@ def test_forward_oot_matches_fp32_chain(dev, q_lens, seq_lens, fused):
     assert ((got_r.view(torch.int16).int() - k_pe.view(torch.int16).int()).abs() <= 1).all()
 
 
-def test_indexer_module_selects_what_the_oracle_selects(dev):
+@pytest.mark.parametrize("variant", ["positions", "tables"])
+def test_indexer_module_selects_what_the_oracle_selects(dev, variant):
+    """``positions``: the patched module (patch_dsv32_indexer.py:77-146, rotary module, interleaved pairs); ``tables``:
+    the custom-model module (npu_dsa.py:105-142, cos / sin rows, half-rotation pairing)."""
     from omni_npu_amd.layers.attention.indexer import DSV32Indexer
     from omni_npu_amd.layers.rotary_embedding import HIPRotaryEmbedding
     torch.manual_seed(0)
@@ -130,7 +133,15 @@ def test_indexer_module_selects_what_the_oracle_selects(dev):
     meta = builder.build(0, _to(common, dev))
     x = torch.randn(t, hidden, generator=g).bfloat16()
     qr = torch.randn(t, q_lora, generator=g).bfloat16()
-    sel = idx(x.to(dev), qr.to(dev), positions.to(dev), rotary, kv_cache, meta)
+    cos, sin = O.rope_tables(positions)
+    if variant == "positions":
+        sel = idx(x.to(dev), qr.to(dev), positions.to(dev), rotary, kv_cache, meta)
+        rotate = O.interleave_rope
+    else:
+        sel, k_out = idx.forward_tables(x.to(dev), qr.to(dev), cos.to(dev).view(-1, 1, 1, 64), sin.to(dev).view(-1, 1, 1, 64),
+                                        meta, kv_cache)
+        assert k_out.shape == (t, 1, 128)
+        rotate = O.rotary_mul
     assert sel.shape == (t, 1, topk) and idx.topk_indices_buffer.data_ptr() == sel.data_ptr()
 
     # the module's q, k, weights restated on the CPU from its own parameters; selection by the oracle on those
@@ -138,9 +149,10 @@ def test_indexer_module_selects_what_the_oracle_selects(dev):
     q = (qr.float() @ cpu(idx.wq_b)["weight"].T).bfloat16().view(t, 64, 128)
     kk = torch.nn.functional.layer_norm((x.float() @ cpu(idx.wk)["weight"].T).bfloat16().float(), (128,),
                                         cpu(idx.k_norm)["weight"], cpu(idx.k_norm)["bias"], 1e-6).bfloat16()
-    cos, sin = O.rope_tables(positions)
-    q = torch.cat([O.interleave_rope(q[..., :64], cos, sin), q[..., 64:]], -1)
-    kk = torch.cat([O.interleave_rope(kk[:, :64], cos, sin), kk[:, 64:]], -1)
+    q = torch.cat([rotate(q[..., :64], cos, sin), q[..., 64:]], -1)
+    kk = torch.cat([rotate(kk[:, :64], cos, sin), kk[:, 64:]], -1)
+    if variant == "tables":
+        assert ((k_out.cpu().view(t, 128).view(torch.int16).int() - kk.view(torch.int16).int()).abs() <= 2).all()
     wts = (x.float() @ cpu(idx.weights_proj)["weight"].T).bfloat16().float()
     sm = common.slot_mapping.cpu()
     # the new key rows in the cache: quantised like the oracle quantises them (GEMM / LayerNorm rounding may move a bf16
