@@ -104,6 +104,72 @@ def test_forward_oot_matches_fp32_chain(dev, q_lens, seq_lens, fused):
     assert ((got_r.view(torch.int16).int() - k_pe.view(torch.int16).int()).abs() <= 1).all()
 
 
+@pytest.mark.parametrize("q_lens,seq_lens", [([1] * 5, [200, 31, 129, 500, 1000]), ([2, 2, 2], [150, 400, 77]),
+                                             ([40, 7, 130], [40, 7, 130])])
+def test_custom_model_module_matches_fp32_chain(dev, q_lens, seq_lens):
+    """``NPUDeepseekMLAAttention.forward(hidden_states, cos, sin)`` (src/omni_npu/v1/layers/attention/npu_mla.py:152-348):
+    all-decode batches (MTP too) and all-prefill batches without cached context, against the fp32 chain on the CPU."""
+    from omni_npu_amd.layers.attention.npu_mla_wrapper import MLAAttention
+    from omni_npu_amd.v1.layers.attention import NPUDeepseekMLAAttention
+    g = torch.Generator().manual_seed(sum(seq_lens) + len(q_lens))
+    hidden, n, q_lora = 256, 16, 128
+    w = _weights(g, hidden, n, q_lora)
+    common = _common(q_lens, seq_lens)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    common.slot_mapping = torch.cat([O.slots_for(common.block_table_tensor, b, s - ql, s)
+                                     for b, (ql, s) in enumerate(zip(q_lens, seq_lens))])
+    positions = torch.cat([torch.arange(s - ql, s) for ql, s in zip(q_lens, seq_lens)])
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    x = torch.randn(t, hidden, generator=g).bfloat16()
+
+    impl, w_kv_b = _mk_impl(mla.NPUMLAImpl, n, dev, seed=5)
+    attn = MLAAttention(impl)
+    raw = torch.cat([nope.reshape(-1), rope.reshape(-1)]).to(dev).view(torch.uint8)
+    attn.kv_cache = [mla.NPUMLABackend.reshape_kv_cache(raw, nblk, 128, 1, 576, dtype=torch.bfloat16)]
+    wq_a, wkv_a = w["qkv_a"][:, :q_lora].contiguous(), w["qkv_a"][:, q_lora:].contiguous()
+    mod = NPUDeepseekMLAAttention(hidden, n, 128, 64, 128, q_lora, 512, attn, _Lin(wq_a.to(dev)), _Norm(w["q_norm"].to(dev)),
+                                  _Lin(w["q_b"].to(dev)), _Lin(wkv_a.to(dev)), _Norm(w["kv_norm"].to(dev)), _Lin(w["o"].to(dev)))
+    builder = mla.NPUMLAMetadataBuilder(V.AttentionSpec(128, 1, 576, torch.bfloat16), ["l"], _cfg(cap=2), dev)
+
+    # ---- fp32 chain on the CPU (bf16 rounding only where the GPU chain stores bf16 tensors) ----
+    q_c = torch.nn.functional.rms_norm((x.float() @ wq_a.float()).bfloat16().float(), (q_lora,), w["q_norm"].float(),
+                                       EPS).bfloat16()
+    q = (q_c.float() @ w["q_b"].float()).bfloat16().view(t, n, 192)
+    kv = (x.float() @ wkv_a.float()).bfloat16()
+    cos, sin = O.rope_tables(positions)
+    kv_a = O.rms_norm(kv[:, :512], w["kv_norm"], EPS)
+    k_pe = O.interleave_rope(kv[:, 512:], cos, sin)
+    q = torch.cat([q[..., :128], O.interleave_rope(q[..., 128:], cos, sin)], -1)
+    attn_ref = _oracle_mla(q.float(), kv_a, k_pe.view(t, 1, 64), w_kv_b, nope.clone(), rope.clone(), common, n, impl.scale)
+    ref = attn_ref.bfloat16().float() @ w["o"].float()
+
+    meta = builder.build(0, _to(common, dev))
+    assert (meta.prefill is None) != (meta.decode is None)
+    cd, sd = cos.to(dev).view(-1, 1, 1, 64), sin.to(dev).view(-1, 1, 1, 64)
+    with V.set_forward_context(attn_metadata={attn.layer_name: meta}):
+        out = mod(x.to(dev), cd, sd)
+    assert out.shape == (t, hidden)
+    err = (out.float().cpu() - ref).abs().max().item()
+    assert err <= 3e-2 * ref.abs().max().item(), f"max err {err:.4g} vs scale {ref.abs().max().item():.4g}"
+    sm = common.slot_mapping.cpu()
+    got_n = attn.kv_cache[0][0].cpu().view(-1, 512)[sm]
+    got_r = attn.kv_cache[0][1].cpu().view(-1, 64)[sm]
+    # (the kv projection is a bf16 GEMM on the GPU and an fp32 product rounded once here, so a projected value can land on
+    # the other side of a rounding boundary: the bar is one bf16 step of the value, or of 1/16 for values that are
+    # differences of larger terms, and almost all of them identical to the last bit but one)
+    for got, want in ((got_n, kv_a), (got_r, k_pe)):
+        step = 2.0 ** -7 * want.float().abs().clamp(min=1 / 16)
+        assert ((got.float() - want.float()).abs() <= step).all()
+        d = (got.view(torch.int16).int() - want.view(torch.int16).int()).abs()
+        assert float((d <= 1).float().mean()) >= 0.999
+    # memory-profiling run: no metadata, no cache access, the projections still run
+    with V.set_forward_context(attn_metadata=None):
+        dry = mod(x.to(dev), cd, sd)
+    assert dry.shape == (t, hidden) and float(dry.abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("variant", ["positions", "tables"])
 def test_indexer_module_selects_what_the_oracle_selects(dev, variant):
     """``positions``: the patched module (patch_dsv32_indexer.py:77-146, rotary module, interleaved pairs); ``tables``:
