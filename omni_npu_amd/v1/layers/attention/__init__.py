@@ -1,3 +1,4 @@
+from .npu_dsa import NPUDeepseekSparseAttention
 from .npu_mla import NPUDeepseekMLAAttention
 
-__all__ = ["NPUDeepseekMLAAttention"]
+__all__ = ["NPUDeepseekMLAAttention", "NPUDeepseekSparseAttention"]

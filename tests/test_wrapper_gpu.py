@@ -170,6 +170,80 @@ def test_custom_model_module_matches_fp32_chain(dev, q_lens, seq_lens):
     assert dry.shape == (t, hidden) and float(dry.abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("q_lens,seq_lens", [([1, 1, 1], [700, 90, 300]), ([40, 9], [40, 9])])
+def test_custom_model_sparse_module(dev, q_lens, seq_lens):
+    """``NPUDeepseekSparseAttention.forward(hidden_states, cos, sin)`` (src/omni_npu/v1/layers/attention/npu_dsa.py:296-586):
+    the output against the oracle's sparse attention over the positions the module's own indexer selected (the selection
+    itself is covered by test_indexer_module_selects_what_the_oracle_selects), wrapped in the fp32 chain of projections."""
+    from omni_npu_amd.layers.attention.indexer import DSV32Indexer
+    from omni_npu_amd.layers.attention.npu_mla_wrapper import MLAAttention
+    from omni_npu_amd.v1.layers.attention import NPUDeepseekSparseAttention
+    torch.manual_seed(1)
+    g = torch.Generator().manual_seed(sum(seq_lens))
+    hidden, n, q_lora, topk = 256, 128, 128, 64
+    w = _weights(g, hidden, n, q_lora)
+    common = _common(q_lens, seq_lens)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    common.slot_mapping = torch.cat([O.slots_for(common.block_table_tensor, b, s - ql, s)
+                                     for b, (ql, s) in enumerate(zip(q_lens, seq_lens))])
+    positions = torch.cat([torch.arange(s - ql, s) for ql, s in zip(q_lens, seq_lens)])
+    raw = torch.zeros(nblk * 128 * 704, dtype=torch.bfloat16, device=dev).view(torch.uint8)
+    kv_cache = dsa.NPUDSABackend.reshape_kv_cache(raw, nblk, 128, 1, 704, dtype=torch.bfloat16)
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    kv_cache[0].copy_(nope.view(nblk, 128, 1, 512)); kv_cache[1].copy_(rope.view(nblk, 128, 1, 64))
+    k8_ref, ks_ref = O.fp8_quant_token(torch.randn(nblk, 128, 128, generator=g).bfloat16().float())
+    k8v, ksv = dsa.indexer_cache_views(kv_cache[2])
+    k8v.copy_(k8_ref.view(torch.uint8)); ksv.copy_(ks_ref)
+    x = torch.randn(t, hidden, generator=g).bfloat16()
+
+    impl, w_kv_b = _mk_impl(dsa.NPUDSAImpl, n, dev, seed=5)
+    attn = MLAAttention(impl)
+    attn.kv_cache = [kv_cache]
+    idx = DSV32Indexer(hidden, q_lora, topk, max_tokens=t, device=dev)
+    wq_a, wkv_a = w["qkv_a"][:, :q_lora].contiguous(), w["qkv_a"][:, q_lora:].contiguous()
+    mod = NPUDeepseekSparseAttention(hidden, n, 128, 64, 128, q_lora, 512, attn, idx, _Lin(wq_a.to(dev)),
+                                     _Norm(w["q_norm"].to(dev)), _Lin(w["q_b"].to(dev)), _Lin(wkv_a.to(dev)),
+                                     _Norm(w["kv_norm"].to(dev)), _Lin(w["o"].to(dev)))
+    builder = dsa.NPUDSAMetadataBuilder(V.AttentionSpec(128, 1, 704, torch.bfloat16), ["l"], _cfg(cap=1), dev)
+    meta = builder.build(0, _to(common, dev))
+    cos, sin = O.rope_tables(positions)
+    cd, sd = cos.to(dev).view(-1, 1, 1, 64), sin.to(dev).view(-1, 1, 1, 64)
+    with V.set_forward_context(attn_metadata={attn.layer_name: meta}):
+        out = mod(x.to(dev), cd, sd)
+    assert out.shape == (t, hidden)
+    sel = idx.topk_indices_buffer[:t].view(t, 1, topk).cpu()
+
+    q_c = torch.nn.functional.rms_norm((x.float() @ wq_a.float()).bfloat16().float(), (q_lora,), w["q_norm"].float(),
+                                       EPS).bfloat16()
+    q = (q_c.float() @ w["q_b"].float()).bfloat16().view(t, n, 192)
+    kv = (x.float() @ wkv_a.float()).bfloat16()
+    kv_a = O.rms_norm(kv[:, :512], w["kv_norm"], EPS)
+    k_pe = O.interleave_rope(kv[:, 512:], cos, sin)
+    q_pe = O.interleave_rope(q[..., 128:], cos, sin)
+    sm = common.slot_mapping.cpu()
+    O.cache_write(nope, sm, kv_a); O.cache_write(rope, sm, k_pe)
+    ql = O.q_absorb(q[..., :128], impl.W_UK_T.cpu())
+    attn_ref = torch.zeros(t, n * 128)
+    tok = 0
+    for b, (qlen, L) in enumerate(zip(q_lens, seq_lens)):
+        for i in range(qlen):
+            vis = L - qlen + i + 1
+            valid = sel[tok, 0][sel[tok, 0] >= 0]
+            assert valid.numel() == min(topk, vis) and int(valid.max()) < vis
+            o = O.sparse_decode(ql[tok:tok + 1].bfloat16(), q_pe[tok:tok + 1], nope, rope,
+                                common.block_table_tensor[b:b + 1].cpu(), [vis], sel[tok:tok + 1], impl.scale)
+            attn_ref[tok] = O.v_up_proj(o.transpose(0, 1).contiguous().bfloat16(), impl.W_UV.cpu()).view(-1)
+            tok += 1
+    ref = attn_ref.bfloat16().float() @ w["o"].float()
+    err = (out.float().cpu() - ref).abs().max().item()
+    assert err <= 3e-2 * ref.abs().max().item(), f"max err {err:.4g} vs scale {ref.abs().max().item():.4g}"
+    with V.set_forward_context(attn_metadata=None):
+        dry = mod(x.to(dev), cd, sd)
+    assert dry.shape == (t, hidden) and float(dry.abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("variant", ["positions", "tables"])
 def test_indexer_module_selects_what_the_oracle_selects(dev, variant):
     """``positions``: the patched module (patch_dsv32_indexer.py:77-146, rotary module, interleaved pairs); ``tables``:
