@@ -307,3 +307,47 @@ def test_default_split_count_is_a_function_of_shapes_only():
         for l in (1, 255, 256, 257, 10 ** 6):
             s = K.default_num_splits(b, 1, 128, l)
             assert 1 <= s <= 256 and (s == 1 or l / s >= 128)
+
+
+# ---- the custom-model modules: routing (reference tests/unit/layers/test_npu_dsa.py:242-295) -----------------------
+def _custom_module(cls, **extra):
+    norm = SimpleNamespace(weight=torch.ones(512), variance_epsilon=1e-6)
+    attn = SimpleNamespace(layer_name="model.layers.3.self_attn.attn", impl=None, kv_cache=[None])
+    lin = lambda x: (x, None)
+    return cls(256, 16, 128, 64, 128, 128, 512, attn, *extra.values(), lin, lin, lin, lin, norm, lin,
+               prefix="model.layers.3.self_attn"), attn
+
+
+def test_custom_model_mla_module_routes_by_metadata(monkeypatch):
+    from omni_npu_amd.v1.layers.attention import NPUDeepseekMLAAttention
+    mod, attn = _custom_module(NPUDeepseekMLAAttention)
+    seen = []
+    monkeypatch.setattr(mod, "_forward_prefill", lambda h, c, s, ctx, meta: seen.append(("prefill", meta)) or "p")
+    monkeypatch.setattr(mod, "_forward_decode", lambda h, c, s, ctx, meta: seen.append(("decode", meta)) or "d")
+    x = torch.zeros(2, 256)
+    with V.set_forward_context(attn_metadata=None):                                    # profile run -> prefill branch
+        assert mod(x, None, None) == "p" and seen[-1] == ("prefill", None)
+    pre = SimpleNamespace(prefill=object(), decode=None)
+    dec = SimpleNamespace(prefill=None, decode=object())
+    with V.set_forward_context(attn_metadata={attn.layer_name: pre, "other": dec}):     # dict: looked up by layer name
+        assert mod(x, None, None) == "p" and seen[-1] == ("prefill", pre)
+    with V.set_forward_context(attn_metadata=dec):
+        assert mod(x, None, None) == "d" and seen[-1] == ("decode", dec)
+    with V.set_forward_context(attn_metadata=SimpleNamespace(prefill=object(), decode=object())):
+        with pytest.raises(NotImplementedError):
+            mod(x, None, None)
+
+
+def test_custom_model_modules_need_a_norm_with_parameters():
+    from omni_npu_amd.v1.layers.attention import NPUDeepseekMLAAttention, NPUDeepseekSparseAttention
+    lin = lambda x: (x, None)
+    attn = SimpleNamespace(layer_name="l", impl=None, kv_cache=[None])
+    with pytest.raises(TypeError):
+        NPUDeepseekMLAAttention(256, 16, 128, 64, 128, 128, 512, attn, lin, lin, lin, lin, lambda v: v, lin)
+    with pytest.raises(TypeError):
+        NPUDeepseekSparseAttention(256, 16, 128, 64, 128, 128, 512, attn, None, lin, lin, lin, lin, lambda v: v, lin)
+    mod = NPUDeepseekSparseAttention(256, 16, 128, 64, 128, 128, 512, attn, None, lin, lin, lin, lin,
+                                     SimpleNamespace(weight=torch.ones(512), eps=1e-6), lin)
+    with V.set_forward_context(attn_metadata=SimpleNamespace(prefill=object(), decode=object())):
+        with pytest.raises(NotImplementedError):
+            mod(torch.zeros(2, 256), None, None)
