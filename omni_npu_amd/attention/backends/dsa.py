@@ -148,6 +148,11 @@ class LightningIndexer:
                  device=None):
         self.topk_tokens, self.n_head, self.head_dim = topk_tokens, n_head, head_dim
         self.topk_indices_buffer = torch.full((max_tokens, topk_tokens), -1, dtype=torch.int32, device=device)
+        # what the sparse attention reads: the picks as flat cache rows and their number per token, written by the same
+        # launch that writes the positions (the block ids of the three DSA cache tensors are the same)
+        self.rows_buffer = torch.zeros((max_tokens, topk_tokens), dtype=torch.int32, device=device)
+        self.counts_buffer = torch.zeros((max_tokens,), dtype=torch.int32, device=device)
+        self._rows_meta = None       # the metadata object the row buffers were filled for
         self._logits = None
         self._logits_kept = []       # outgrown score buffers: a captured graph may still hold their address, never freed
 
@@ -186,9 +191,18 @@ class LightningIndexer:
             sl = slice(off, off + ntok)
             K.indexer_scores(q8[sl], w[sl], k8, ks, meta.block_table, lens, lg, q_len=q_len, q_scale=qs[sl],
                              query_start_loc=qsl, max_seq_len=max_len)
-            K.topk(lg, lens, self.topk_tokens, out[sl], q_len=q_len, query_start_loc=qsl)
+            K.topk(lg, lens, self.topk_tokens, out[sl], q_len=q_len, query_start_loc=qsl, block_table=meta.block_table,
+                   page_size=k8.shape[1], num_pages=k8.shape[0], rows=self.rows_buffer[sl], counts=self.counts_buffer[sl])
             off += ntok
+        self._rows_meta = attn_metadata
         return out.view(t, 1, self.topk_tokens)
+
+    def rows_for(self, attn_metadata):
+        """(cache rows [max_tokens, k], counts [max_tokens]) of the picks if the last selection ran for this very metadata
+        object, else None (the caller then translates ``topk_indices_buffer`` itself)."""
+        if attn_metadata is not None and self._rows_meta is attn_metadata:
+            return self.rows_buffer, self.counts_buffer
+        return None
 
 
 class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
@@ -236,17 +250,21 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
                 and out.dtype == torch.bfloat16 and out.stride(-1) == 1 and out.stride(0) % 4 == 0 and out.data_ptr() % 8 == 0)
 
     def _apply_sparse_attention(self, q_nope, q_pe, kv_cache, meta, lens, q_len, qsl, topk_indices,
-                                proj_out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+                                proj_out: Optional[torch.Tensor] = None, rows_counts=None) -> Optional[torch.Tensor]:
         """Absorbed MLA over the indexer's positions (reference dsa.py:259-291); token-major [T,N,512].  With
         ``proj_out`` ([T, N*V]) the value up-projection (dsa.py:233-240) is fused into the merge of the partials and
-        nothing is returned."""
+        nothing is returned.  ``rows_counts``: the picks of these tokens already translated into cache rows, with their
+        counts (LightningIndexer.rows_for); without it the positions are translated here."""
         bs = q_nope.shape[0]
         k = topk_indices.shape[-1]
         nope, rope = kv_cache[0], kv_cache[1]
-        rows = torch.empty(bs, k, dtype=torch.int32, device=q_nope.device)
-        counts = torch.empty(bs, dtype=torch.int32, device=q_nope.device)
-        K.build_sparse_rows(topk_indices.reshape(bs, k), meta.block_table, lens, nope.shape[1], nope.shape[0], rows, counts,
-                            q_len=q_len, query_start_loc=qsl)
+        if rows_counts is not None:
+            rows, counts = rows_counts
+        else:
+            rows = torch.empty(bs, k, dtype=torch.int32, device=q_nope.device)
+            counts = torch.empty(bs, dtype=torch.int32, device=q_nope.device)
+            K.build_sparse_rows(topk_indices.reshape(bs, k), meta.block_table, lens, nope.shape[1], nope.shape[0], rows,
+                                counts, q_len=q_len, query_start_loc=qsl)
         if proj_out is not None:
             K.sparse_decode(q_nope, q_pe, nope, rope, rows, counts, self.scale, proj_out, w_uv=self.W_UV, counts_bounded=True)
             return None
@@ -289,6 +307,9 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         ndt = attn_metadata.num_decode_tokens
         K.cache_write(k_c_normed, k_pe, attn_metadata.slot_mapping, k_nope, k_rope)
         topk = self.indexer.topk_indices_buffer
+        rows_for = getattr(self.indexer, "rows_for", None)
+        rc = rows_for(attn_metadata) if rows_for is not None else None
+        part = lambda a, b: None if rc is None else (rc[0][a:b], rc[1][a:b])
 
         if has_prefill:
             p = attn_metadata.prefill
@@ -297,7 +318,8 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
             fused = output[ndt:] if self._fusable_w_uv(output[ndt:]) else None
             attn_out = self._apply_sparse_attention(q_nope, q_pe, kv_cache, p, p.kv_lens, p.max_query_len,
                                                     p.query_start_loc.to(torch.int32).contiguous(),
-                                                    topk[ndt:num_actual_toks], proj_out=fused)
+                                                    topk[ndt:num_actual_toks], proj_out=fused,
+                                                    rows_counts=part(ndt, num_actual_toks))
             if fused is None:
                 self._v_up_proj(attn_out, out=output[ndt:])
         if has_decode:
@@ -306,7 +328,7 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
             q_nope, q_pe = self._absorb_prolog(q[:ndt])
             fused = output[:ndt] if self._fusable_w_uv(output[:ndt]) else None
             attn_out = self._apply_sparse_attention(q_nope, q_pe, kv_cache, d, d.seq_lens, d.q_len, d.query_start_loc,
-                                                    topk[:ndt], proj_out=fused)
+                                                    topk[:ndt], proj_out=fused, rows_counts=part(0, ndt))
             if fused is None:
                 self._v_up_proj(attn_out, out=output[:ndt])
         return output_padded

@@ -73,8 +73,10 @@ class NPUDeepseekSparseAttention(torch.nn.Module):
             d = meta.decode
             part, lens, q_len, qsl = d, d.seq_lens, d.q_len, d.query_start_loc
         fused = out if impl._fusable_w_uv(out) else None
+        select = getattr(self.indexer, "select", self.indexer)
+        rc = select.rows_for(meta) if hasattr(select, "rows_for") else None
         attn_out = impl._apply_sparse_attention(ql_nope, q_pe, kv_cache, part, lens, q_len, qsl, topk_indices[:t],
-                                                proj_out=fused)
+                                                proj_out=fused, rows_counts=None if rc is None else (rc[0][:t], rc[1][:t]))
         if fused is None:
             impl._v_up_proj(attn_out, out=out)
         return self.o_proj(out)[0]

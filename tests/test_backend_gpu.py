@@ -171,7 +171,14 @@ def test_dsa_impl_forward_with_indexer(dev):
     assert torch.equal(k8v.cpu()[sm // 128, sm % 128], k8_new.view(torch.uint8))
     assert torch.equal(ksv.cpu()[sm // 128, sm % 128], ks_new)
     out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    assert indexer.rows_for(meta) is not None and indexer.rows_for(object()) is None
     impl.forward(None, q.to(dev), kvc.to(dev), kpe.to(dev), kv_cache, meta, output=out)
+    # the same forward when the picks come without their cache rows (an indexer that only fills the index buffer): the
+    # positions are translated by a launch of their own, same result bit for bit
+    indexer._rows_meta = None
+    out2 = torch.zeros_like(out)
+    impl.forward(None, q.to(dev), kvc.to(dev), kpe.to(dev), kv_cache, meta, output=out2)
+    assert torch.equal(out, out2)
 
     # oracle: caches after the write, per-token visible length, sparse attention on the selected positions
     O.cache_write(nope, common.slot_mapping.cpu(), kvc); O.cache_write(rope, common.slot_mapping.cpu(), kpe.view(-1, 64))
