@@ -207,6 +207,7 @@ class LightningIndexer:
 
 class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
     can_return_lse_for_decode: bool = False
+    cache_written_for = None     # see NPUMLAImpl.cache_written_for
 
     def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: int, alibi_slopes: Optional[list],
                  sliding_window: Optional[int], kv_cache_dtype: str, logits_soft_cap: Optional[float], attn_type: str,
@@ -305,7 +306,9 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         has_decode = attn_metadata.num_decodes > 0
         has_prefill = attn_metadata.num_prefills > 0
         ndt = attn_metadata.num_decode_tokens
-        K.cache_write(k_c_normed, k_pe, attn_metadata.slot_mapping, k_nope, k_rope)
+        written, self.cache_written_for = self.cache_written_for is attn_metadata, None
+        if not written:                                            # (else the caller's fused norm + rope launch wrote them)
+            K.cache_write(k_c_normed, k_pe, attn_metadata.slot_mapping, k_nope, k_rope)
         topk = self.indexer.topk_indices_buffer
         rows_for = getattr(self.indexer, "rows_for", None)
         rc = rows_for(attn_metadata) if rows_for is not None else None

@@ -163,6 +163,9 @@ class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
 
 class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
     can_return_lse_for_decode: bool = True
+    # Set by a caller whose fused norm + rope launch has already written the step's rows into the cache: the metadata
+    # object of that step.  forward() then skips its own write once and clears the mark.
+    cache_written_for = None
 
     def __init__(self, num_heads: int, head_size: int, scale: float, num_kv_heads: int,
                  alibi_slopes: Optional[list], sliding_window: Optional[int], kv_cache_dtype: str,
@@ -403,8 +406,12 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         num_decode_tokens = attn_metadata.num_decode_tokens
         decode_q = q[:num_decode_tokens]
 
-        # write the latent and rope rows of the new tokens (one launch)
-        if self.fp8_cache:
+        # write the latent and rope rows of the new tokens (one launch), unless the caller's fused norm + rope launch has
+        # put them there already and said so for this very metadata object
+        written, self.cache_written_for = self.cache_written_for is attn_metadata, None
+        if written:
+            pass
+        elif self.fp8_cache:
             K.cache_write_fp8(k_c_normed, k_pe, attn_metadata.slot_mapping, kv_cache[0])
         else:
             K.cache_write(k_c_normed, k_pe, attn_metadata.slot_mapping, kv_cache[0], kv_cache[1])

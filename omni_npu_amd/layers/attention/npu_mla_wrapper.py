@@ -4,8 +4,9 @@ Mirrors ``NPUMultiHeadLatentAttentionWrapper.forward_oot`` (src/omni_npu/layers/
 attention layer it calls (``self.mla_attn``: the kv cache is ``kv_cache[forward_context.virtual_engine]``, the metadata
 ``forward_context.attn_metadata[layer_name]``, src/omni_npu/v1/layers/attention/npu_mla.py:159-162, 176).  The projection
 modules are the caller's (any callable returning ``(tensor, bias)`` like vLLM's linear layers: library GEMMs, as in the
-reference); what this file adds on the GPU side is that the RMSNorm of the compressed KV and the rotary embedding of the
-shared rope key run as ONE kernel when the norm and the rotary module expose their parameters."""
+reference); what this file adds on the GPU side is that the RMSNorm of the compressed KV, the rotary embedding of the
+shared rope key and the write of both into the paged cache run as ONE kernel when the norm and the rotary module expose
+their parameters (the backend impl is told, through ``cache_written_for``, that the rows of this step are in place)."""
 from __future__ import annotations
 
 from typing import Any, Optional
@@ -59,13 +60,35 @@ class NPUMultiHeadLatentAttentionWrapper(torch.nn.Module):
                 and kv_lora.dtype == torch.bfloat16 and kv_lora.shape[-1] == K.D_NOPE + K.D_ROPE:
             t = kv_lora.shape[0]
             cos, sin = rope.get_cos_sin(positions)
-            kv_c_normed = torch.empty(t, K.D_NOPE, dtype=kv_lora.dtype, device=kv_lora.device)
-            k_pe = torch.empty(t, K.D_ROPE, dtype=kv_lora.dtype, device=kv_lora.device)
-            K.kv_rmsnorm_rope_cache(kv_lora, norm.weight, cos, sin, None, None, None, eps=eps, kv_a_out=kv_c_normed,
+            kv_c_normed = torch.zeros(t, K.D_NOPE, dtype=kv_lora.dtype, device=kv_lora.device)
+            k_pe = torch.zeros(t, K.D_ROPE, dtype=kv_lora.dtype, device=kv_lora.device)
+            slots, nope_c, rope_c = self._cache_target()
+            K.kv_rmsnorm_rope_cache(kv_lora, norm.weight, cos, sin, slots, nope_c, rope_c, eps=eps, kv_a_out=kv_c_normed,
                                     k_pe_out=k_pe)
             return kv_c_normed, k_pe.unsqueeze(1), (cos, sin)
         kv_c, k_pe = kv_lora.split([self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
         return norm(kv_c), k_pe.unsqueeze(1), None
+
+    def _cache_target(self):
+        """Where the fused launch may also write the new tokens' cache rows: (slot_mapping, latent cache, rope cache or
+        None for the fp8 cache) when the step has metadata, the layer a cache, every token a slot, and the backend impl
+        agrees to skip its own write for this metadata object; (None, None, None) otherwise."""
+        impl = getattr(self.mla_attn, "impl", None)
+        if impl is None or not hasattr(impl, "cache_written_for"):
+            return None, None, None
+        ctx = V.get_forward_context()
+        meta = ctx.attn_metadata
+        if isinstance(meta, dict):
+            meta = meta.get(self.mla_attn.layer_name)
+        kv_cache = self.mla_attn.kv_cache[ctx.virtual_engine]
+        if meta is None or kv_cache is None or getattr(meta, "slot_mapping", None) is None:
+            return None, None, None
+        if meta.slot_mapping.numel() < meta.num_actual_tokens:
+            return None, None, None
+        impl.cache_written_for = meta
+        if getattr(impl, "fp8_cache", False):
+            return meta.slot_mapping, kv_cache[0], None
+        return meta.slot_mapping, kv_cache[0], kv_cache[1]
 
     def forward_oot(self, positions: torch.Tensor, hidden_states: torch.Tensor,
                     llama_4_scaling: Optional[torch.Tensor] = None) -> torch.Tensor:

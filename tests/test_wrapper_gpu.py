@@ -47,7 +47,7 @@ def _weights(g, hidden, n, q_lora):
 @pytest.mark.parametrize("q_lens,seq_lens,fused", [([1] * 6, [200, 31, 129, 500, 64, 1000], True),
                                                    ([1, 1, 24], [300, 77, 24], True),
                                                    ([2, 2], [150, 400], False)])
-def test_forward_oot_matches_fp32_chain(dev, q_lens, seq_lens, fused):
+def test_forward_oot_matches_fp32_chain(dev, monkeypatch, q_lens, seq_lens, fused):
     from omni_npu_amd.layers.attention.npu_mla_wrapper import MLAAttention, NPUMultiHeadLatentAttentionWrapper
     from omni_npu_amd.layers.rotary_embedding import HIPRotaryEmbedding
     g = torch.Generator().manual_seed(sum(seq_lens))
@@ -91,9 +91,15 @@ def test_forward_oot_matches_fp32_chain(dev, q_lens, seq_lens, fused):
     ref = attn_ref.bfloat16().float() @ w["o"].float()
 
     meta = builder.build(0, _to(common, dev))
+    from omni_npu_amd import kernels as K
+    writes = []
+    real_write = K.cache_write
+    monkeypatch.setattr(K, "cache_write", lambda *a, **k: writes.append(1) or real_write(*a, **k))
     with V.set_forward_context(attn_metadata={attn.layer_name: meta}):
         out = wrap.forward_oot(positions.to(dev), x.to(dev))
     assert out.shape == (t, hidden)
+    # fused path: the norm + rope launch wrote the cache rows and the impl skipped its own write; two-module path: the impl's
+    assert len(writes) == (0 if fused else 1) and impl.cache_written_for is None
     err = (out.float().cpu() - ref).abs().max().item()
     assert err <= 3e-2 * ref.abs().max().item(), f"max err {err:.4g} vs scale {ref.abs().max().item():.4g}"
     # the cache rows of the new tokens hold the normalised latent and the rotated key (to the last bf16 bit but one)
