@@ -668,6 +668,120 @@ def bench_epilogue(K, dev, args):
     }
 
 
+def bench_layer(K, dev, args):
+    """The attention part of one decode layer the way the backend runs it (the classes a vLLM worker would call, on the
+    headline shape): fused RMSNorm + rotary embedding + cache write of the new tokens, rotary embedding of the query,
+    then ``NPUMLAImpl.forward`` = absorption GEMM, split-KV kernel, merge fused with the value up-projection into the
+    layer's [T, N*128] output.  Timed as queued eager launches and as HIP-graph replays."""
+    import time
+    from types import SimpleNamespace
+    from oracle import mla_oracle as O
+    from omni_npu_amd import _vllm_compat as V
+    from omni_npu_amd.attention.backends import mla
+    B, N, EPS = args.batch, args.heads, 1e-6
+    case = build_workload(args.seed, B, N, args.len_lo, args.len_hi, 1)
+    lens = case["seq_lens"]
+    gen = torch.Generator().manual_seed(args.seed + 7)
+    w_kv_b = (torch.randn(512, N * 256, generator=gen) * 0.05).bfloat16()
+    q = torch.randn(B, N, 192, generator=gen).bfloat16()
+    kv = torch.randn(B, 576, generator=gen).bfloat16()
+    gamma = (1 + 0.1 * torch.randn(512, generator=gen)).bfloat16()
+    cos, sin = O.rope_tables(lens.long() - 1)
+    impl = mla.NPUMLAImpl(num_heads=N, head_size=576, scale=192 ** -0.5, num_kv_heads=1, alibi_slopes=None,
+                          sliding_window=None, kv_cache_dtype="auto", logits_soft_cap=None,
+                          attn_type=V.AttentionType.DECODER, kv_sharing_target_layer_name=None, q_lora_rank=None,
+                          kv_lora_rank=512, qk_nope_head_dim=128, qk_rope_head_dim=64, qk_head_dim=192, v_head_dim=128,
+                          kv_b_proj=lambda x: (x @ w_kv_b.to(x.device),))
+    kvw = w_kv_b.view(512, N, 256)
+    impl.W_UK_T = kvw[..., :128].permute(1, 2, 0).contiguous().to(dev)
+    impl.W_UV = kvw[..., 128:].transpose(0, 1).contiguous().to(dev)
+    qsl = torch.arange(B + 1, dtype=torch.int32)
+    common = V.CommonAttentionMetadata(
+        query_start_loc=qsl.to(dev), query_start_loc_cpu=qsl.clone(), seq_lens=lens.to(dev), seq_lens_cpu=lens.clone(),
+        num_computed_tokens_cpu=lens - 1, num_reqs=B, num_actual_tokens=B, max_query_len=1, max_seq_len=int(lens.max()),
+        block_table_tensor=case["block_table"].to(dev), slot_mapping=case["slot_mapping"].to(dev))
+    cfg = SimpleNamespace(
+        scheduler_config=SimpleNamespace(max_num_seqs=B), model_config=SimpleNamespace(max_model_len=16384, dtype=torch.bfloat16),
+        cache_config=SimpleNamespace(block_size=128, cache_dtype="auto"),
+        parallel_config=SimpleNamespace(cp_kv_cache_interleave_size=1, decode_context_parallel_size=1, worker_cls=None),
+        compilation_config=SimpleNamespace(max_cudagraph_capture_size=B, pass_config=None), kv_transfer_config=None,
+        speculative_config=None)
+    builder = mla.NPUMLAMetadataBuilder(V.AttentionSpec(128, 1, 576, torch.bfloat16), ["layer"], cfg, dev)
+    meta = builder.build(0, common)
+    nope, rope = case["nope"].to(dev), case["rope"].to(dev)
+    d_q, d_kv, d_gamma, d_cos, d_sin = (x.to(dev) for x in (q, kv, gamma, cos, sin))
+    kvc = torch.empty(B, 512, dtype=torch.bfloat16, device=dev)
+    kpe = torch.empty(B, 64, dtype=torch.bfloat16, device=dev)
+    q_in = d_q.clone()
+    out = torch.zeros(B, N * 128, dtype=torch.bfloat16, device=dev)
+
+    def layer():
+        K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, nope, rope, eps=EPS, kv_a_out=kvc, k_pe_out=kpe)
+        q_in[..., 128:] = K.interleave_rope(d_q[..., 128:], d_cos, d_sin, table="half")
+        impl.cache_written_for = meta
+        impl.forward(None, q_in, kvc, kpe.unsqueeze(1), (nope, rope), meta, output=out)
+
+    def timed(fn, n):
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(e) * 1e3 / n
+
+    clock_ramp(layer)
+    for _ in range(args.warmup):
+        layer()
+    t_eager = sorted(timed(layer, args.steps) for _ in range(3))[1]
+    reps = 10
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        layer()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(reps):
+                layer()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        graph.replay()
+    t_graph = sorted(timed(graph.replay, max(1, args.steps // reps)) for _ in range(3))[1] / reps
+
+    # oracle chain on the host for a sample of sequences
+    sample = min(8, B)
+    cpu_info = cpu_fields()
+    t0 = time.perf_counter()
+    kv_a = O.rms_norm(kv[:, :512], gamma, EPS)
+    k_pe = O.interleave_rope(kv[:, 512:], cos, sin)
+    c_nope, c_rope = case["nope"].clone(), case["rope"].clone()
+    O.cache_write(c_nope, case["slot_mapping"], kv_a)
+    O.cache_write(c_rope, case["slot_mapping"], k_pe)
+    q_pe = O.interleave_rope(q[:sample, :, 128:], cos[:sample], sin[:sample])
+    ql = O.q_absorb(q[:sample, :, :128], impl.W_UK_T.cpu()).bfloat16()
+    ref_o = O.absorbed_decode(ql, q_pe, c_nope, c_rope, case["block_table"][:sample], lens[:sample], impl.scale)
+    ref = O.v_up_proj(ref_o.transpose(0, 1).contiguous().bfloat16(), impl.W_UV.cpu()).view(sample, -1)
+    cpu_s = time.perf_counter() - t0
+    err = (out[:sample].float().cpu() - ref.float()).abs().max().item()
+    alg = algorithmic_bytes(case, N)
+    alg_bytes = alg["kv"] + alg["cache_write"] + alg["tables"] + B * N * (192 + 128) * 2 + 2 * N * 128 * 512 * 2
+    return {
+        "metric": f"MLA decode attention of one layer through the backend classes, us/layer (B={B}, ctx {args.len_lo // 1024}k-{args.len_hi // 1024}k, {N} heads)",
+        "value": round(t_eager, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1] through NPUMLAMetadataBuilder + NPUMLAImpl.forward: norm + rope + cache write, "
+                               "query rope, absorption GEMM, split-KV decode, merge + W_UV", "batch": B, "heads": N,
+                   "sum_seq_len": int(lens.sum()), "seed": args.seed},
+        "layer_us": {"eager_launches_queued": round(t_eager, 2), "hip_graph_replay": round(t_graph, 2)},
+        "roofline": {"kernel": "whole layer", "bound": "hbm", "achieved": round(alg_bytes / t_eager / 1e3, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(alg_bytes / t_eager / 1e3 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "algorithmic_bytes": alg_bytes},
+        "cpu_baseline": {"value": round(cpu_s * B / sample * 1e6, 1), "unit": "us/layer", **cpu_info, "kind": "port",
+                         "sample": f"oracle chain (torch fp32) of {sample} of {B} sequences, scaled by sequence count",
+                         "gpu_vs_oracle_max_abs": err},
+    }
+
+
 def bench_window(K, dev, args):
     """Decode with static sink tokens and a sliding window (the reference's variant of attention/backends/mla.py:705-779):
     B=64, 128 heads, 4096-8192 keys behind a 128-key sink, window 4096.  One step = window plan + dense split kernel over
@@ -763,8 +877,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue", "window"],
-                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue", "window", "layer"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel; layer = the attention part of a decode layer through the backend classes (NPUMLAMetadataBuilder + NPUMLAImpl.forward with the fused steps around it)")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -800,6 +914,9 @@ def main():
         return
     if args.workload == "window":
         print(json.dumps(bench_window(K, dev, args)))
+        return
+    if args.workload == "layer":
+        print(json.dumps(bench_layer(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len
