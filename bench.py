@@ -717,7 +717,7 @@ def bench_layer(K, dev, args):
 
     def layer():
         K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, nope, rope, eps=EPS, kv_a_out=kvc, k_pe_out=kpe)
-        q_in[..., 128:] = K.interleave_rope(d_q[..., 128:], d_cos, d_sin, table="half")
+        K.interleave_rope(d_q[..., 128:], d_cos, d_sin, out=q_in[..., 128:], table="half")
         impl.cache_written_for = meta
         impl.forward(None, q_in, kvc, kpe.unsqueeze(1), (nope, rope), meta, output=out)
 

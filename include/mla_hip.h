@@ -87,7 +87,7 @@ int mla_kv_rmsnorm_rope_cache_fp8(const void* kv_a, int64_t kv_a_stride, const v
 
 /* Replaces torch_npu.npu_interleave_rope (npu_mla.py:210, 316; npu_dsa.py:407, 528) for the query's rope part:
  * x [T, N, 64] through its strides -> out [T, N, 64], same rotation and table conventions as above.  In place
- * (out == x) only with interleaved_out = 1. */
+ * (out == x with the same strides) is allowed. */
 int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_stride_h, int64_t num_tokens, int32_t num_heads,
                         const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, int32_t interleaved_out,
                         void* out, int64_t out_stride_t, int64_t out_stride_h, mlahip_stream_t stream);

@@ -268,9 +268,10 @@ extern "C" int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_
   MLA_REQUIRE(x_stride_t % 8 == 0 && x_stride_h % 8 == 0 && out_stride_t % 8 == 0 && out_stride_h % 8 == 0 &&
                   (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0,
               MLA_ERR_SHAPE, "mla_interleave_rope: rows must be 16-byte aligned");
-  // in place is fine only when a thread's reads and writes cover the same bytes
-  MLA_REQUIRE(x != out || interleaved_out, MLA_ERR_UNSUPPORTED,
-              "mla_interleave_rope: the de-interleaved output cannot be written in place");
+  // In place (out == x, same strides) is fine in both output layouts: the eight threads of a row are neighbouring lanes
+  // of one wavefront, whose load instruction has returned for all of them before its store instruction is issued.
+  MLA_REQUIRE(x != out || (x_stride_t == out_stride_t && x_stride_h == out_stride_h), MLA_ERR_UNSUPPORTED,
+              "mla_interleave_rope: in place needs the same strides for x and out");
   if (num_tokens == 0) return MLA_OK;
   RopeParams p;
   p.x = (const __bf16*)x; p.x_st = x_stride_t; p.x_sh = x_stride_h; p.out = (__bf16*)out; p.o_st = out_stride_t;

@@ -111,7 +111,7 @@ class NPUMultiHeadLatentAttentionWrapper(torch.nn.Module):
         kv_c_normed, k_pe, cos_sin = self._kv_norm_rope(positions, kv_lora)
         if self.rotary_emb is not None:
             if cos_sin is not None:                            # k_pe is rotated already: only the query is left
-                q[..., self.qk_nope_head_dim:] = K.interleave_rope(q[..., self.qk_nope_head_dim:], *cos_sin, table="half")
+                K.interleave_rope(q[..., self.qk_nope_head_dim:], *cos_sin, out=q[..., self.qk_nope_head_dim:], table="half")
             else:
                 q[..., self.qk_nope_head_dim:], k_pe = self.rotary_emb(positions, q[..., self.qk_nope_head_dim:], k_pe)
 

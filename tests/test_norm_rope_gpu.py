@@ -129,13 +129,9 @@ def test_query_rope_strided_and_in_place(dev, layout, interleaved):
     qd = q.to(dev)
     got = K.interleave_rope(qd[..., 128:], cos.to(dev), sin.to(dev), table=layout, interleaved_out=interleaved)
     _ulp_close(got, want)
-    if interleaved:
-        K.interleave_rope(qd[..., 128:], cos.to(dev), sin.to(dev), out=qd[..., 128:], table=layout, interleaved_out=True)
-        assert torch.equal(qd[..., 128:], got) and torch.equal(qd[..., :128].cpu(), q[..., :128])
-    else:
-        from omni_npu_amd._lib import MlaHipError
-        with pytest.raises(MlaHipError):
-            K.interleave_rope(qd[..., 128:], cos.to(dev), sin.to(dev), out=qd[..., 128:], table=layout)
+    # in place, in either output layout: the rope part of the query is rotated where it lies
+    K.interleave_rope(qd[..., 128:], cos.to(dev), sin.to(dev), out=qd[..., 128:], table=layout, interleaved_out=interleaved)
+    assert torch.equal(qd[..., 128:], got) and torch.equal(qd[..., :128].cpu(), q[..., :128])
 
 
 @pytest.mark.parametrize("layout", ["half", "repeat"])
