@@ -716,8 +716,8 @@ def bench_layer(K, dev, args):
     out = torch.zeros(B, N * 128, dtype=torch.bfloat16, device=dev)
 
     def layer():
-        K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, nope, rope, eps=EPS, kv_a_out=kvc, k_pe_out=kpe)
-        K.interleave_rope(d_q[..., 128:], d_cos, d_sin, out=q_in[..., 128:], table="half")
+        K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, nope, rope, eps=EPS, kv_a_out=kvc, k_pe_out=kpe,
+                                q_rope=d_q[..., 128:], q_out=q_in[..., 128:])
         impl.cache_written_for = meta
         impl.forward(None, q_in, kvc, kpe.unsqueeze(1), (nope, rope), meta, output=out)
 

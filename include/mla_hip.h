@@ -92,6 +92,27 @@ int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_stride_h, i
                         const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step, int32_t interleaved_out,
                         void* out, int64_t out_stride_t, int64_t out_stride_h, mlahip_stream_t stream);
 
+/* mla_kv_rmsnorm_rope_cache[_fp8] and mla_interleave_rope of the same tokens in ONE launch: the whole rotary / norm /
+ * cache-write prologue of a decode step (npu_mla.py:196-210: the reference issues the two vendor ops back to back).
+ * q [T, num_heads, 64] through its strides -> q_out (may be q itself, same strides); same tables and the same
+ * interleaved_out convention for the key and the query. */
+int mla_kv_rmsnorm_rope_cache_q(const void* kv_a, int64_t kv_a_stride, const void* k_pe, int64_t k_pe_stride,
+                                const void* gamma, const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step,
+                                int32_t interleaved_out, const int64_t* slot_mapping, int32_t num_tokens, float eps,
+                                void* nope_cache, int64_t nope_page_stride, int64_t nope_row_stride, void* rope_cache,
+                                int64_t rope_page_stride, int64_t rope_row_stride, int32_t page_size, int64_t num_pages,
+                                void* kv_a_out, int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride,
+                                const void* q, int64_t q_stride_t, int64_t q_stride_h, int32_t num_heads, void* q_out,
+                                int64_t q_out_stride_t, int64_t q_out_stride_h, mlahip_stream_t stream);
+int mla_kv_rmsnorm_rope_cache_q_fp8(const void* kv_a, int64_t kv_a_stride, const void* k_pe, int64_t k_pe_stride,
+                                    const void* gamma, const void* cos, const void* sin, int64_t cs_stride,
+                                    int32_t cos_step, int32_t interleaved_out, const int64_t* slot_mapping,
+                                    int32_t num_tokens, float eps, void* cache, int64_t page_stride_bytes,
+                                    int64_t row_stride_bytes, int32_t page_size, int64_t num_pages, void* kv_a_out,
+                                    int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride, const void* q,
+                                    int64_t q_stride_t, int64_t q_stride_h, int32_t num_heads, void* q_out,
+                                    int64_t q_out_stride_t, int64_t q_out_stride_h, mlahip_stream_t stream);
+
 /* Replaces torch_npu.npu_rotary_mul as the indexer calls it (v1/layers/attention/npu_dsa.py:120, 130): the
  * half-rotation pairing, element i with element i + 32, out = cat(x1*c - x2*s, x2*c + x1*s) with x = cat(x1, x2)
  * (the neox branch of layers/rotary_embedding/rotary_embedding_torch_npu.py:146-163).  x [T, N, 64] through its

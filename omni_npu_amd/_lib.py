@@ -26,6 +26,10 @@ SIGNATURES = {
                                             I32, I64, P, I64, P, I64, P]),
     "mla_kv_rmsnorm_rope_cache_fp8": (c_int32, [P, I64, P, I64, P, P, P, I64, I32, I32, P, I32, F32, P, I64, I64, I32, I64,
                                                 P, I64, P, I64, P]),
+    "mla_kv_rmsnorm_rope_cache_q": (c_int32, [P, I64, P, I64, P, P, P, I64, I32, I32, P, I32, F32, P, I64, I64, P, I64, I64,
+                                              I32, I64, P, I64, P, I64, P, I64, I64, I32, P, I64, I64, P]),
+    "mla_kv_rmsnorm_rope_cache_q_fp8": (c_int32, [P, I64, P, I64, P, P, P, I64, I32, I32, P, I32, F32, P, I64, I64, I32,
+                                                  I64, P, I64, P, I64, P, I64, I64, I32, P, I64, I64, P]),
     "mla_interleave_rope": (c_int32, [P, I64, I64, I64, I32, P, P, I64, I32, I32, P, I64, I64, P]),
     "mla_rotary_mul": (c_int32, [P, I64, I64, I64, I32, P, P, I64, I32, P, I64, I64, P]),
     "mla_decode_fp8": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32, I32, I32, F32, P, I64,

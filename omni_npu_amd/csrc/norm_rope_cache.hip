@@ -57,9 +57,9 @@ __device__ __forceinline__ void rope4(const bf16x8& x, const __bf16* c, const __
 }
 
 template <bool kFp8>
-__global__ __launch_bounds__(256) void kv_rmsnorm_rope_cache_kernel(NormRopeParams p) {
+__device__ __forceinline__ void kv_norm_rope_body(const NormRopeParams& p, int64_t block) {
   const int lane = threadIdx.x & 63;
-  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t t = block * 4 + (threadIdx.x >> 6);
   if (t >= p.num_tokens) return;
   const int64_t slot = p.slots ? p.slots[t] : -1;
   const bool store = slot >= 0 && slot < p.num_pages * p.page_size;
@@ -129,6 +129,11 @@ __global__ __launch_bounds__(256) void kv_rmsnorm_rope_cache_kernel(NormRopePara
   }
 }
 
+template <bool kFp8>
+__global__ __launch_bounds__(256) void kv_rmsnorm_rope_cache_kernel(NormRopeParams p) {
+  kv_norm_rope_body<kFp8>(p, blockIdx.x);
+}
+
 struct RopeParams {
   const __bf16* x; int64_t x_st, x_sh;
   __bf16* out; int64_t o_st, o_sh;
@@ -137,8 +142,8 @@ struct RopeParams {
 };
 
 // One thread per (token, head, group of four pairs).
-__global__ __launch_bounds__(256) void interleave_rope_kernel(RopeParams p) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void interleave_rope_body(const RopeParams& p, int64_t block) {
+  const int64_t i = block * 256 + threadIdx.x;
   const int j = (int)(i & 7);
   const int64_t th = i >> 3;
   const int64_t t = th / p.num_heads;
@@ -157,6 +162,16 @@ __global__ __launch_bounds__(256) void interleave_rope_kernel(RopeParams p) {
     *(bf16x4*)(dst + j * 8) = o1;
     *(bf16x4*)(dst + 64 + j * 8) = o2;
   }
+}
+
+__global__ __launch_bounds__(256) void interleave_rope_kernel(RopeParams p) { interleave_rope_body(p, blockIdx.x); }
+
+// Both in one launch (the decode step's prologue: a handful of tokens, launch latency is all there is): the first
+// kv_blocks workgroups normalise, rotate and store the keys, the others rotate the query's rope part.
+template <bool kFp8>
+__global__ __launch_bounds__(256) void kv_q_prologue_kernel(NormRopeParams p, RopeParams q, int32_t kv_blocks) {
+  if ((int)blockIdx.x < kv_blocks) kv_norm_rope_body<kFp8>(p, blockIdx.x);
+  else interleave_rope_body(q, (int64_t)blockIdx.x - kv_blocks);
 }
 
 // Half-rotation ("neox") pairing: element i pairs with element i + 32, the result keeps the input's layout, so the
@@ -193,8 +208,10 @@ static int norm_rope_impl(bool fp8, const void* kv_a, int64_t kv_a_stride, const
                           int32_t interleaved_out, const int64_t* slot_mapping, int32_t num_tokens, float eps,
                           void* nope_cache, int64_t nope_sp_b, int64_t nope_sr_b, void* rope_cache, int64_t rope_sp_b,
                           int64_t rope_sr_b, int32_t page_size, int64_t num_pages, void* kv_a_out,
-                          int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride, hipStream_t stream) {
-  const char* who = fp8 ? "mla_kv_rmsnorm_rope_cache_fp8" : "mla_kv_rmsnorm_rope_cache";
+                          int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride, hipStream_t stream,
+                          const RopeParams* q = nullptr) {
+  const char* who = fp8 ? (q ? "mla_kv_rmsnorm_rope_cache_q_fp8" : "mla_kv_rmsnorm_rope_cache_fp8")
+                        : (q ? "mla_kv_rmsnorm_rope_cache_q" : "mla_kv_rmsnorm_rope_cache");
   // without a slot mapping nothing is cached: the normalised latent and the rotated key only go to the plain outputs
   MLA_REQUIRE(kv_a && k_pe && gamma && (slot_mapping ? (nope_cache && (fp8 || rope_cache)) : (kv_a_out && k_pe_out)),
               MLA_ERR_NULL, "%s: null pointer argument", who);
@@ -221,9 +238,38 @@ static int norm_rope_impl(bool fp8, const void* kv_a, int64_t kv_a_stride, const
   p.kv_a_out = (__bf16*)kv_a_out; p.kv_a_out_stride = kv_a_out_stride;
   p.k_pe_out = (__bf16*)k_pe_out; p.k_pe_out_stride = k_pe_out_stride;
   const dim3 grid((unsigned)((num_tokens + 3) / 4));
+  if (q) {
+    const int64_t q_blocks = (q->num_tokens * q->num_heads * 8 + 255) / 256;
+    MLA_REQUIRE((int64_t)grid.x + q_blocks < (1ll << 31), MLA_ERR_SHAPE, "%s: too many rows for one launch", who);
+    const dim3 both((unsigned)(grid.x + q_blocks));
+    if (fp8) hipLaunchKernelGGL(kv_q_prologue_kernel<true>, both, dim3(256), 0, stream, p, *q, (int32_t)grid.x);
+    else hipLaunchKernelGGL(kv_q_prologue_kernel<false>, both, dim3(256), 0, stream, p, *q, (int32_t)grid.x);
+    return check_launch(who);
+  }
   if (fp8) hipLaunchKernelGGL(kv_rmsnorm_rope_cache_kernel<true>, grid, dim3(256), 0, stream, p);
   else hipLaunchKernelGGL(kv_rmsnorm_rope_cache_kernel<false>, grid, dim3(256), 0, stream, p);
   return check_launch(who);
+}
+
+// Argument checks and parameters of the query rotation shared by mla_interleave_rope and the fused prologue entries.
+static int rope_params(const char* who, const void* x, int64_t x_stride_t, int64_t x_stride_h, int64_t num_tokens,
+                       int32_t num_heads, const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step,
+                       int32_t interleaved_out, void* out, int64_t out_stride_t, int64_t out_stride_h, RopeParams* p) {
+  MLA_REQUIRE(x && out, MLA_ERR_NULL, "%s: null pointer argument", who);
+  if (int rc = check_tables(who, cos, sin, cs_stride, cos_step)) return rc;
+  MLA_REQUIRE(num_tokens >= 0 && num_heads >= 1 && num_tokens * num_heads < (1ll << 40), MLA_ERR_SHAPE,
+              "%s: num_tokens=%lld num_heads=%d", who, (long long)num_tokens, num_heads);
+  MLA_REQUIRE(x_stride_t % 8 == 0 && x_stride_h % 8 == 0 && out_stride_t % 8 == 0 && out_stride_h % 8 == 0 &&
+                  (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0,
+              MLA_ERR_SHAPE, "%s: query rows must be 16-byte aligned", who);
+  // In place (out == x, same strides) is fine in both output layouts: the eight threads of a row are neighbouring lanes
+  // of one wavefront, whose load instruction has returned for all of them before its store instruction is issued.
+  MLA_REQUIRE(x != out || (x_stride_t == out_stride_t && x_stride_h == out_stride_h), MLA_ERR_UNSUPPORTED,
+              "%s: in place needs the same strides for x and out", who);
+  p->x = (const __bf16*)x; p->x_st = x_stride_t; p->x_sh = x_stride_h; p->out = (__bf16*)out; p->o_st = out_stride_t;
+  p->o_sh = out_stride_h; p->cos = (const __bf16*)cos; p->sin = (const __bf16*)sin; p->cs_stride = cs_stride;
+  p->cos_step = cos_step; p->num_tokens = num_tokens; p->num_heads = num_heads; p->interleaved_out = interleaved_out;
+  return MLA_OK;
 }
 
 }  // namespace mlahip
@@ -261,25 +307,54 @@ extern "C" int mla_interleave_rope(const void* x, int64_t x_stride_t, int64_t x_
                                    int32_t num_heads, const void* cos, const void* sin, int64_t cs_stride, int32_t cos_step,
                                    int32_t interleaved_out, void* out, int64_t out_stride_t, int64_t out_stride_h,
                                    hipStream_t stream) {
-  MLA_REQUIRE(x && out, MLA_ERR_NULL, "mla_interleave_rope: null pointer argument");
-  if (int rc = check_tables("mla_interleave_rope", cos, sin, cs_stride, cos_step)) return rc;
-  MLA_REQUIRE(num_tokens >= 0 && num_heads >= 1 && num_tokens * num_heads < (1ll << 40), MLA_ERR_SHAPE,
-              "mla_interleave_rope: num_tokens=%lld num_heads=%d", (long long)num_tokens, num_heads);
-  MLA_REQUIRE(x_stride_t % 8 == 0 && x_stride_h % 8 == 0 && out_stride_t % 8 == 0 && out_stride_h % 8 == 0 &&
-                  (uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0,
-              MLA_ERR_SHAPE, "mla_interleave_rope: rows must be 16-byte aligned");
-  // In place (out == x, same strides) is fine in both output layouts: the eight threads of a row are neighbouring lanes
-  // of one wavefront, whose load instruction has returned for all of them before its store instruction is issued.
-  MLA_REQUIRE(x != out || (x_stride_t == out_stride_t && x_stride_h == out_stride_h), MLA_ERR_UNSUPPORTED,
-              "mla_interleave_rope: in place needs the same strides for x and out");
-  if (num_tokens == 0) return MLA_OK;
   RopeParams p;
-  p.x = (const __bf16*)x; p.x_st = x_stride_t; p.x_sh = x_stride_h; p.out = (__bf16*)out; p.o_st = out_stride_t;
-  p.o_sh = out_stride_h; p.cos = (const __bf16*)cos; p.sin = (const __bf16*)sin; p.cs_stride = cs_stride;
-  p.cos_step = cos_step; p.num_tokens = num_tokens; p.num_heads = num_heads; p.interleaved_out = interleaved_out;
+  if (int rc = rope_params("mla_interleave_rope", x, x_stride_t, x_stride_h, num_tokens, num_heads, cos, sin, cs_stride,
+                           cos_step, interleaved_out, out, out_stride_t, out_stride_h, &p))
+    return rc;
+  if (num_tokens == 0) return MLA_OK;
   const int64_t threads = num_tokens * num_heads * 8;
   hipLaunchKernelGGL(interleave_rope_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, p);
   return check_launch("mla_interleave_rope");
+}
+
+// mla_kv_rmsnorm_rope_cache and mla_interleave_rope of the same tokens (same tables, same output convention) in one launch.
+extern "C" int mla_kv_rmsnorm_rope_cache_q(const void* kv_a, int64_t kv_a_stride, const void* k_pe, int64_t k_pe_stride,
+                                           const void* gamma, const void* cos, const void* sin, int64_t cs_stride,
+                                           int32_t cos_step, int32_t interleaved_out, const int64_t* slot_mapping,
+                                           int32_t num_tokens, float eps, void* nope_cache, int64_t nope_page_stride,
+                                           int64_t nope_row_stride, void* rope_cache, int64_t rope_page_stride,
+                                           int64_t rope_row_stride, int32_t page_size, int64_t num_pages, void* kv_a_out,
+                                           int64_t kv_a_out_stride, void* k_pe_out, int64_t k_pe_out_stride, const void* q,
+                                           int64_t q_stride_t, int64_t q_stride_h, int32_t num_heads, void* q_out,
+                                           int64_t q_out_stride_t, int64_t q_out_stride_h, hipStream_t stream) {
+  MLA_REQUIRE(nope_page_stride % 8 == 0 && nope_row_stride % 8 == 0 && rope_page_stride % 8 == 0 && rope_row_stride % 8 == 0,
+              MLA_ERR_SHAPE, "mla_kv_rmsnorm_rope_cache_q: cache rows must be 16-byte aligned");
+  RopeParams qp;
+  if (int rc = rope_params("mla_kv_rmsnorm_rope_cache_q", q, q_stride_t, q_stride_h, num_tokens, num_heads, cos, sin, cs_stride,
+                           cos_step, interleaved_out, q_out, q_out_stride_t, q_out_stride_h, &qp))
+    return rc;
+  return norm_rope_impl(false, kv_a, kv_a_stride, k_pe, k_pe_stride, gamma, cos, sin, cs_stride, cos_step, interleaved_out,
+                        slot_mapping, num_tokens, eps, nope_cache, nope_page_stride * 2, nope_row_stride * 2, rope_cache,
+                        rope_page_stride * 2, rope_row_stride * 2, page_size, num_pages, kv_a_out, kv_a_out_stride, k_pe_out,
+                        k_pe_out_stride, stream, &qp);
+}
+
+extern "C" int mla_kv_rmsnorm_rope_cache_q_fp8(const void* kv_a, int64_t kv_a_stride, const void* k_pe, int64_t k_pe_stride,
+                                               const void* gamma, const void* cos, const void* sin, int64_t cs_stride,
+                                               int32_t cos_step, int32_t interleaved_out, const int64_t* slot_mapping,
+                                               int32_t num_tokens, float eps, void* cache, int64_t page_stride_bytes,
+                                               int64_t row_stride_bytes, int32_t page_size, int64_t num_pages,
+                                               void* kv_a_out, int64_t kv_a_out_stride, void* k_pe_out,
+                                               int64_t k_pe_out_stride, const void* q, int64_t q_stride_t,
+                                               int64_t q_stride_h, int32_t num_heads, void* q_out, int64_t q_out_stride_t,
+                                               int64_t q_out_stride_h, hipStream_t stream) {
+  RopeParams qp;
+  if (int rc = rope_params("mla_kv_rmsnorm_rope_cache_q_fp8", q, q_stride_t, q_stride_h, num_tokens, num_heads, cos, sin,
+                           cs_stride, cos_step, interleaved_out, q_out, q_out_stride_t, q_out_stride_h, &qp))
+    return rc;
+  return norm_rope_impl(true, kv_a, kv_a_stride, k_pe, k_pe_stride, gamma, cos, sin, cs_stride, cos_step, interleaved_out,
+                        slot_mapping, num_tokens, eps, cache, page_stride_bytes, row_stride_bytes, nullptr, 0, 0, page_size,
+                        num_pages, kv_a_out, kv_a_out_stride, k_pe_out, k_pe_out_stride, stream, &qp);
 }
 
 extern "C" int mla_rotary_mul(const void* x, int64_t x_stride_t, int64_t x_stride_h, int64_t num_tokens, int32_t num_heads,

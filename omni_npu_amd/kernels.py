@@ -117,11 +117,14 @@ def kv_rmsnorm_rope_cache(kv: torch.Tensor, gamma: torch.Tensor, cos: torch.Tens
                           slot_mapping: Optional[torch.Tensor], nope_cache: Optional[torch.Tensor],
                           rope_cache: Optional[torch.Tensor],
                           eps: float = 1e-6, table: str = "half", interleaved_out: bool = False,
-                          kv_a_out: Optional[torch.Tensor] = None, k_pe_out: Optional[torch.Tensor] = None) -> None:
+                          kv_a_out: Optional[torch.Tensor] = None, k_pe_out: Optional[torch.Tensor] = None,
+                          q_rope: Optional[torch.Tensor] = None, q_out: Optional[torch.Tensor] = None) -> None:
     """RMSNorm(kv[:, :512]) * gamma and the rotary embedding of kv[:, 512:] written into the paged cache rows
     ``slot_mapping`` names, in one launch (reference: torch_npu.npu_kv_rmsnorm_rope_cache,
     src/omni_npu/v1/layers/attention/npu_mla.py:196-206).  ``rope_cache=None`` selects the fp8 cache
-    (``nope_cache`` = uint8 [num_blocks, page, 656]); ``slot_mapping=None`` caches nothing and only fills ``kv_a_out`` / ``k_pe_out``."""
+    (``nope_cache`` = uint8 [num_blocks, page, 656]); ``slot_mapping=None`` caches nothing and only fills ``kv_a_out`` / ``k_pe_out``.
+    ``q_rope`` (bf16 [T, N, 64], any strides with a contiguous last dim): the rotary embedding of the same tokens' query
+    heads (npu_interleave_rope, npu_mla.py:210) runs in the same launch, into ``q_out`` (default: in place)."""
     _need_cuda(kv, gamma, cos, sin, slot_mapping, nope_cache)
     lib = _lib.load()
     kv = kv.reshape(kv.shape[0], -1)
@@ -140,34 +143,47 @@ def kv_rmsnorm_rope_cache(kv: torch.Tensor, gamma: torch.Tensor, cos: torch.Tens
     outs = (kv_a_out.data_ptr() if kv_a_out is not None else None, kv_a_out.stride(0) if kv_a_out is not None else 0,
             k_pe_out.data_ptr() if k_pe_out is not None else None, k_pe_out.stride(0) if k_pe_out is not None else 0)
     k_pe = kv[:, D_NOPE:]
+    qargs, sfx = (), ""
+    if q_rope is not None:
+        _need_cuda(q_rope, q_out)
+        q_out = q_rope if q_out is None else q_out
+        if q_rope.dim() != 3 or q_rope.shape[0] < t or q_rope.shape[-1] != D_ROPE or q_rope.dtype != torch.bfloat16 \
+                or q_rope.stride(-1) != 1 or q_out.shape != q_rope.shape or q_out.dtype != q_rope.dtype or q_out.stride(-1) != 1:
+            raise ValueError("q_rope / q_out must be bf16 [T, N, 64] with a contiguous last dim")
+        qargs = (q_rope.data_ptr(), q_rope.stride(0), q_rope.stride(1), q_rope.shape[1], q_out.data_ptr(), q_out.stride(0),
+                 q_out.stride(1))
+        sfx = "_q"
     if slot_mapping is None:
         if kv_a_out is None or k_pe_out is None:
             raise ValueError("without a slot mapping both kv_a_out and k_pe_out are required")
-        rc = lib.mla_kv_rmsnorm_rope_cache(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
-                                           cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out), None, t,
-                                           float(eps), None, 0, 0, None, 0, 0, 1, 1, *outs, _stream(kv))
-        _lib.check(rc, "mla_kv_rmsnorm_rope_cache")
+        name = "mla_kv_rmsnorm_rope_cache" + sfx
+        rc = getattr(lib, name)(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
+                                cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out), None, t,
+                                float(eps), None, 0, 0, None, 0, 0, 1, 1, *outs, *qargs, _stream(kv))
+        _lib.check(rc, name)
         return
     if rope_cache is None:
         c = nope_cache
         if c.dtype != torch.uint8 or c.dim() != 3 or c.shape[-1] != FP8_ROW_BYTES or c.stride(-1) != 1:
             raise ValueError(f"fp8 cache must be uint8 [num_blocks, page, {FP8_ROW_BYTES}], got {c.dtype} {tuple(c.shape)}")
-        rc = lib.mla_kv_rmsnorm_rope_cache_fp8(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
-                                               cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out),
-                                               slot_mapping.data_ptr(), t, float(eps), c.data_ptr(), c.stride(0), c.stride(1),
-                                               c.shape[1], c.shape[0], *outs, _stream(kv))
-        _lib.check(rc, "mla_kv_rmsnorm_rope_cache_fp8")
+        name = "mla_kv_rmsnorm_rope_cache" + sfx + "_fp8"
+        rc = getattr(lib, name)(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
+                                cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out),
+                                slot_mapping.data_ptr(), t, float(eps), c.data_ptr(), c.stride(0), c.stride(1),
+                                c.shape[1], c.shape[0], *outs, *qargs, _stream(kv))
+        _lib.check(rc, name)
         return
     _need_cuda(rope_cache)
     nope, rope = _cache3(nope_cache, D_NOPE), _cache3(rope_cache, D_ROPE)
     if nope.dtype != torch.bfloat16 or rope.dtype != torch.bfloat16 or nope.shape[:2] != rope.shape[:2]:
         raise ValueError("nope / rope caches must be bf16 and agree on [num_blocks, page]")
-    rc = lib.mla_kv_rmsnorm_rope_cache(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
-                                       cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out),
-                                       slot_mapping.data_ptr(), t, float(eps), nope.data_ptr(), nope.stride(0), nope.stride(1),
-                                       rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[1], nope.shape[0], *outs,
-                                       _stream(kv))
-    _lib.check(rc, "mla_kv_rmsnorm_rope_cache")
+    name = "mla_kv_rmsnorm_rope_cache" + sfx
+    rc = getattr(lib, name)(kv.data_ptr(), kv.stride(0), k_pe.data_ptr(), kv.stride(0), gamma.data_ptr(),
+                            cos.data_ptr(), sin.data_ptr(), cos.stride(0), step, int(interleaved_out),
+                            slot_mapping.data_ptr(), t, float(eps), nope.data_ptr(), nope.stride(0), nope.stride(1),
+                            rope.data_ptr(), rope.stride(0), rope.stride(1), nope.shape[1], nope.shape[0], *outs, *qargs,
+                            _stream(kv))
+    _lib.check(rc, name)
 
 
 def interleave_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, out: Optional[torch.Tensor] = None,

@@ -52,8 +52,9 @@ class NPUMultiHeadLatentAttentionWrapper(torch.nn.Module):
         self.kv_a_proj_with_mqa, self.q_proj = kv_a_proj_with_mqa, q_proj
         self.indexer, self.is_sparse, self.indexer_rope_emb = indexer, is_sparse, indexer_rope_emb
 
-    def _kv_norm_rope(self, positions: torch.Tensor, kv_lora: torch.Tensor):
-        """kv_a_layernorm(kv_c) and rotary(k_pe): one fused launch when possible, the two modules otherwise."""
+    def _kv_norm_rope(self, positions: torch.Tensor, kv_lora: torch.Tensor, q: Optional[torch.Tensor] = None):
+        """kv_a_layernorm(kv_c) and rotary(k_pe): one fused launch when possible (which then also rotates the rope part
+        of ``q`` in place and writes the cache rows), the two modules otherwise."""
         norm, rope = self.kv_a_layernorm, self.rotary_emb
         eps = getattr(norm, "variance_epsilon", getattr(norm, "eps", None))
         if isinstance(rope, HIPRotaryEmbedding) and hasattr(norm, "weight") and eps is not None and kv_lora.is_cuda \
@@ -63,9 +64,12 @@ class NPUMultiHeadLatentAttentionWrapper(torch.nn.Module):
             kv_c_normed = torch.zeros(t, K.D_NOPE, dtype=kv_lora.dtype, device=kv_lora.device)
             k_pe = torch.zeros(t, K.D_ROPE, dtype=kv_lora.dtype, device=kv_lora.device)
             slots, nope_c, rope_c = self._cache_target()
+            q_rope = None
+            if q is not None and q.dtype == torch.bfloat16 and q.stride(-1) == 1 and q.shape[0] == t:
+                q_rope = q[..., self.qk_nope_head_dim:]
             K.kv_rmsnorm_rope_cache(kv_lora, norm.weight, cos, sin, slots, nope_c, rope_c, eps=eps, kv_a_out=kv_c_normed,
-                                    k_pe_out=k_pe)
-            return kv_c_normed, k_pe.unsqueeze(1), (cos, sin)
+                                    k_pe_out=k_pe, q_rope=q_rope)
+            return kv_c_normed, k_pe.unsqueeze(1), (cos, sin, q_rope is not None)
         kv_c, k_pe = kv_lora.split([self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
         return norm(kv_c), k_pe.unsqueeze(1), None
 
@@ -108,10 +112,12 @@ class NPUMultiHeadLatentAttentionWrapper(torch.nn.Module):
             q = self.q_proj(hidden_states)[0]
 
         q = q.view(-1, self.num_heads, self.qk_head_dim)
-        kv_c_normed, k_pe, cos_sin = self._kv_norm_rope(positions, kv_lora)
+        kv_c_normed, k_pe, cos_sin = self._kv_norm_rope(positions, kv_lora, q if self.rotary_emb is not None else None)
         if self.rotary_emb is not None:
-            if cos_sin is not None:                            # k_pe is rotated already: only the query is left
-                K.interleave_rope(q[..., self.qk_nope_head_dim:], *cos_sin, out=q[..., self.qk_nope_head_dim:], table="half")
+            if cos_sin is not None:                            # k_pe is rotated already, and q too unless it did not qualify
+                if not cos_sin[2]:
+                    K.interleave_rope(q[..., self.qk_nope_head_dim:], cos_sin[0], cos_sin[1],
+                                      out=q[..., self.qk_nope_head_dim:], table="half")
             else:
                 q[..., self.qk_nope_head_dim:], k_pe = self.rotary_emb(positions, q[..., self.qk_nope_head_dim:], k_pe)
 

@@ -52,19 +52,19 @@ class NPUDeepseekSparseAttention(torch.nn.Module):
         q = self.q_b_proj(q_lora)[0].view(-1, self.num_local_heads, self.qk_head_dim)
         t, dev = q.shape[0], q.device
         ql_nope = torch.bmm(q[..., :self.qk_nope_head_dim].transpose(0, 1), impl.W_UK_T).transpose(0, 1)
-        q_pe = K.interleave_rope(q[..., self.qk_nope_head_dim:], cos, sin, table="half")
+        q_pe = q[..., self.qk_nope_head_dim:]                   # rotated in place by the fused launches below
         out = torch.empty(t, self.num_local_heads * self.v_head_dim, dtype=q.dtype, device=dev)
         if meta is None:
             # memory-profiling run (:401-407, :317-324): norm and rope without a cache, zero attention output
             kv_a = torch.empty(t, self.kv_lora_rank, dtype=q.dtype, device=dev)
             k_pe = torch.empty(t, self.qk_rope_head_dim, dtype=q.dtype, device=dev)
             K.kv_rmsnorm_rope_cache(latent, self.kv_a_layernorm.weight, cos, sin, None, None, None, eps=self._eps(),
-                                    kv_a_out=kv_a, k_pe_out=k_pe)
+                                    kv_a_out=kv_a, k_pe_out=k_pe, q_rope=q_pe)
             return self.o_proj(out.fill_(0))[0]
         kv_cache = self.attn.kv_cache[ctx.virtual_engine]
         assert len(kv_cache) == 3, f"{len(kv_cache)=}."
         K.kv_rmsnorm_rope_cache(latent, self.kv_a_layernorm.weight, cos, sin, meta.slot_mapping, kv_cache[0], kv_cache[1],
-                                eps=self._eps())
+                                eps=self._eps(), q_rope=q_pe)
         topk_indices = self.indexer.forward_tables(hidden_states, q_lora, cos, sin, meta, kv_cache)[0]
         if meta.prefill is not None:
             p = meta.prefill

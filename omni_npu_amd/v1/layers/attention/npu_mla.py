@@ -6,8 +6,8 @@ either all decode (:169-242) or all prefill without cached context (:244-348, th
 prefill disabled).  The projection modules are the caller's (callables returning ``(tensor, bias)`` like vLLM's linear
 layers: library GEMMs, as in the reference).  On this side of the boundary:
 
-* decode: RMSNorm + rotary embedding + cache write is one launch (``npu_kv_rmsnorm_rope_cache``, :196-206), the query's
-  rotary embedding one (``npu_interleave_rope``, :210), the attention call (:213-232) is the split-KV kernel, and the
+* decode: RMSNorm + rotary embedding + cache write (``npu_kv_rmsnorm_rope_cache``, :196-206) and the query's rotary
+  embedding (``npu_interleave_rope``, :210) are one launch, the attention call (:213-232) is the split-KV kernel, and the
   ``W_UV`` product (:235-240) is fused into the merge of its partials;
 * prefill: the same fused launch also returns the normalised latent and the rotated key (``is_output_kv``, :296-309), the
   varlen kernel runs causally over the step's own tokens (:329-344).
@@ -77,8 +77,9 @@ class NPUDeepseekMLAAttention(torch.nn.Module):
         t = q.shape[0]
         # (N, T, P) @ W_UK_T (N, P, L) -> token-major [T, N, L]
         ql_nope = torch.bmm(q[..., :self.qk_nope_head_dim].transpose(0, 1), impl.W_UK_T).transpose(0, 1)
-        K.kv_rmsnorm_rope_cache(kv, self.kv_a_layernorm.weight, cos, sin, meta.slot_mapping, nope_c, rope_c, eps=self._eps())
-        q_pe = K.interleave_rope(q[..., self.qk_nope_head_dim:], cos, sin, table="half")
+        q_pe = q[..., self.qk_nope_head_dim:]                   # rotated in place by the launch that writes the cache
+        K.kv_rmsnorm_rope_cache(kv, self.kv_a_layernorm.weight, cos, sin, meta.slot_mapping, nope_c, rope_c, eps=self._eps(),
+                                q_rope=q_pe)
         out = torch.empty(t, self.num_local_heads * self.v_head_dim, dtype=q.dtype, device=q.device)
         impl._forward_decode(ql_nope, q_pe, kv_cache, meta, proj_out=out)
         return self.o_proj(out)[0]
@@ -97,9 +98,9 @@ class NPUDeepseekMLAAttention(torch.nn.Module):
             attn_output.fill_(0)
             return self.o_proj(attn_output.view(t, -1))[0]
         _, nope_c, rope_c = self._caches(ctx)
+        q_pe = q[..., self.qk_nope_head_dim:]
         K.kv_rmsnorm_rope_cache(kv, self.kv_a_layernorm.weight, cos, sin, meta.slot_mapping, nope_c, rope_c,
-                                eps=self._eps(), kv_a_out=kv_a, k_pe_out=k_pe)
-        q_pe = K.interleave_rope(q[..., self.qk_nope_head_dim:], cos, sin, table="half")
+                                eps=self._eps(), kv_a_out=kv_a, k_pe_out=k_pe, q_rope=q_pe)
         k_nope, v = impl._kv_up(kv_a)
         cu = meta.prefill.query_start_loc.to(torch.int32).contiguous()
         K.prefill_varlen(q[..., :self.qk_nope_head_dim], q_pe, k_nope, k_pe, v, cu, cu, meta.prefill.max_query_len,

@@ -134,6 +134,42 @@ def test_query_rope_strided_and_in_place(dev, layout, interleaved):
     assert torch.equal(qd[..., 128:], got) and torch.equal(qd[..., :128].cpu(), q[..., :128])
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_fused_prologue_with_query_equals_the_two_launches(dev, fp8):
+    """One launch for the key side (norm, rope, cache write, plain outputs) and the query's rope part, in place on a strided
+    view: the same bits as the two launches, in the caches, the plain outputs and the query."""
+    from omni_npu_amd import kernels as K
+    t, n = 67, 128
+    kv, kv_view, gamma, pos, slots, nblk = _case(t, seed=12)
+    g = torch.Generator().manual_seed(13)
+    q = torch.randn(t, n, 192, generator=g).bfloat16()
+    cos, sin = O.rope_tables(pos)
+    cd, sd, gd, sl = cos.to(dev), sin.to(dev), gamma.to(dev), slots.to(dev)
+
+    def caches():
+        if fp8:
+            return torch.zeros(nblk, 128, 656, dtype=torch.uint8, device=dev), None
+        return torch.zeros(nblk, 128, 512, dtype=torch.bfloat16, device=dev), torch.zeros(nblk, 128, 64, dtype=torch.bfloat16, device=dev)
+
+    n1, r1 = caches()
+    a1, p1 = torch.zeros(t, 512, dtype=torch.bfloat16, device=dev), torch.zeros(t, 64, dtype=torch.bfloat16, device=dev)
+    q1 = q.to(dev)
+    K.kv_rmsnorm_rope_cache(kv_view(dev), gd, cd, sd, sl, n1, r1, eps=EPS, kv_a_out=a1, k_pe_out=p1)
+    K.interleave_rope(q1[..., 128:], cd, sd, out=q1[..., 128:])
+    n2, r2 = caches()
+    a2, p2 = torch.zeros_like(a1), torch.zeros_like(p1)
+    q2 = q.to(dev)
+    K.kv_rmsnorm_rope_cache(kv_view(dev), gd, cd, sd, sl, n2, r2, eps=EPS, kv_a_out=a2, k_pe_out=p2, q_rope=q2[..., 128:])
+    assert torch.equal(n1, n2) and (fp8 or torch.equal(r1, r2)) and torch.equal(a1, a2) and torch.equal(p1, p2)
+    assert torch.equal(q1, q2) and torch.equal(q2[..., :128].cpu(), q[..., :128])
+    _ulp_close(q2[..., 128:], O.interleave_rope(q[..., 128:], cos, sin))
+    # without a cache (profile run) and into a separate query tensor
+    q3 = torch.zeros(t, n, 64, dtype=torch.bfloat16, device=dev)
+    K.kv_rmsnorm_rope_cache(kv_view(dev), gd, cd, sd, None, None, None, eps=EPS, kv_a_out=a2, k_pe_out=p2,
+                            q_rope=q.to(dev)[..., 128:], q_out=q3)
+    assert torch.equal(q3, q1[..., 128:]) and torch.equal(a1, a2)
+
+
 @pytest.mark.parametrize("layout", ["half", "repeat"])
 def test_rotary_mul_strided_and_in_place(dev, layout):
     """The half-rotation pairing of the indexer's rope dims (npu_dsa.py:116-131) on a strided view, then in place."""
