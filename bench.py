@@ -782,6 +782,147 @@ def bench_layer(K, dev, args):
     }
 
 
+def bench_dsa_layer(K, dev, args):
+    """The attention part of one DSA decode layer through the backend classes, on the configs[3] shape (B = 32, contexts
+    uniform[32768, 65536], 64 fp8 index heads, top-2048, 128 heads): fused RMSNorm + rotary embedding + cache write + query
+    rope, ``LightningIndexer`` (quantise q and the new index keys, key-cache write, fp8 scores, top-k with cache rows),
+    ``NPUDSAImpl.forward`` (absorption GEMM, sparse split-KV kernel, merge fused with the value up-projection)."""
+    import time
+    from types import SimpleNamespace
+    from oracle import mla_oracle as O
+    from omni_npu_amd import _vllm_compat as V
+    from omni_npu_amd.attention.backends import dsa
+    B, H, N, k, EPS = 32, 64, 128, 2048, 1e-6
+    g = torch.Generator().manual_seed(args.seed)
+    lens = torch.randint(32768, 65537, (B,), generator=g).to(torch.int32)
+    nblk_seq = (lens + 127) // 128
+    nblk = int(nblk_seq.sum())
+    perm = torch.randperm(nblk, generator=g)
+    bt = torch.zeros(B, int(nblk_seq.max()), dtype=torch.int32)
+    o = 0
+    for b in range(B):
+        n = int(nblk_seq[b])
+        bt[b, :n] = perm[o:o + n].to(torch.int32)
+        o += n
+    btd = bt.to(dev)
+    raw = torch.zeros(nblk * 128 * 704, dtype=torch.bfloat16, device=dev).view(torch.uint8)
+    kv_cache = dsa.NPUDSABackend.reshape_kv_cache(raw, nblk, 128, 1, 704, dtype=torch.bfloat16)
+    torch.manual_seed(args.seed)
+    step_blk = 2048
+    for b0 in range(0, nblk, step_blk):
+        b1 = min(nblk, b0 + step_blk)
+        kv_cache[0][b0:b1].copy_(torch.randn(b1 - b0, 128, 1, 512, device=dev))
+        kv_cache[1][b0:b1].copy_(torch.randn(b1 - b0, 128, 1, 64, device=dev))
+    k8v, ksv = dsa.indexer_cache_views(kv_cache[2])
+    for b in range(B):
+        L = int(lens[b])
+        pos = torch.arange(L, device=dev)
+        K.quant_rows_fp8(torch.randn(L, 128, device=dev).bfloat16(), k8v, ksv,
+                         slot_mapping=btd[b, pos // 128].long() * 128 + pos % 128)
+    slots = torch.stack([bt[b, (int(lens[b]) - 1) // 128].long() * 128 + (int(lens[b]) - 1) % 128 for b in range(B)])
+    w_kv_b = (torch.randn(512, N * 256, generator=g) * 0.05).bfloat16()
+    q = torch.randn(B, N, 192, generator=g).bfloat16()
+    kv = torch.randn(B, 576, generator=g).bfloat16()
+    gamma = (1 + 0.1 * torch.randn(512, generator=g)).bfloat16()
+    iq, ik = torch.randn(B, H, 128, generator=g).bfloat16(), torch.randn(B, 128, generator=g).bfloat16()
+    iw = torch.randn(B, H, generator=g)
+    cos, sin = O.rope_tables(lens.long() - 1)
+    cfg = SimpleNamespace(
+        scheduler_config=SimpleNamespace(max_num_seqs=B), model_config=SimpleNamespace(max_model_len=65536, dtype=torch.bfloat16),
+        cache_config=SimpleNamespace(block_size=128, cache_dtype="auto"),
+        parallel_config=SimpleNamespace(cp_kv_cache_interleave_size=1, decode_context_parallel_size=1, worker_cls=None),
+        compilation_config=SimpleNamespace(max_cudagraph_capture_size=B, pass_config=None), kv_transfer_config=None,
+        speculative_config=None)
+    impl = dsa.NPUDSAImpl(num_heads=N, head_size=576, scale=192 ** -0.5, num_kv_heads=1, alibi_slopes=None,
+                          sliding_window=None, kv_cache_dtype="auto", logits_soft_cap=None,
+                          attn_type=V.AttentionType.DECODER, kv_sharing_target_layer_name=None, q_lora_rank=None,
+                          kv_lora_rank=512, qk_nope_head_dim=128, qk_rope_head_dim=64, qk_head_dim=192, v_head_dim=128,
+                          kv_b_proj=lambda x: (x @ w_kv_b.to(x.device),))
+    kvw = w_kv_b.view(512, N, 256)
+    impl.W_UK_T = kvw[..., :128].permute(1, 2, 0).contiguous().to(dev)
+    impl.W_UV = kvw[..., 128:].transpose(0, 1).contiguous().to(dev)
+    indexer = dsa.LightningIndexer(k, H, 128, max_tokens=B, device=dev)
+    impl.indexer = indexer
+    qsl = torch.arange(B + 1, dtype=torch.int32)
+    common = V.CommonAttentionMetadata(
+        query_start_loc=qsl.to(dev), query_start_loc_cpu=qsl.clone(), seq_lens=lens.to(dev), seq_lens_cpu=lens.clone(),
+        num_computed_tokens_cpu=lens - 1, num_reqs=B, num_actual_tokens=B, max_query_len=1, max_seq_len=int(lens.max()),
+        block_table_tensor=btd, slot_mapping=slots.to(dev))
+    builder = dsa.NPUDSAMetadataBuilder(V.AttentionSpec(128, 1, 704, torch.bfloat16), ["layer"], cfg, dev)
+    meta = builder.build(0, common)
+    d_q, d_kv, d_gamma, d_cos, d_sin, d_iq, d_ik, d_iw = (x.to(dev) for x in (q, kv, gamma, cos, sin, iq, ik, iw))
+    kvc = torch.empty(B, 512, dtype=torch.bfloat16, device=dev)
+    kpe = torch.empty(B, 64, dtype=torch.bfloat16, device=dev)
+    q_in = d_q.clone()
+    out = torch.zeros(B, N * 128, dtype=torch.bfloat16, device=dev)
+
+    def layer():
+        K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, kv_cache[0], kv_cache[1], eps=EPS, kv_a_out=kvc,
+                                k_pe_out=kpe, q_rope=d_q[..., 128:], q_out=q_in[..., 128:])
+        indexer(d_iq, d_ik, d_iw, kv_cache, meta)
+        impl.cache_written_for = meta
+        impl.forward(None, q_in, kvc, kpe.unsqueeze(1), kv_cache, meta, output=out)
+
+    def timed(fn, n):
+        a, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        a.record()
+        for _ in range(n):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(e) * 1e3 / n
+
+    clock_ramp(layer)
+    for _ in range(args.warmup):
+        layer()
+    t_eager = sorted(timed(layer, args.steps) for _ in range(3))[1]
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        layer()
+        with torch.cuda.graph(graph, stream=side):
+            layer()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        graph.replay()
+    t_graph = sorted(timed(graph.replay, args.steps) for _ in range(3))[1]
+
+    # oracle: sparse attention over the positions the GPU picked, on the caches as the GPU left them, for two sequences
+    cpu_info = cpu_fields()
+    sel = indexer.topk_indices_buffer[:B].cpu()
+    checks, cpu_s = [], 0.0
+    for b in (0, B - 1):
+        L = int(lens[b])
+        picks = sel[b][sel[b] >= 0]
+        assert picks.numel() == min(k, L) and int(picks.max()) < L and picks.unique().numel() == picks.numel()
+        pages = bt[b, :int(nblk_seq[b])].long()
+        c_nope = kv_cache[0][pages.to(dev)].cpu().view(-1, 128, 512)
+        c_rope = kv_cache[1][pages.to(dev)].cpu().view(-1, 128, 64)
+        t0 = time.perf_counter()
+        q_pe = O.interleave_rope(q[b:b + 1, :, 128:], cos[b:b + 1], sin[b:b + 1])
+        ql = O.q_absorb(q[b:b + 1, :, :128], impl.W_UK_T.cpu()).bfloat16()
+        local_bt = torch.arange(pages.numel(), dtype=torch.int32).view(1, -1)
+        ref_o = O.sparse_decode(ql, q_pe, c_nope, c_rope, local_bt, [L], sel[b:b + 1], impl.scale)
+        ref = O.v_up_proj(ref_o.transpose(0, 1).contiguous().bfloat16(), impl.W_UV.cpu()).view(-1)
+        cpu_s += time.perf_counter() - t0
+        checks.append((out[b].float().cpu() - ref.float()).abs().max().item())
+    return {
+        "metric": "DSA decode attention of one layer through the backend classes, us/layer (B=32, ctx 32k-64k, top-2048, 128 heads)",
+        "value": round(t_eager, 2), "unit": "us/layer", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": False, "dtype": "fp8 (indexer) / bf16 (attention)", "data": "synthetic",
+        "config": {"workload": "configs[3] through NPUDSAMetadataBuilder + LightningIndexer + NPUDSAImpl.forward with the fused "
+                               "prologue in front", "batch": B, "heads": N, "index_heads": H, "topk": k,
+                   "sum_seq_len": int(lens.sum()), "seed": args.seed},
+        "layer_us": {"eager_launches_queued": round(t_eager, 2), "hip_graph_replay": round(t_graph, 2)},
+        "roofline": None,
+        "cpu_baseline": {"value": round(cpu_s * B / 2 * 1e6, 1), "unit": "us/layer", **cpu_info, "kind": "port",
+                         "sample": "oracle rope + absorption + sparse attention + up-projection (torch fp32) of 2 of 32 tokens on the "
+                                   "GPU's picks, scaled by token count; the indexer is not in this sample",
+                         "gpu_vs_oracle_max_abs": max(checks)},
+    }
+
+
 def bench_window(K, dev, args):
     """Decode with static sink tokens and a sliding window (the reference's variant of attention/backends/mla.py:705-779):
     B=64, 128 heads, 4096-8192 keys behind a 128-key sink, window 4096.  One step = window plan + dense split kernel over
@@ -877,8 +1018,8 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 512 MiB device copy three times: its known traffic calibrates the FETCH_SIZE / "
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
-    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue", "window", "layer"],
-                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel; layer = the attention part of a decode layer through the backend classes (NPUMLAMetadataBuilder + NPUMLAImpl.forward with the fused steps around it)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue", "window", "layer", "dsa-layer"],
+                    help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel; layer = the attention part of a decode layer through the backend classes (NPUMLAMetadataBuilder + NPUMLAImpl.forward with the fused steps around it); dsa-layer = the same for configs[3] (LightningIndexer + NPUDSAImpl.forward)")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -917,6 +1058,9 @@ def main():
         return
     if args.workload == "layer":
         print(json.dumps(bench_layer(K, dev, args)))
+        return
+    if args.workload == "dsa-layer":
+        print(json.dumps(bench_dsa_layer(K, dev, args)))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
     heads, b, q_len = args.heads, args.batch, args.q_len

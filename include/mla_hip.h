@@ -285,6 +285,14 @@ int dsa_quant_rows_fp8(const void* src, int64_t src_stride, int64_t rows, const 
                        void* dst8, int64_t dst_page_stride_bytes, int64_t dst_row_stride_bytes, float* dst_scale,
                        int64_t scale_page_stride, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
 
+/* dsa_quant_rows_fp8 twice in one launch, the way the indexer needs it every step (patch_dsv32_indexer.py:116-131: the new
+ * index keys go into the cache, the queries are handed to the scoring op): q rows [q_rows, 128] -> q8 [q_rows, 128] +
+ * q_scale [q_rows]; k rows [k_rows, 128] -> row slot_mapping[r] of the paged key cache and of its scale plane. */
+int dsa_quant_qk_fp8(const void* q, int64_t q_stride, int64_t q_rows, void* q8, float* q_scale, const void* k,
+                     int64_t k_stride, int64_t k_rows, const int64_t* slot_mapping, void* k8_cache,
+                     int64_t cache_page_stride_bytes, int64_t cache_row_stride_bytes, float* scale_cache,
+                     int64_t scale_page_stride, int32_t page_size, int64_t num_pages, mlahip_stream_t stream);
+
 /* With a workspace of dsa_topk_workspace_bytes() the selection of a token is spread over several workgroups (three
  * launches that meet in the workspace: slice histograms, boundary-bin gather, ordered write), which is what a
  * decode step with few tokens and long rows needs; with workspace == NULL one workgroup per token does everything and

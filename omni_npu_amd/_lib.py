@@ -59,6 +59,7 @@ SIGNATURES = {
     "dsa_indexer_scores_fp8": (c_int32, [P, I64, I64, P, I64, P, I64, P, I64, I64, P, I64, I64, I32, P, I64, I32, P, P, I32,
                                          I32, I32, I32, P, I64, P]),
     "dsa_quant_rows_fp8": (c_int32, [P, I64, I64, P, P, I64, I64, P, I64, I32, I64, P]),
+    "dsa_quant_qk_fp8": (c_int32, [P, I64, I64, P, P, P, I64, I64, P, P, I64, I64, P, I64, I32, I64, P]),
     "dsa_topk_workspace_bytes": (SZ, [I32, I32, I64]),
     "dsa_topk": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, SZ, P]),
     "dsa_topk_rows": (c_int32, [P, I64, P, P, I32, I32, I32, P, I64, P, I64, I32, I32, I64, P, I64, P, P, SZ, P]),

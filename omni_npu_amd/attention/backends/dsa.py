@@ -162,10 +162,11 @@ class LightningIndexer:
         assert len(kv_cache) >= 3, f"Expected kv_cache to have at least 3 elements, but got {len(kv_cache)}"
         k8, ks = indexer_cache_views(kv_cache[2])
         t = q.shape[0]
-        K.quant_rows_fp8(k.reshape(-1, self.head_dim), k8, ks, attn_metadata.slot_mapping)
         q8 = torch.empty(t, self.n_head, self.head_dim, dtype=torch.uint8, device=q.device)
         qs = torch.empty(t, self.n_head, dtype=torch.float32, device=q.device)
-        K.quant_rows_fp8(q.reshape(t * self.n_head, self.head_dim), q8, qs)
+        # the new keys into the cache and the queries into plain buffers: one launch
+        K.quant_qk_fp8(q.reshape(t * self.n_head, self.head_dim), q8, qs, k.reshape(-1, self.head_dim), k8, ks,
+                       attn_metadata.slot_mapping)
         w = weights.float().contiguous()
         out = self.topk_indices_buffer[:t]
         off = 0

@@ -215,12 +215,18 @@ __global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerPa
 // optionally scattered through a slot mapping into a paged fp8 cache + scale cache: the indexer-K write of
 // src/omni_npu/vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:116-121 with quantisation fused in, and
 // the query quantisation (no slot mapping).  One wavefront per row, lane l owns elements 2l, 2l+1.
-__global__ __launch_bounds__(256) void dsa_quant_rows_kernel(const __bf16* src, int64_t src_stride, int64_t rows,
-                                                             const int64_t* slots, uint8_t* dst8, int64_t d_sp, int64_t d_sr,
-                                                             float* dscale, int64_t s_sp, int32_t page_size,
-                                                             int64_t num_pages) {
+struct QuantRows {
+  const __bf16* src; int64_t src_stride, rows;
+  const int64_t* slots;
+  uint8_t* dst8; int64_t d_sp, d_sr;
+  float* dscale; int64_t s_sp;
+  int32_t page_size; int64_t num_pages;
+};
+
+__device__ __forceinline__ void quant_row(const __bf16* src, int64_t src_stride, int64_t rows, const int64_t* slots,
+                                          uint8_t* dst8, int64_t d_sp, int64_t d_sr, float* dscale, int64_t s_sp,
+                                          int32_t page_size, int64_t num_pages, int64_t r) {
   const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= rows) return;
   int64_t slot = slots ? slots[r] : r;
   if (slot < 0 || slot >= num_pages * page_size) return;
@@ -237,8 +243,50 @@ __global__ __launch_bounds__(256) void dsa_quant_rows_kernel(const __bf16* src, 
   if (lane == 0) dscale[pg * s_sp + off] = scale;
 }
 
+__global__ __launch_bounds__(256) void dsa_quant_rows_kernel(const __bf16* src, int64_t src_stride, int64_t rows,
+                                                             const int64_t* slots, uint8_t* dst8, int64_t d_sp, int64_t d_sr,
+                                                             float* dscale, int64_t s_sp, int32_t page_size,
+                                                             int64_t num_pages) {
+  quant_row(src, src_stride, rows, slots, dst8, d_sp, d_sr, dscale, s_sp, page_size, num_pages,
+            (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6));
+}
+
+// Two row sets in one launch (the indexer's step: the query rows into plain buffers, the new key rows into the cache):
+// the first a_blocks workgroups take set a, the others set b.
+__global__ __launch_bounds__(256) void dsa_quant_rows2_kernel(const QuantRows a, const QuantRows b, int32_t a_blocks) {
+  const bool first = (int)blockIdx.x < a_blocks;
+  const QuantRows& q = first ? a : b;
+  quant_row(q.src, q.src_stride, q.rows, q.slots, q.dst8, q.d_sp, q.d_sr, q.dscale, q.s_sp, q.page_size, q.num_pages,
+            (int64_t)(first ? blockIdx.x : blockIdx.x - a_blocks) * 4 + (threadIdx.x >> 6));
+}
+
 }  // namespace mlahip
 using namespace mlahip;
+
+// dsa_quant_rows_fp8 of the query rows (plain outputs) and of the new key rows (into the paged index-key cache) in one launch.
+extern "C" int dsa_quant_qk_fp8(const void* q, int64_t q_stride, int64_t q_rows, void* q8, float* q_scale, const void* k,
+                                int64_t k_stride, int64_t k_rows, const int64_t* slot_mapping, void* k8_cache,
+                                int64_t cache_page_stride_bytes, int64_t cache_row_stride_bytes, float* scale_cache,
+                                int64_t scale_page_stride, int32_t page_size, int64_t num_pages, hipStream_t stream) {
+  MLA_REQUIRE(q && q8 && q_scale && k && slot_mapping && k8_cache && scale_cache, MLA_ERR_NULL,
+              "dsa_quant_qk_fp8: null pointer argument");
+  MLA_REQUIRE(q_rows >= 0 && k_rows >= 0 && page_size >= 1 && num_pages >= 1 && q_stride % 2 == 0 && k_stride % 2 == 0 &&
+                  cache_row_stride_bytes >= 128 && cache_row_stride_bytes % 2 == 0 && cache_page_stride_bytes % 2 == 0 &&
+                  (uintptr_t)q % 4 == 0 && (uintptr_t)k % 4 == 0 && (uintptr_t)q8 % 2 == 0 && (uintptr_t)k8_cache % 2 == 0 &&
+                  q_rows < (1ll << 31) && k_rows < (1ll << 31),
+              MLA_ERR_SHAPE, "dsa_quant_qk_fp8: q_rows=%lld k_rows=%lld page_size=%d", (long long)q_rows, (long long)k_rows,
+              page_size);
+  if (q_rows + k_rows == 0) return MLA_OK;
+  // (set a has no slot mapping: row r is "slot" r of one page that holds them all)
+  const QuantRows a{(const __bf16*)q, q_stride, q_rows, nullptr, (uint8_t*)q8, 0, 128, q_scale, 0,
+                    (int32_t)(q_rows > 0 ? q_rows : 1), 1};
+  const QuantRows b{(const __bf16*)k, k_stride, k_rows, slot_mapping, (uint8_t*)k8_cache, cache_page_stride_bytes,
+                    cache_row_stride_bytes, scale_cache, scale_page_stride, page_size, num_pages};
+  const int64_t a_blocks = (q_rows + 3) / 4, b_blocks = (k_rows + 3) / 4;
+  hipLaunchKernelGGL(dsa_quant_rows2_kernel, dim3((unsigned)(a_blocks + b_blocks)), dim3(256), 0, stream, a, b,
+                     (int32_t)a_blocks);
+  return check_launch("dsa_quant_rows2_kernel");
+}
 
 extern "C" int dsa_quant_rows_fp8(const void* src, int64_t src_stride, int64_t rows, const int64_t* slot_mapping,
                                   void* dst8, int64_t dst_page_stride_bytes, int64_t dst_row_stride_bytes,

@@ -874,6 +874,38 @@ def decode_fp8(q_nope: torch.Tensor, q_rope: torch.Tensor, cache: torch.Tensor, 
     return out
 
 
+def quant_qk_fp8(q: torch.Tensor, q8: torch.Tensor, q_scale: torch.Tensor, k: torch.Tensor, k8_cache: torch.Tensor,
+                 scale_cache: torch.Tensor, slot_mapping: torch.Tensor) -> None:
+    """quant_rows_fp8(q, q8, q_scale) and quant_rows_fp8(k, k8_cache, scale_cache, slot_mapping) in one launch: the
+    indexer's two quantisations of a step (src/omni_npu/vllm_patches/patches/models/deepseek/patch_dsv32_indexer.py:116-131)."""
+    _need_cuda(q, q8, q_scale, k, k8_cache, scale_cache, slot_mapping)
+    lib = _lib.load()
+    q2, k2 = q.reshape(-1, q.shape[-1]), k.reshape(-1, k.shape[-1])
+    o8, sc = q8.reshape(-1, 128), q_scale.reshape(-1)
+    if k8_cache.dim() == 4 and k8_cache.shape[2] == 1:
+        k8_cache = k8_cache.squeeze(2)
+    for x in (q2, k2):
+        if x.shape[-1] != 128 or x.dtype != torch.bfloat16 or x.stride(-1) != 1:
+            raise TypeError("quant_qk_fp8: bf16 rows of 128")
+    if o8.data_ptr() != q8.data_ptr() or not o8.is_contiguous() or o8.element_size() != 1 or o8.shape[0] < q2.shape[0] or \
+            sc.dtype != torch.float32 or not sc.is_contiguous() or sc.numel() < q2.shape[0]:
+        raise ValueError("quant_qk_fp8: q8 / q_scale must be contiguous 1-byte [R,128] / fp32 [R]")
+    if k8_cache.dim() != 3 or k8_cache.element_size() != 1 or k8_cache.stride(-1) != 1 or scale_cache.dtype != torch.float32 or \
+            scale_cache.shape[:2] != k8_cache.shape[:2]:
+        raise ValueError("quant_qk_fp8: paged outputs must be 1-byte [nblk,page,128] and fp32 [nblk,page]")
+    ksc = scale_cache.reshape(k8_cache.shape[0], k8_cache.shape[1])
+    if ksc.stride(-1) != 1:
+        raise ValueError("quant_qk_fp8: scale rows must be contiguous")
+    if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+        slot_mapping = slot_mapping.to(torch.int64).contiguous()
+    n = min(k2.shape[0], slot_mapping.numel())
+    rc = lib.dsa_quant_qk_fp8(q2.data_ptr(), q2.stride(0), q2.shape[0], o8.data_ptr(), sc.data_ptr(), k2.data_ptr(),
+                              k2.stride(0), n, slot_mapping.data_ptr(), k8_cache.data_ptr(), k8_cache.stride(0),
+                              k8_cache.stride(1), ksc.data_ptr(), ksc.stride(0), k8_cache.shape[1], k8_cache.shape[0],
+                              _stream(q))
+    _lib.check(rc, "dsa_quant_qk_fp8")
+
+
 def quant_rows_fp8(x: torch.Tensor, out8: torch.Tensor, out_scale: torch.Tensor,
                    slot_mapping: Optional[torch.Tensor] = None) -> None:
     """Per-row e4m3 quantisation of bf16 rows [R,128] (scale = amax/448).  Without ``slot_mapping``: out8 [R,128] (1-byte

@@ -237,3 +237,35 @@ def test_indexer_topk_rows_random_shapes(dev, i, batch, lo, hi, q_len, k, single
         b = tt // q_len
         pos = torch.tensor(got, dtype=torch.long)
         assert torch.equal(rows_c[tt, :len(got)].long(), c["block_table"][b, pos // 128].long() * 128 + pos % 128)
+
+
+def test_quant_qk_in_one_launch_equals_the_two_launches(dev):
+    """The indexer's two quantisations of a step (queries into plain buffers, new keys into the paged cache with pad slots
+    skipped) as one launch: the same bytes and scales as two dsa_quant_rows_fp8 launches."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(17)
+    t, h, nblk = 37, 64, 5
+    q = torch.randn(t * h, 128, generator=g).bfloat16().to(dev)
+    k = (torch.randn(t, 128, generator=g) * 3).bfloat16().to(dev)
+    k[3] = 0                                                  # an all-zero row: scale 1
+    slots = torch.randperm(nblk * 128, generator=g)[:t]
+    slots[5] = -1
+    slots = slots.to(dev)
+    def run(one):
+        q8 = torch.zeros(t * h, 128, dtype=torch.uint8, device=dev)
+        qs = torch.zeros(t * h, dtype=torch.float32, device=dev)
+        k8 = torch.full((nblk, 128, 128), 7, dtype=torch.uint8, device=dev)
+        ks = torch.full((nblk, 128), -1.0, dtype=torch.float32, device=dev)
+        if one:
+            K.quant_qk_fp8(q, q8, qs, k, k8, ks, slots)
+        else:
+            K.quant_rows_fp8(q, q8, qs)
+            K.quant_rows_fp8(k, k8, ks, slot_mapping=slots)
+        return q8, qs, k8, ks
+    a, b = run(True), run(False)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    ref8, refs = O.fp8_quant_token(k.float().cpu())
+    sm = slots.cpu()
+    ok = sm >= 0
+    assert torch.equal(a[2].cpu().view(-1, 128)[sm[ok]], ref8.view(torch.uint8)[ok]) and torch.equal(a[3].cpu().view(-1)[sm[ok]], refs[ok])
