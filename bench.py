@@ -718,7 +718,7 @@ def bench_layer(K, dev, args):
     def layer():
         K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, nope, rope, eps=EPS, kv_a_out=kvc, k_pe_out=kpe,
                                 q_rope=d_q[..., 128:], q_out=q_in[..., 128:])
-        impl.cache_written_for = meta
+        impl.cache_written_for = (meta, B)
         impl.forward(None, q_in, kvc, kpe.unsqueeze(1), (nope, rope), meta, output=out)
 
     def timed(fn, n):
@@ -860,7 +860,7 @@ def bench_dsa_layer(K, dev, args):
         K.kv_rmsnorm_rope_cache(d_kv, d_gamma, d_cos, d_sin, meta.slot_mapping, kv_cache[0], kv_cache[1], eps=EPS, kv_a_out=kvc,
                                 k_pe_out=kpe, q_rope=d_q[..., 128:], q_out=q_in[..., 128:])
         indexer(d_iq, d_ik, d_iw, kv_cache, meta)
-        impl.cache_written_for = meta
+        impl.cache_written_for = (meta, B)
         impl.forward(None, q_in, kvc, kpe.unsqueeze(1), kv_cache, meta, output=out)
 
     def timed(fn, n):

@@ -10,8 +10,7 @@ import os
 from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# OMNI_NPU_AMD_LIB points at another build of the same library (kernel experiments)
-LIB_PATH = os.environ.get("OMNI_NPU_AMD_LIB") or os.path.join(_HERE, "libmla_hip.so")
+LIB_PATH = os.path.join(_HERE, "libmla_hip.so")
 
 P, I32, I64, F32, SZ = c_void_p, c_int32, c_int64, c_float, c_size_t
 

@@ -329,3 +329,33 @@ if HAVE_VLLM:  # pragma: no cover
     from vllm.v1.attention.backends.utils import split_decodes_and_prefills  # noqa: F401
 
 PAD_SLOT_ID = -1
+
+
+class _DeviceBytes:
+    """A span of device memory named by address only, for ``torch.as_tensor``: the tensor built over it owns nothing."""
+
+    def __init__(self, ptr: int, nbytes: int):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 3,
+                                         "strides": None}
+
+
+def _weak_ref_tensor(t):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.numel() == 0:
+        return t
+    # the smallest span of the storage the view can touch
+    span = 1 + sum((n - 1) * st for n, st in zip(t.shape, t.stride()))
+    with torch.cuda.device(t.device):
+        raw = torch.as_tensor(_DeviceBytes(t.data_ptr(), span * t.element_size()), device=t.device)
+    return raw.view(t.dtype).as_strided(t.shape, t.stride())
+
+
+def weak_ref_tensors(out):
+    """Aliases of ``out`` (a tensor, or a list / tuple of them) that do not keep its storage alive, as vLLM's helper of the
+    same name gives: a captured graph's output then lives in the graph's memory pool alone, and the pool can hand the
+    bytes to the next graph (reference acl_graph.py:209-222).  Without vLLM the alias is built over the bare address."""
+    if HAVE_VLLM:  # pragma: no cover
+        from vllm.utils.torch_utils import weak_ref_tensors as _w
+        return _w(out)
+    if isinstance(out, (list, tuple)):
+        return type(out)(weak_ref_tensors(o) for o in out)
+    return _weak_ref_tensor(out)

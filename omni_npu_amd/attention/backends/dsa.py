@@ -17,6 +17,7 @@ from typing import ClassVar, Optional, Tuple
 import torch
 
 from ... import kernels as K
+from .mla import _caller_wrote_cache, _persistent_int32
 from ..._vllm_compat import (PAD_SLOT_ID, AttentionCGSupport, AttentionType, MLACommonBackend, MLACommonBaseImpl,
                              MLACommonDecodeMetadata, MLACommonMetadata, MLACommonMetadataBuilder,
                              MLACommonPrefillMetadata, QueryLenSupport, get_current_vllm_config)
@@ -111,7 +112,7 @@ class NPUDSAMetadataBuilder(MLACommonMetadataBuilder[NPUDSAMetadata]):
         n = qlens.numel()
         max_q = int(qlens.max()) if n else 1
         uniform = n > 0 and int(qlens.min()) == max_q
-        return NPUDSADecodeMetadata(block_table=block_table_tensor, seq_lens=seq_lens_device.to(torch.int32),
+        return NPUDSADecodeMetadata(block_table=block_table_tensor, seq_lens=_persistent_int32(self, "_seq_lens_i32", seq_lens_device),
                                     dcp_tot_seq_lens=dcp_tot_seq_lens_device, query_cumlens=query_start_loc_device[1:],
                                     query_start_loc=None if uniform else query_start_loc_device.to(torch.int32).contiguous(),
                                     q_len=max_q)
@@ -307,7 +308,7 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
         has_decode = attn_metadata.num_decodes > 0
         has_prefill = attn_metadata.num_prefills > 0
         ndt = attn_metadata.num_decode_tokens
-        written, self.cache_written_for = self.cache_written_for is attn_metadata, None
+        written = _caller_wrote_cache(self, attn_metadata, num_actual_toks)
         if not written:                                            # (else the caller's fused norm + rope launch wrote them)
             K.cache_write(k_c_normed, k_pe, attn_metadata.slot_mapping, k_nope, k_rope)
         topk = self.indexer.topk_indices_buffer

@@ -109,6 +109,23 @@ class NPUMLAMetadata(MLACommonMetadata[NPUMLADecodeMetadata]):
     pass
 
 
+def _persistent_int32(owner, name: str, t: torch.Tensor) -> torch.Tensor:
+    """``t`` itself when it is int32 already (the runner's persistent buffer: captured graphs read it in place).  A
+    runner that keeps its lengths in another integer type (the reference widens them, npu_model_runner.py:81-86) gets
+    them copied into ONE int32 buffer owned by the builder, which only ever grows, so that a graph captured over a step
+    reads the lengths of every later step from the same address instead of from a fresh tensor per build."""
+    if t.dtype == torch.int32:
+        return t
+    buf = getattr(owner, name, None)
+    if buf is None or buf.numel() < t.numel() or buf.device != t.device:
+        buf = torch.zeros(max(t.numel(), 2 * (buf.numel() if buf is not None else 0)), dtype=torch.int32,
+                          device=t.device)
+        setattr(owner, name, buf)
+    view = buf[:t.numel()]
+    view.copy_(t)
+    return view
+
+
 class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
     _cudagraph_support: ClassVar[AttentionCGSupport] = AttentionCGSupport.ALWAYS
     supports_uniform_spec_as_decode: ClassVar[bool] = True
@@ -139,7 +156,7 @@ class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
         uniform = num_decodes > 0 and int(qlens.min()) == max_q
         return NPUMLADecodeMetadata(
             block_table=block_table_tensor,
-            seq_lens=seq_lens_device.to(torch.int32),
+            seq_lens=_persistent_int32(self, "_seq_lens_i32", seq_lens_device),
             dcp_tot_seq_lens=dcp_tot_seq_lens_device,
             query_cumlens=query_start_loc_device[1:],
             query_start_loc=None if uniform else query_start_loc_device.to(torch.int32).contiguous(),
@@ -159,6 +176,16 @@ class NPUMLAMetadataBuilder(MLACommonMetadataBuilder[NPUMLAMetadata]):
             metadata.prefill.query_cumlens = common_attn_metadata.query_start_loc_cpu[1:].tolist()
             metadata.prefill.seq_lens = metadata.prefill.query_cumlens
         return metadata
+
+
+def _caller_wrote_cache(impl, attn_metadata, num_tokens: int) -> bool:
+    """Consumes ``impl.cache_written_for``: True when the caller's fused norm + rope launch has written the cache rows
+    of this very metadata object and at least ``num_tokens`` of them (the mark is ``(metadata, rows written)``)."""
+    mark, impl.cache_written_for = impl.cache_written_for, None
+    if mark is None:
+        return False
+    meta, rows = mark
+    return meta is attn_metadata and rows >= num_tokens
 
 
 class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
@@ -408,7 +435,7 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
 
         # write the latent and rope rows of the new tokens (one launch), unless the caller's fused norm + rope launch has
         # put them there already and said so for this very metadata object
-        written, self.cache_written_for = self.cache_written_for is attn_metadata, None
+        written = _caller_wrote_cache(self, attn_metadata, num_actual_toks)
         if written:
             pass
         elif self.fp8_cache:

@@ -12,12 +12,17 @@ from __future__ import annotations
 
 import copy
 import dataclasses
+import logging
 import os
+from contextlib import ExitStack
 from typing import Any, Callable, Optional
+from unittest.mock import patch
 
 import torch
 
-from .._vllm_compat import BatchDescriptor, CUDAGraphMode, get_forward_context
+from .._vllm_compat import BatchDescriptor, CUDAGraphMode, get_forward_context, weak_ref_tensors
+
+logger = logging.getLogger(__name__)
 
 
 @dataclasses.dataclass
@@ -30,6 +35,10 @@ class HIPGraphEntry:
 
 @dataclasses.dataclass
 class HIPGraphOptions:
+    """The reference's options (acl_graph.py:190-222), acted on the same way: ``debug_log_enable`` logs each capture,
+    ``gc_disable`` turns ``gc.collect`` and ``torch.cuda.empty_cache`` into no-ops for the duration of a capture (a
+    piecewise model captures one graph per layer), ``weak_ref_output`` lets go of the strong reference to the output
+    inside the capture (safe for the last graph of a forward only)."""
     debug_log_enable: bool = True
     gc_disable: bool = False
     weak_ref_output: bool = True
@@ -70,15 +79,24 @@ class HIPGraphWrapper:
             entry = self.concrete_graph_entries[batch_descriptor] = HIPGraphEntry(batch_descriptor=batch_descriptor)
 
         if entry.graph is None:
+            if self.graph_options.debug_log_enable:
+                logger.debug("Capturing a hipGraph on (%s,%s)", self.runtime_mode.name, entry.batch_descriptor)
             entry.input_addresses = [x.data_ptr() for x in args if isinstance(x, torch.Tensor)]
             graph = torch.cuda.CUDAGraph()
-            forward_context.capturing = True
-            try:
-                with torch.cuda.graph(graph, pool=self.graph_pool):
-                    output = self.runnable(*args, **kwargs)
-            finally:
-                forward_context.capturing = False
-            entry.output = output          # plain aliases: the graph's memory pool keeps them alive
+            with ExitStack() as stack:
+                if self.graph_options.gc_disable:
+                    stack.enter_context(patch("gc.collect", lambda: None))
+                    stack.enter_context(patch("torch.cuda.empty_cache", lambda: None))
+                forward_context.capturing = True
+                try:
+                    with torch.cuda.graph(graph, pool=self.graph_pool):
+                        output = self.runnable(*args, **kwargs)
+                        if self.graph_options.weak_ref_output:
+                            output = weak_ref_tensors(output)
+                finally:
+                    forward_context.capturing = False
+            # the entry never holds a strong reference: the graph's memory pool owns the bytes
+            entry.output = weak_ref_tensors(output)
             entry.graph = graph
             return output
 

@@ -94,18 +94,6 @@ __device__ __forceinline__ int wave_incl_scan_dpp(int v) {
 }
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
-#ifdef MLA_V3_TRACE
-__device__ unsigned long long* g_trace;                     // [workgroup][wave][8]: clock sums per phase, block count
-#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0, tr_k0 = 0, tr_e0 = 0, tr_ep = 0, tr_p[4] = {0, 0, 0, 0}; TR_STAMP(tr_k0)
-#define TR_PRO(k) do { if (tr_p[k] == 0) { TR_STAMP(tr_b); tr_p[k] = tr_b - tr_start; } } while (0)
-#define TR_STAMP(x) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x)::"memory")
-#define TR_ADD(k) do { TR_STAMP(tr_b); tr_t[k] += tr_b - tr_a; tr_a = tr_b; } while (0)
-#else
-#define TR_DECL
-#define TR_STAMP(x)
-#define TR_ADD(k)
-#define TR_PRO(k)
-#endif
 
 // kRG = groups of 32 query rows that can hold rows at all (4: any launch; 1 or 2: launches with at most 32 / 64 query rows
 // per request, e.g. the 16 heads a tensor-parallel rank of eight owns).  With few rows the 128-row schedule spends the same
@@ -117,10 +105,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
   static_assert(kRG == 1 || kRG == 2 || kRG == 4, "row groups");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-#ifdef MLA_V3_TRACE
-  uint64_t tr_start;
-  TR_STAMP(tr_start);
-#endif
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // 0..7
   const int l16 = lane & 15;                                  // QK: query row of the wave / key of a 16-key group
@@ -158,9 +142,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   // With up to 64 sequences a lane holds one sequence's length and query range: everything the plan and the first
   // segment need comes from one round of loads issued together at the start of the kernel (each dependent round trip
   // to memory costs more than a microsecond there, with cold caches).
-#ifdef MLA_V3_TRACE
-  uint64_t tr_x0 = 0, tr_x1 = 0;
-#endif
   int seg_b;
   int64_t v_cur, v_end, v_seq;
   int first_L = -1, first_q0 = 0, first_q1 = 0;               // the first segment's sequence, if known from the plan's loads
@@ -180,9 +161,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     int pe1 = 0;
     if (one_pass) { pe1 = wave_incl_scan_dpp(tot); tot = __builtin_amdgcn_readlane(pe1, 63); }
     else tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
-#ifdef MLA_V3_TRACE
-    TR_STAMP(tr_x0);
-#endif
     // chunk c covers units [floor(c * tot / G), floor((c + 1) * tot / G)); with G <= 65536 that is 32-bit arithmetic:
     // c * tot / G = c * (tot / G) + c * (tot % G) / G exactly (a 64-bit division is a long software routine)
     int64_t cb, ce;
@@ -224,11 +202,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     }
   }
 
-  TR_DECL;
-#ifdef MLA_V3_TRACE
-  TR_STAMP(tr_x1);
-  tr_p[3] = tr_x1 - tr_start;
-#endif
   while (v_cur < v_end) {
   seg_b++;
   if (seg_b >= p.batch) break;
@@ -486,7 +459,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   // copies its own 16 rows global -> LDS whole (one row per instruction, into the tile buffers, which are free at the
   // start of a segment) and picks its operands from there.  The copies of the first key blocks have to wait until
   // every wave has its query in registers (one barrier).
-  TR_PRO(0);
   bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
   // One row group: the two wavefronts that can own rows stage their query in the tile buffer of the segment's FOURTH block,
   // which is not requested before the block loop runs, so the copying wavefronts ask for the first three blocks now and
@@ -547,7 +519,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     for (int kk = 0; kk < 18; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
   }
   lds_barrier();                                              // every wave has read its query: the tile buffers are free
-  TR_PRO(1);
   if constexpr (kRG != 1) issue_first();
 
   f32x16 acc[2][4];                                          // [32-column block of this wave's 64][row group]
@@ -842,7 +813,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     {
       if (nb > 2) MLA_WAIT_VMCNT(18); else if (nb > 1) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);   // (kCopies per block in flight)
       lds_barrier();
-      TR_PRO(2);
       f32x4 s[2];
       Sm st;
       if (has_rows) {
@@ -866,18 +836,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     // brought back (and waited for) now, not at its first use inside the loop.
     asm volatile("" :: "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run), "v"(top_p), "v"(top_tag), "v"(dma_off));
     // ---- steady state: QK(i+1), then P.V(i) with the softmax of block i+1 riding along ----
-#ifdef MLA_V3_TRACE
-    if (tr_t[5] == 0) { TR_STAMP(tr_b); tr_t[5] = tr_b - tr_start; }
-#endif
     for (int i = 0; i + 1 < nb; i++) {
       const int blk = blk_begin + i;
-      TR_STAMP(tr_a);
       // block i+1 has landed, P(i) is published, everyone is done with P.V(i-1)
       if (i + 2 < nb) MLA_WAIT_VMCNT(9); else MLA_WAIT_VMCNT(0);
-      TR_ADD(0);
       lds_barrier();
       if (i + kLead < nb) ids_fetch(blk + kLead);             // (row list) the rows of the block whose copies go out now
-      TR_ADD(1);
       const int fl = flags_read(blk);
       f32x4 s[2];
       if constexpr (kRG < 4) {
@@ -902,18 +866,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       if (i + kLead >= nb || !copier) qk_block(blk + 1, s, std::integral_constant<int, 0>{}, 0);
       else if (kSparse || !full_ok || L - 1 - (blk + kLead) * kBlk < kBlk - 1) qk_block(blk + 1, s, std::integral_constant<int, 1>{}, blk + kLead);
       else qk_block(blk + 1, s, std::integral_constant<int, 2>{}, blk + kLead);
-      TR_ADD(2);
       if (restarts_left > 0 && flags_ask_restart(fl)) { restart = true; restarts_left--; break; }
       Sm st;
       float sc[8];
       unpack_scores(s, sc);
       pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st, has_rows);
-      TR_ADD(3);
       if (has_rows) softmax_finish(blk + 1, sc, st);
-      TR_ADD(4);
-#ifdef MLA_V3_TRACE
-      tr_n++;
-#endif
     }
     if (!restart) {
       const int blk = blk_end - 1;
@@ -925,7 +883,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   } while (restart);
 
   // ---- epilogue ----
-  TR_STAMP(tr_e0);
   // (lane-derived values are worked out again from the hardware lane number: nothing of them has to live through the loop)
   lds_barrier();                                              // all PV done; tile buffers and P buffers are free
   const int e_ln = lane_now();
@@ -1011,20 +968,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       *(u32x2*)(o_part_c + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#ifdef MLA_V3_TRACE
-  TR_STAMP(tr_b); tr_ep += tr_b - tr_e0;
-#endif
   }  // segments
-#ifdef MLA_V3_TRACE
-  if (g_trace && lane == 0) {
-    unsigned long long* t = g_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.z) * 8 + wave) * 16;
-    for (int k = 0; k < 6; k++) t[k] = tr_t[k];
-    t[6] = tr_n;
-    t[7] = tr_ep;
-    for (int k = 0; k < 4; k++) t[8 + k] = tr_p[k];
-    t[12] = tr_x0 - tr_start;
-  }
-#endif
 }
 
 }  // namespace v3
@@ -1046,13 +990,6 @@ static int launch_rows(const DecodeParams& p, dim3 grid, hipStream_t stream) {
 }
 
 int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream) {
-#ifdef MLA_V3_TRACE
-  {
-    const char* e = getenv("MLA_V3_TRACE_PTR");
-    unsigned long long* ptr = e ? (unsigned long long*)strtoull(e, nullptr, 16) : nullptr;
-    hipMemcpyToSymbol(HIP_SYMBOL(v3::g_trace), &ptr, sizeof(ptr));
-  }
-#endif
   if (sparse) return launch_rows<true, false>(p, grid, stream);
   if (p.win_skip) return launch_rows<false, true>(p, grid, stream);
   return launch_rows<false, false>(p, grid, stream);

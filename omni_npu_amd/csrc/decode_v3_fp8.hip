@@ -83,18 +83,6 @@ __device__ __forceinline__ int wave_incl_scan_dpp(int v) {
 }
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
-#ifdef MLA_V3_TRACE
-__device__ unsigned long long* g_trace;                     // [workgroup][wave][8]: clock sums per phase, block count
-#define TR_DECL uint64_t tr_t[6] = {0, 0, 0, 0, 0, 0}, tr_a = 0, tr_b = 0, tr_n = 0, tr_k0 = 0, tr_e0 = 0, tr_ep = 0, tr_p[4] = {0, 0, 0, 0}; TR_STAMP(tr_k0)
-#define TR_PRO(k) do { if (tr_p[k] == 0) { TR_STAMP(tr_b); tr_p[k] = tr_b - tr_start; } } while (0)
-#define TR_STAMP(x) asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(x)::"memory")
-#define TR_ADD(k) do { TR_STAMP(tr_b); tr_t[k] += tr_b - tr_a; tr_a = tr_b; } while (0)
-#else
-#define TR_DECL
-#define TR_STAMP(x)
-#define TR_ADD(k)
-#define TR_PRO(k)
-#endif
 
 // kRG = groups of 32 query rows that can hold rows at all (4: any launch; 1 or 2: at most 32 / 64 query rows per request, as
 // in the bf16 kernel): only the wavefronts that own rows run the S phase and the softmax, P.V covers kRG row groups, the
@@ -103,10 +91,6 @@ template <bool kWindow, int kRG = 4>
 __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodeParams p) {
   static_assert(kRG == 1 || kRG == 2 || kRG == 4, "row groups");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-#ifdef MLA_V3_TRACE
-  uint64_t tr_start;
-  TR_STAMP(tr_start);
-#endif
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // 0..7
   const int l16 = lane & 15;                                  // QK: query row of the wave / key of a 16-key group
@@ -144,9 +128,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   // With up to 64 sequences a lane holds one sequence's length and query range: everything the plan and the first
   // segment need comes from one round of loads issued together at the start of the kernel (each dependent round trip
   // to memory costs more than a microsecond there, with cold caches).
-#ifdef MLA_V3_TRACE
-  uint64_t tr_x0 = 0, tr_x1 = 0;
-#endif
   int seg_b;
   int64_t v_cur, v_end, v_seq;
   int first_L = -1, first_q0 = 0, first_q1 = 0;               // the first segment's sequence, if known from the plan's loads
@@ -166,9 +147,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     int pe1 = 0;
     if (one_pass) { pe1 = wave_incl_scan_dpp(tot); tot = __builtin_amdgcn_readlane(pe1, 63); }
     else tot = __builtin_amdgcn_readfirstlane(wave_sum_i32(tot));
-#ifdef MLA_V3_TRACE
-    TR_STAMP(tr_x0);
-#endif
     // chunk c covers units [floor(c * tot / G), floor((c + 1) * tot / G)); with G <= 65536 that is 32-bit arithmetic:
     // c * tot / G = c * (tot / G) + c * (tot % G) / G exactly (a 64-bit division is a long software routine)
     int64_t cb, ce;
@@ -210,11 +188,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     }
   }
 
-  TR_DECL;
-#ifdef MLA_V3_TRACE
-  TR_STAMP(tr_x1);
-  tr_p[3] = tr_x1 - tr_start;
-#endif
   while (v_cur < v_end) {
   seg_b++;
   if (seg_b >= p.batch) break;
@@ -383,7 +356,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   // copies its own 16 rows global -> LDS whole (one row per instruction, into the tile buffers, which are free at the
   // start of a segment) and picks its operands from there.  The copies of the first key blocks have to wait until
   // every wave has its query in registers (one barrier).
-  TR_PRO(0);
   bf16x8 qf[18];                                             // contraction steps of 32: 16 over the latent part, 2 over rope
   if (!has_rows) {
 #pragma unroll
@@ -441,7 +413,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     for (int kk = 0; kk < 18; kk++) asm volatile("" : "+v"(qf[kk]));           // the query stays in VGPRs
   }
   lds_barrier();                                              // every wave has read its query: the staging area is free
-  TR_PRO(1);
 
   f32x16 acc[2][4];                                          // [32-column block of this wave's 64][row group]
 #pragma unroll
@@ -706,7 +677,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     if (nb > 2) issue_block(blk_begin + 2);
     // ---- block 0: QK, softmax, publish ----
     {
-      TR_PRO(2);
       f32x4 s[2];
       Sm st;
       if (has_rows) {
@@ -730,18 +700,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     // brought back (and waited for) now, not at its first use inside the loop.
     asm volatile("" :: "v"(vbase[0]), "v"(vbase[1]), "v"(m_ref), "v"(l_run));
     // ---- steady state: dequantise block i+2, request block i+3, QK(i+1), then P.V(i) with the softmax of block i+1 ----
-#ifdef MLA_V3_TRACE
-    if (tr_t[5] == 0) { TR_STAMP(tr_b); tr_t[5] = tr_b - tr_start; }
-#endif
     for (int i = 0; i + 1 < nb; i++) {
       const int blk = blk_begin + i;
-      TR_STAMP(tr_a);
       // tile i+1 is complete, raw block i+2 has landed (after this wait and the barrier), P(i) is published, everyone is
       // done with P.V(i-1), i.e. with tile (i+2) % 3, and with raw stage (i+1) & 1
       MLA_WAIT_VMCNT(0);
-      TR_ADD(0);
       lds_barrier();
-      TR_ADD(1);
       const int fl = flags_read(blk);
       // The copying wavefronts dequantise their half of block i+2 (rows 0..15) now, the others theirs (rows 16..31) at the
       // end of the body: the two wavefronts of a SIMD then run half a phase apart, and one's conversions and LDS writes
@@ -752,19 +716,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       if (i + 3 < nb) issue_block(blk + 3);
       f32x4 s[2];
       if (has_rows) qk_block(blk + 1, s);
-      TR_ADD(2);
       if (restarts_left > 0 && flags_ask_restart(fl)) { restart = true; restarts_left--; break; }
       Sm st;
       float sc[8];
       unpack_scores(s, sc);
       pv_softmax(blk, std::true_type{}, std::true_type{}, sc, st, has_rows);
-      TR_ADD(3);
       if (has_rows) softmax_finish(blk + 1, sc, st);
       if (!copier && i + 2 < nb) dequant_block(blk + 2);
-      TR_ADD(4);
-#ifdef MLA_V3_TRACE
-      tr_n++;
-#endif
     }
     if (!restart) {
       const int blk = blk_end - 1;
@@ -776,7 +734,6 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   } while (restart);
 
   // ---- epilogue ----
-  TR_STAMP(tr_e0);
   // (lane-derived values are worked out again from the hardware lane number: nothing of them has to live through the loop)
   lds_barrier();                                              // all PV done; tile buffers and P buffers are free
   const int e_ln = lane_now();
@@ -832,20 +789,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
       *(u32x2*)(o_part_c + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#ifdef MLA_V3_TRACE
-  TR_STAMP(tr_b); tr_ep += tr_b - tr_e0;
-#endif
   }  // segments
-#ifdef MLA_V3_TRACE
-  if (g_trace && lane == 0) {
-    unsigned long long* t = g_trace + ((size_t)(blockIdx.x + gridDim.x * blockIdx.z) * 8 + wave) * 16;
-    for (int k = 0; k < 6; k++) t[k] = tr_t[k];
-    t[6] = tr_n;
-    t[7] = tr_ep;
-    for (int k = 0; k < 4; k++) t[8 + k] = tr_p[k];
-    t[12] = tr_x0 - tr_start;
-  }
-#endif
 }
 
 }  // namespace f8v3
@@ -867,13 +811,6 @@ static int launch_rows_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream)
 }
 
 int launch_decode_v3_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
-#ifdef MLA_V3_TRACE
-  {
-    const char* e = getenv("MLA_V3_TRACE_PTR");
-    unsigned long long* ptr = e ? (unsigned long long*)strtoull(e, nullptr, 16) : nullptr;
-    hipMemcpyToSymbol(HIP_SYMBOL(f8v3::g_trace), &ptr, sizeof(ptr));
-  }
-#endif
   if (p.win_skip) return launch_rows_fp8<true>(p, grid, stream);
   return launch_rows_fp8<false>(p, grid, stream);
 }

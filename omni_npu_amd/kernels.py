@@ -353,11 +353,25 @@ def _workspace(dev: torch.device, nbytes: int, tag: str = "decode") -> torch.Ten
     ``workspace=`` instead."""
     key = (dev.index, torch.cuda.current_stream(dev).cuda_stream, tag)
     bufs = _workspaces.setdefault(key, [])
-    if bufs and bufs[-1].numel() >= nbytes:
-        return bufs[-1]
-    size = max(nbytes, 1, (bufs[-1].numel() * 3) // 2 if bufs else 0)
-    bufs.append(torch.empty(size, dtype=torch.uint8, device=dev))
+    size = _workspace_growth(bufs[-1].numel() if bufs else 0, nbytes)
+    if size:
+        bufs.append(torch.empty(size, dtype=torch.uint8, device=dev))
     return bufs[-1]
+
+
+def _workspace_growth(have: int, nbytes: int) -> int:
+    """Size of the buffer to allocate next to one of ``have`` bytes for a request of ``nbytes`` (0: the one there is
+    enough).  Every new buffer is at least 1.5 x its predecessor, so a key that has seen requests up to M bytes holds at
+    most 2 + log1.5(M / first request) buffers and less than 4.5 M bytes in total (the newest is below 1.5 M, the one
+    before it below M, the older ones shrink geometrically)."""
+    if have >= max(nbytes, 1):
+        return 0
+    return max(nbytes, 1, (have * 3) // 2)
+
+
+def retained_workspace_bytes() -> int:
+    """Bytes of scratch this process holds in all (device, stream, tag) keys; they are released at process end only."""
+    return sum(b.numel() for bufs in _workspaces.values() for b in bufs)
 
 
 # Sparse MLA over many tokens (a DSA prefill chunk) runs in launches of at most this much split-KV scratch, so the scratch

@@ -63,36 +63,43 @@ class NPUMultiHeadLatentAttentionWrapper(torch.nn.Module):
             cos, sin = rope.get_cos_sin(positions)
             kv_c_normed = torch.zeros(t, K.D_NOPE, dtype=kv_lora.dtype, device=kv_lora.device)
             k_pe = torch.zeros(t, K.D_ROPE, dtype=kv_lora.dtype, device=kv_lora.device)
-            slots, nope_c, rope_c = self._cache_target()
+            impl, meta, slots, nope_c, rope_c = self._cache_target()
             q_rope = None
             if q is not None and q.dtype == torch.bfloat16 and q.stride(-1) == 1 and q.shape[0] == t:
                 q_rope = q[..., self.qk_nope_head_dim:]
+            if impl is not None:
+                impl.cache_written_for = None                  # a launch that raises must leave no mark behind
             K.kv_rmsnorm_rope_cache(kv_lora, norm.weight, cos, sin, slots, nope_c, rope_c, eps=eps, kv_a_out=kv_c_normed,
                                     k_pe_out=k_pe, q_rope=q_rope)
+            if impl is not None and slots is not None:
+                # the rows of this step are in place: the impl skips its own write for this metadata object, provided
+                # the launch covered every token it would have written
+                impl.cache_written_for = (meta, min(int(slots.numel()), t))
             return kv_c_normed, k_pe.unsqueeze(1), (cos, sin, q_rope is not None)
         kv_c, k_pe = kv_lora.split([self.kv_lora_rank, self.qk_rope_head_dim], dim=-1)
         return norm(kv_c), k_pe.unsqueeze(1), None
 
     def _cache_target(self):
-        """Where the fused launch may also write the new tokens' cache rows: (slot_mapping, latent cache, rope cache or
-        None for the fp8 cache) when the step has metadata, the layer a cache, every token a slot, and the backend impl
-        agrees to skip its own write for this metadata object; (None, None, None) otherwise."""
+        """Where the fused launch may also write the new tokens' cache rows: (impl, metadata, slot_mapping, latent cache,
+        rope cache or None for the fp8 cache) when the step has metadata, the layer a cache, every token a slot, and the
+        backend impl can skip its own write for a marked metadata object; five times None otherwise.  The mark itself
+        is set by the caller once the launch has been issued."""
+        none = (None, None, None, None, None)
         impl = getattr(self.mla_attn, "impl", None)
         if impl is None or not hasattr(impl, "cache_written_for"):
-            return None, None, None
+            return none
         ctx = V.get_forward_context()
         meta = ctx.attn_metadata
         if isinstance(meta, dict):
             meta = meta.get(self.mla_attn.layer_name)
         kv_cache = self.mla_attn.kv_cache[ctx.virtual_engine]
         if meta is None or kv_cache is None or getattr(meta, "slot_mapping", None) is None:
-            return None, None, None
+            return none
         if meta.slot_mapping.numel() < meta.num_actual_tokens:
-            return None, None, None
-        impl.cache_written_for = meta
+            return none
         if getattr(impl, "fp8_cache", False):
-            return meta.slot_mapping, kv_cache[0], None
-        return meta.slot_mapping, kv_cache[0], kv_cache[1]
+            return impl, meta, meta.slot_mapping, kv_cache[0], None
+        return impl, meta, meta.slot_mapping, kv_cache[0], kv_cache[1]
 
     def forward_oot(self, positions: torch.Tensor, hidden_states: torch.Tensor,
                     llama_4_scaling: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -239,3 +239,41 @@ def test_graph_wrapper_captures_and_replays_the_decode_forward(dev):
             assert torch.equal(got, eager), f"replay {trial} differs from eager"
     with V.set_forward_context({"l": meta}, desc, V.CUDAGraphMode.NONE):
         assert wrapper(q) is out and len(wrapper.concrete_graph_entries) == 1
+
+
+def test_graph_wrapper_options_act_on_the_capture(dev):
+    """``gc_disable`` silences gc.collect / empty_cache for the duration of a capture only, ``weak_ref_output`` hands back an
+    alias that owns nothing (the graph's pool keeps the bytes), and replays still see new input contents
+    (reference acl_graph.py:190-222)."""
+    import gc
+    from omni_npu_amd.compilation.acl_graph import HIPGraphOptions
+    real_collect, real_empty = gc.collect, torch.cuda.empty_cache
+    seen = {}
+
+    def runnable(x):
+        seen["collect"], seen["empty"] = gc.collect, torch.cuda.empty_cache
+        return x * 2 + 1, x.float().sum(dim=-1)
+
+    x = torch.arange(24, dtype=torch.bfloat16, device=dev).view(4, 6)
+    runnable(x)
+    torch.cuda.synchronize()
+    for gc_disable, weak in ((True, True), (False, False)):
+        w = HIPGraphWrapper(runnable, _cfg(), V.CUDAGraphMode.FULL,
+                            cudagraph_options=HIPGraphOptions(debug_log_enable=False, gc_disable=gc_disable,
+                                                              weak_ref_output=weak))
+        desc = V.BatchDescriptor(num_tokens=4, num_reqs=4, uniform=True)
+        with V.set_forward_context(None, desc, V.CUDAGraphMode.FULL):
+            first = w(x)
+            assert (seen["collect"] is not real_collect) == gc_disable and (seen["empty"] is not real_empty) == gc_disable
+            assert gc.collect is real_collect and torch.cuda.empty_cache is real_empty     # restored after the capture
+            held = w.concrete_graph_entries[desc].output
+            assert isinstance(first, tuple) and isinstance(held, tuple)
+            for a, b in zip(first, held):
+                assert a.data_ptr() == b.data_ptr() and a.shape == b.shape and a.dtype == b.dtype
+                # the entry's copy never owns the bytes: its storage is a bare span, not the allocator's block
+                assert b.untyped_storage().data_ptr() == b.data_ptr()
+            for k in range(3):
+                x.copy_(torch.arange(24, dtype=torch.bfloat16).view(4, 6) + k)
+                y, ssum = w(x)
+                torch.cuda.synchronize()
+                assert torch.equal(y, x * 2 + 1) and torch.equal(ssum, x.float().sum(dim=-1))

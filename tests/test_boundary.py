@@ -351,3 +351,44 @@ def test_custom_model_modules_need_a_norm_with_parameters():
     with V.set_forward_context(attn_metadata=SimpleNamespace(prefill=object(), decode=object())):
         with pytest.raises(NotImplementedError):
             mod(torch.zeros(2, 256), None, None)
+
+
+def test_workspace_growth_keeps_the_retained_scratch_bounded():
+    """Scratch buffers are never freed (captured graphs hold their addresses); the growth rule bounds what a key retains:
+    at most 2 + log1.5(max / first) buffers and less than 4.5 x the largest request in total."""
+    import math
+    import random
+    from omni_npu_amd import kernels as K
+    rng = random.Random(0)
+    for trial in range(200):
+        reqs = [rng.randint(64, 1 << rng.randint(7, 30)) for _ in range(rng.randint(1, 60))]
+        sizes, have = [], 0
+        for r in reqs:
+            new = K._workspace_growth(have, r)
+            if new:
+                assert new >= r and new >= (have * 3) // 2
+                sizes.append(new)
+                have = new
+            assert have >= r
+        m = max(reqs)
+        assert len(sizes) <= 2 + math.log(m / sizes[0]) / math.log(1.49)
+        assert sum(sizes) < 4.5 * m + len(sizes)
+    assert K._workspace_growth(100, 100) == 0 and K._workspace_growth(0, 0) == 1 and K._workspace_growth(100, 101) == 150
+
+
+def test_builder_keeps_widened_seq_lens_in_one_int32_buffer():
+    """A runner that hands over int64 lengths (the reference widens them, npu_model_runner.py:81-86) must not give every
+    step a fresh int32 tensor: a graph captured over one step would read stale lengths.  int32 input passes through."""
+    spec = V.AttentionSpec(128, 1, 576, torch.bfloat16)
+    for builder in (mla.NPUMLAMetadataBuilder(spec, ["l0"], _cfg(cap=4), torch.device("cpu")),
+                    dsa.NPUDSAMetadataBuilder(spec, ["l0"], _cfg(cap=4), torch.device("cpu"))):
+        c = _common([1, 1, 1], [300, 130, 2])
+        assert builder.build(0, c).decode.seq_lens.data_ptr() == c.seq_lens.data_ptr()
+        ptrs = []
+        for lens in ([300, 130, 2], [301, 131, 3], [5, 6, 7]):
+            c = _common([1, 1, 1], lens)
+            c.seq_lens = c.seq_lens.to(torch.int64)
+            d = builder.build(0, c).decode
+            assert d.seq_lens.dtype == torch.int32 and d.seq_lens.tolist() == lens
+            ptrs.append(d.seq_lens.data_ptr())
+        assert len(set(ptrs)) == 1

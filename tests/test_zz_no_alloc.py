@@ -63,3 +63,54 @@ def test_static_scratch_decode_refuses_what_does_not_fit(dev):
     rc = lib.mla_decode_bf16_static(p, 512, 512, p, 64, 64, p, 65536, 512, p, 8192, 64, 1, p, 1, 1, p, None, batch, q_len, heads,
                                     0.1, p, 512, 512, None, splits, None)
     assert rc == -4 and b"built-in array" in lib.mlahip_last_error_string()
+
+
+def test_static_scratch_decode_allocates_nothing_and_replays_from_a_graph(dev):
+    """After one warm-up call outside capture (address lookup, LDS limit) a call moves neither the device's free memory
+    nor the torch allocator's counters, and a call recorded into a HIP graph replays to the eager bytes every time, with
+    the program's own eager work between the replays."""
+    from omni_npu_amd import _lib
+    lib = _lib.load()
+    batch, heads, splits = 6, 128, 3
+    c = O.make_decode_case(batch, heads, 300, 1200, seed=23)
+    g = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in c.items()}
+    qn, qr, nope, rope, bt, sl = (g[k] for k in ("q_nope", "q_rope", "nope", "rope", "block_table", "seq_lens"))
+    out = torch.zeros(batch, heads, 512, dtype=torch.bfloat16, device=dev)
+    lse = torch.zeros(batch, heads, dtype=torch.float32, device=dev)
+
+    def call():
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.mla_decode_bf16_static(_ptr(qn), qn.stride(0), qn.stride(1), _ptr(qr), qr.stride(0), qr.stride(1),
+                                        _ptr(nope), nope.stride(0), nope.stride(1), _ptr(rope), rope.stride(0), rope.stride(1),
+                                        nope.shape[0], _ptr(bt), bt.stride(0), bt.shape[1], _ptr(sl), None, batch, 1, heads,
+                                        float(c["scale"]), _ptr(out), out.stride(0), out.stride(1), _ptr(lse), splits, stream)
+        assert rc == 0, lib.mlahip_last_error_string()
+
+    call()                                                    # warm-up outside capture
+    torch.cuda.synchronize()
+    free0, stats0 = torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_stats(dev)
+    call()
+    torch.cuda.synchronize()
+    free1, stats1 = torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_stats(dev)
+    assert free1 == free0, f"device free memory moved by {free0 - free1} bytes across a call"
+    for k in ("allocation.all.allocated", "allocated_bytes.all.allocated", "segment.all.allocated", "reserved_bytes.all.allocated"):
+        assert stats1[k] == stats0[k], k
+    eager = (out.clone(), lse.clone())
+    ref = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], c["scale"])
+    assert (eager[0].float().cpu() - ref).abs().max().item() <= 2e-2
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for rep in range(3):
+        # eager work of the program between the replays: another static call on other lengths, then the outputs cleared
+        sl.copy_((c["seq_lens"] // 2).to(dev))
+        call()
+        sl.copy_(c["seq_lens"].to(dev))
+        out.zero_()
+        lse.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager[0].view(torch.int16)), f"replay {rep}: output differs from eager"
+        assert torch.equal(lse, eager[1]), f"replay {rep}: log-sum-exp differs from eager"
