@@ -668,24 +668,29 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     // (small forms only, where the matrix pipe has time to spare: the block's last MFMAs have written their accumulators
     // before anything the compiler may place behind this statement reads them)
 #define PV_SETTLE(rg) asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+a"(acc[0][rg]), "+a"(acc[1][rg]))
+    // The small forms have matrix time to spare and spend it on precision: a probability goes through P.V as TWO bf16
+    // numbers, its rounded value and the rounding's remainder (fragments rg + 2 of the exchange buffer), each fragment of
+    // V^T feeding both.  The product then carries 16 significant bits of every probability instead of 8, and the result's
+    // error is the rounding of the output alone.
     if constexpr (kRG == 1) {
-      // one row group: two MFMAs per k-block, the softmax steps in the shadow of the LDS reads
-      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); }
+      // one row group: four MFMAs per k-block, the softmax steps in the shadow of the LDS reads
+      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 2, 0); }
       if constexpr (kSm) { if (sm_on) { sm_head(sc, st); SM_EXP2(0, 1); SM_EXP2(2, 3); } }
-      if constexpr (kPv) { PV_MFMA2(0, pr0, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); }
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_MFMA2(0, pr1, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); PV_PREAD(pr1, 2, 1); }
       if constexpr (kSm) { if (sm_on) { SM_EXP2(4, 5); SM_EXP2(6, 7); sm_pm(st); } }
-      if constexpr (kPv) { PV_MFMA2(0, pr0, 0); PV_SETTLE(0); }
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_MFMA2(0, pr1, 0); PV_SETTLE(0); }
       if constexpr (kSm) { if (sm_on) { sm_sum_lo(sc, st); sm_sum_hi(sc, st); } }
     } else if constexpr (kRG == 2) {
-      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 1, 0); }
+      // (two register quads for the four P^T fragments of a k-block, each refilled as soon as its MFMAs are issued)
+      if constexpr (kPv) { PV_VREAD(0); PV_PREAD(pr0, 0, 0); PV_PREAD(pr1, 2, 0); }
       if constexpr (kSm) { if (sm_on) { sm_head(sc, st); SM_EXP2(0, 1); } }
-      if constexpr (kPv) PV_MFMA2(0, pr0, 1);
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_PREAD(pr0, 1, 0); PV_MFMA2(0, pr1, 1); PV_PREAD(pr1, 3, 0); }
       if constexpr (kSm) { if (sm_on) SM_EXP2(2, 3); }
-      if constexpr (kPv) { PV_MFMA2(1, pr1, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); PV_PREAD(pr1, 1, 1); }
+      if constexpr (kPv) { PV_MFMA2(1, pr0, 1); PV_MFMA2(1, pr1, 0); PV_VREAD(1); PV_PREAD(pr0, 0, 1); PV_PREAD(pr1, 2, 1); }
       if constexpr (kSm) { if (sm_on) { SM_EXP2(4, 5); SM_EXP2(6, 7); sm_pm(st); } }
-      if constexpr (kPv) PV_MFMA2(0, pr0, 1);
+      if constexpr (kPv) { PV_MFMA2(0, pr0, 1); PV_PREAD(pr0, 1, 1); PV_MFMA2(0, pr1, 1); PV_PREAD(pr1, 3, 1); }
       if constexpr (kSm) { if (sm_on) sm_sum_lo(sc, st); }
-      if constexpr (kPv) { PV_MFMA2(1, pr1, 0); PV_SETTLE(0); PV_SETTLE(1); }
+      if constexpr (kPv) { PV_MFMA2(1, pr0, 1); PV_MFMA2(1, pr1, 0); PV_SETTLE(0); PV_SETTLE(1); }
       if constexpr (kSm) { if (sm_on) sm_sum_hi(sc, st); }
     } else {
     (void)sm_on;
@@ -752,6 +757,19 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     const uint32_t pw = lds0 + (blk & 1) * kPBufB + p_w_off_now();
     const u32x2 w0 = {st.pw[0], st.pw[1]}, w1 = {st.pw[2], st.pw[3]};
     asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %2 offset:1024" :: "v"(pw), "v"(w0), "v"(w1) : "memory");
+    if constexpr (kRG < 4) {
+      // what the rounding to bf16 left of every probability, as a second bf16 (row groups 2 and 3 of the buffer)
+      uint32_t lo[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float r0 = sc[2 * j] - __builtin_bit_cast(float, st.pw[j] << 16);
+        const float r1 = sc[2 * j + 1] - __builtin_bit_cast(float, st.pw[j] & 0xffff0000u);
+        const bf16x2 pr2 = {(__bf16)r0, (__bf16)r1};
+        lo[j] = __builtin_bit_cast(uint32_t, pr2);
+      }
+      const u32x2 l0 = {lo[0], lo[1]}, l1 = {lo[2], lo[3]};
+      asm volatile("ds_write_b64 %0, %1 offset:4096\n\tds_write_b64 %0, %2 offset:5120" :: "v"(pw), "v"(l0), "v"(l1) : "memory");
+    }
     const bool flag = st.t > kRestartThreshold;               // asks the workgroup to restart with better references
     const bool any = __builtin_amdgcn_ballot_w64(flag) != 0;
     if (any) {
@@ -777,6 +795,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       const uint32_t pw = lds0 + p_w_off_now();
       asm volatile("ds_write_b64 %0, %1\n\tds_write_b64 %0, %1 offset:1024\n\tds_write_b64 %0, %1 offset:8192\n\tds_write_b64 %0, %1 offset:9216"
                    :: "v"(pw), "v"(z) : "memory");
+      // and the slots of the remainders, two row groups further on, when this wavefront's row group is one that P.V reads
+      // (the wavefronts of row groups 2 and 3 have just cleared the remainder slots of groups 0 and 1 by the lines above;
+      // a barrier stands between these writes and the first published block)
+      if (wave < 4)
+        asm volatile("ds_write_b64 %0, %1 offset:4096\n\tds_write_b64 %0, %1 offset:5120\n\tds_write_b64 %0, %1 offset:12288\n\t"
+                     "ds_write_b64 %0, %1 offset:13312" :: "v"(pw), "v"(z) : "memory");
     }
   }
   bool restart = false;
@@ -910,7 +934,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     KernArgPtr kp = cold();
     const __bf16* nope0 = kp->nope;
     const __bf16* vrow = nope0;
-    if (e_row_ok && top_tok >= 0 && top_p * 16.f > l_tot) {
+    // (the small forms carry every probability's rounding remainder through P.V themselves: nothing to add back)
+    if (kRG == 4 && e_row_ok && top_tok >= 0 && top_p * 16.f > l_tot) {
       corr = (top_p - (float)(__bf16)top_p) * inv;
       if constexpr (kSparse) {
         int64_t slot = kp->sparse_rows[(int64_t)b * kp->sparse_stride + top_tok];

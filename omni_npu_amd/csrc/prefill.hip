@@ -11,6 +11,13 @@
 // 192-wide query in registers (B operand of S^T = K Q^T) and a 128 x 32 fp32 accumulator O^T.  Key tiles of 64 keys
 // (nope 64 x 256 B, rope 64 x 128 B, V 64 x 256 B) are copied global -> LDS without touching registers, double
 // buffered; V^T operands come from transposed LDS reads, so P^T stays in registers exactly as in the decode kernel.
+//
+// P.V runs on fp16: the V part of a landed tile is converted from bf16 to fp16 where it lies (same size, same swizzle:
+// element by element), once for the four wavefronts, and the probabilities are rounded to fp16, so they keep 11
+// significant bits instead of bf16's 8.  (With bf16 probabilities AND a bf16 result, flat attention over values
+// unrelated to the keys lands at 2.2e-3 of mean relative error whatever else a kernel does: each rounding alone is
+// 1.4e-3 to 1.7e-3.)  The conversion is exact for |v| in [2^-14, 65504]; smaller values lose at most 2^-25 absolute,
+// larger ones saturate (round toward zero never makes an infinity).
 #include "mla_common.hpp"
 
 namespace mlahip {
@@ -239,32 +246,53 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
     }
 
     for (int tile = first_tile; tile < tiles; tile++) {
-      const char* buf = lds + (tile & 1) * kPfBufB;
-      if (tile + 1 < tiles) {
-        issue(tile + 1, lds0 + ((tile + 1) & 1) * kPfBufB);
-        MLA_WAIT_VMCNT(10);
-      } else {
-        MLA_WAIT_VMCNT(0);
-      }
+      char* buf = lds + (tile & 1) * kPfBufB;
+      // this tile has landed (only its copies are in flight here) and everyone is done with the other buffer
+      MLA_WAIT_VMCNT(0);
       lds_barrier();
+      if (tile + 1 < tiles) issue(tile + 1, lds0 + ((tile + 1) & 1) * kPfBufB);
       const int key_base = tile * kPfTile;
+      char* vt = buf + kPfKnB + kPfKrB + (int)threadIdx.x * 16;
 #pragma unroll 1
       for (int tb = 0; tb < 2; tb++) {
-        if (key_base + tb * 32 >= wave_max_limit) break;      // behind everything a row of this wavefront sees (causal diagonal)
-        if (key_base + tb * 32 + 32 <= wg_lo) continue;       // in front of every row's window
+        // (every wavefront runs both rounds, so the barrier below is reached by all; what a wavefront skips is wave-uniform)
+        const bool active = key_base + tb * 32 < wave_max_limit    // else behind everything a row of this wavefront sees
+                            && key_base + tb * 32 + 32 > wg_lo;     // else in front of every row's window
+        // the V conversion of this tile rides on the first block's score MFMAs: reads before, arithmetic and writes behind
+        u32x4 w[4];
+        if (tb == 0) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) w[i] = *(const u32x4*)(vt + i * 4096);
+        }
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
+          if (!active) break;
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 256 + koff[kk]);
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
         }
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
+          if (!active) break;
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 128 + roff[kk]);
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[8 + kk], s, 0, 0, 0);
         }
+        if (tb == 0) {
+#pragma unroll
+          for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float f_lo = __builtin_bit_cast(float, w[i][e] << 16);
+              const float f_hi = __builtin_bit_cast(float, w[i][e] & 0xffff0000u);
+              w[i][e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(f_lo, f_hi));
+            }
+#pragma unroll
+          for (int i = 0; i < 4; i++) *(u32x4*)(vt + i * 4096) = w[i];
+          lds_barrier();
+        }
+        if (!active) continue;
         // Only blocks that some row of this wave cannot see in full pay for the mask (causal diagonal, end of the keys,
         // rows past the end of the sequence); everywhere else the scores go straight to the maximum.  The scale is
         // folded into the exponent's multiply-add (scale > 0, so the maximum of the raw scores is the raw maximum).
@@ -299,11 +327,11 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][r] *= alpha;
         }
-        bf16x8 pb[2];
+        f16x8 pb[2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-          for (int e = 0; e < 8; e++) pb[kb][e] = (__bf16)s[kb * 8 + e];
+          for (int e = 0; e < 8; e++) pb[kb][e] = (_Float16)s[kb * 8 + e];
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -311,10 +339,9 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
             bf16x4 lo = lds_read_tr16(buf + (tb * 32 + kb * 16) * 256 + voff[0][db]);
             bf16x4 hi = lds_read_tr16(buf + (tb * 32 + kb * 16) * 256 + voff[1][db]);
             bf16x8 a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[kb], acc[db], 0, 0, 0);
+            acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), pb[kb], acc[db], 0, 0, 0);
           }
       }
-      lds_barrier();
     }
   }
 

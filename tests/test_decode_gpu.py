@@ -43,7 +43,31 @@ def test_decode_config1_plumbing(dev, num_splits):
     assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=0)
 
 
-@pytest.mark.parametrize("heads,num_splits", [(16, 1), (16, 3), (128, 2)])
+@pytest.mark.parametrize("heads,num_splits", [(16, 1), (16, 3), (64, 2)])
+def test_small_forms_leave_no_dominant_key_records(dev, heads, num_splits):
+    """With at most 64 query rows per request every probability goes through P.V as two bf16 numbers (value and rounding
+    remainder), so there is nothing for the merge phase to add back: the correction factors stay zero, and the result is
+    the output rounding away from the oracle."""
+    from omni_npu_amd import kernels as K
+    from omni_npu_amd import _lib
+    case = O.make_decode_case(4, heads, 128, 1024, seed=0)
+    b, n = 4, heads
+    ws = torch.zeros(_lib.load().mla_decode_workspace_bytes(b, 1, n, num_splits), dtype=torch.uint8, device=dev)
+    out = torch.empty(b, n, 512, dtype=torch.bfloat16, device=dev)
+    K.decode(case["q_nope"].to(dev), case["q_rope"].to(dev), case["nope"].to(dev), case["rope"].to(dev),
+             case["block_table"].to(dev), case["seq_lens"].to(dev), case["scale"], out, q_len=1, num_splits=num_splits,
+             workspace=ws)
+    torch.cuda.synchronize()
+    rows = b * (num_splits + 1) * n
+    off = rows * 512 * 2 + rows * 4
+    assert not ws.cpu()[off:off + rows * 4].view(torch.float32).any()
+    ref = O.absorbed_decode(case["q_nope"], case["q_rope"], case["nope"], case["rope"], case["block_table"],
+                            case["seq_lens"], case["scale"])
+    ma, mr = attn_close(out, ref, MAX_ABS, MEAN_REL)
+    assert mr <= 1.6e-3, mr
+
+
+@pytest.mark.parametrize("heads,num_splits", [(128, 1), (128, 2), (128, 3)])
 def test_decode_dominant_key_records_name_the_right_cache_row(dev, heads, num_splits):
     """The split phase leaves, per partial row, the cache row of the chunk's most probable key when that key carries more
     than 1/16 of the chunk's weight (the merge phase takes the bf16 rounding of that probability out again).  A record

@@ -76,3 +76,33 @@ def test_decode_random_shapes(dev, i, batch, heads, q_len, lo, hi, splits):
                         num_splits=splits)
         ref_s = O.sparse_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], idx, c["scale"])
         attn_close(out_s, ref_s, 2e-2, 2e-3)
+
+
+# Shapes of the kind that read 2.002e-3 to 2.06e-3 in wide random sweeps while every probability went through P.V as ONE
+# bf16 number: one or a few tokens, 8 or 16 heads (a tensor-parallel rank's share), a few hundred keys, one chunk.  An
+# ideal kernel with bf16 probabilities and a bf16 result sits at 1.85e-3 to 1.9e-3 there, and an output of a few thousand
+# numbers scatters by several percent around that.  The forms for at most 64 query rows now carry the rounding remainder
+# of every probability as a second bf16 number, which leaves the output rounding alone (1.41e-3).
+@pytest.mark.parametrize("batch,heads,q_len,lo,hi,splits,seed", [
+    (1, 8, 1, 500, 500, 1, 11), (1, 8, 1, 500, 500, 1, 12), (1, 8, 1, 500, 500, 1, 13), (1, 16, 1, 300, 300, 1, 14),
+    (2, 8, 1, 200, 640, 1, 15), (1, 16, 1, 1000, 1000, 1, 16), (3, 16, 2, 129, 429, 2, 17), (1, 8, 4, 500, 540, 1, 18),
+    (2, 16, 4, 31, 331, 3, 19), (1, 40, 1, 500, 800, 1, 20), (4, 8, 3, 127, 167, None, 21), (1, 64, 1, 400, 400, 1, 22),
+])
+@pytest.mark.parametrize("unrelated_values", [False, True])
+def test_few_query_rows_keep_a_tenth_of_the_bar_in_hand(dev, batch, heads, q_len, lo, hi, splits, seed, unrelated_values):
+    from omni_npu_amd import kernels as K
+    c = O.make_decode_case(batch, heads, lo, hi, seed=seed, q_len=q_len)
+    if unrelated_values:
+        # the value part of the cache unrelated to what the scores see: queries that only look at the rope part
+        c["q_nope"] = torch.zeros_like(c["q_nope"])
+        c["q_rope"] = (c["q_rope"].float() * 3).bfloat16()
+    t = batch * q_len
+    ref = O.absorbed_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], c["scale"])
+    args = [c[k].to(dev) for k in ("q_nope", "q_rope", "nope", "rope", "block_table", "seq_lens")]
+    out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.decode(*args, c["scale"], out, q_len=q_len, num_splits=splits)
+    ma, mr = attn_close(out, ref, 2e-2, 2e-3)
+    if q_len * heads <= 64:
+        assert mr <= 1.6e-3, f"mean_rel={mr:.4g}: the headroom of the two-term probabilities is gone"
+    else:
+        assert mr <= 1.8e-3, f"mean_rel={mr:.4g}"

@@ -45,7 +45,7 @@ def test_prefill_varlen_matches_oracle(dev, causal, q_lens, k_lens, n):
     K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
                      torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
                      max(q_lens), scale, causal, out, lse)
-    attn_close(out, ref, 2e-2, 2e-3)
+    attn_close(out, ref, 2e-2, 4e-4)                          # fp32 result: only the fp16 rounding of P (2^-12 each) is left
     got_lse = lse.cpu()
     fin = torch.isfinite(ref_lse)
     assert torch.equal(torch.isfinite(got_lse), fin)
@@ -54,10 +54,9 @@ def test_prefill_varlen_matches_oracle(dev, causal, q_lens, k_lens, n):
     K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
                      torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
                      max(q_lens), scale, causal, out_bf)
-    # bf16 output: its rounding alone is 2^-10 = 1e-3 of mean relative error, and with a few dozen keys per row the bf16
-    # rounding of the probabilities (2^-9 each) does not average out; such rows measure 2.0e-3 to 2.1e-3, so rows shorter
-    # than one 64-key block get 2.5e-3, all others the 2e-3 bar
-    attn_close(out_bf, ref, 2e-2, 2e-3 if min(k for k in k_lens if k) >= 64 else 2.5e-3)
+    # bf16 output: its rounding alone is 1.4e-3 of mean relative error; the probabilities go through P.V as fp16 (11
+    # significant bits), which leaves the rest of the 2e-3 bar unused whatever the number of keys
+    attn_close(out_bf, ref, 2e-2, 2e-3)
 
 
 def test_chunked_context_flow_gather_attend_merge(dev):
@@ -185,7 +184,7 @@ def test_prefill_continued_equals_attention_over_all_keys(dev, n, q_lens, k1, k2
         l2 = torch.empty(t, n, dtype=torch.float32, device=dev)
         K.prefill_varlen(d(qn), d(qp), d(kn2), d(kp2), d(v2), ti(cu_q), ti(cu2), max(q_lens), scale, causal2, o2, l2,
                          prev_out=o1, prev_lse=l1)
-        attn_close(o2, ref, 2e-2, 2e-3 if dt == torch.float32 else 2.5e-3)
+        attn_close(o2, ref, 2e-2, 4e-4 if dt == torch.float32 else 2e-3)
         fin = torch.isfinite(ref_lse)
         assert torch.equal(torch.isfinite(l2.cpu()), fin)
         assert torch.allclose(l2.cpu()[fin], ref_lse[fin], atol=2e-2, rtol=0)
@@ -232,8 +231,63 @@ def test_prefill_varlen_random_shapes(dev, i, causal, q_lens, k_lens, n):
     K.prefill_varlen(dq[..., :128], dq[..., 128:], dkv[..., :128], dpe, dkv[..., 128:],
                      torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
                      max(q_lens), scale, causal, out, lse)
-    attn_close(out, ref, 2e-2, 2e-3)
+    attn_close(out, ref, 2e-2, 4e-4)                          # fp32 result: only the fp16 rounding of P (2^-12 each) is left
     got_lse = lse.cpu()
     fin = torch.isfinite(ref_lse)
     assert torch.equal(torch.isfinite(got_lse), fin)
     assert torch.allclose(got_lse[fin], ref_lse[fin], atol=2e-2)
+
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_flat_attention_over_unrelated_values_keeps_the_bf16_bar(dev, seed):
+    """The recipe of the chunked-prefill benchmark, reduced: q, k and v independent N(0,1), scale 1/sqrt(192), a 256-token
+    chunk over 4096 cached keys continued by the causal suffix.  Scores then have unit variance (flat softmax) and the
+    values have nothing to do with the keys: the case in which probabilities rounded to bf16 cost 1.7e-3 by themselves
+    and a bf16 result cannot meet 2e-3.  With fp16 probabilities the bf16 result stays below 1.6e-3."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(100 + seed)
+    n, q_len, ctx = 4, 256, 4096
+    scale = 192 ** -0.5
+    bf = lambda *shape: torch.randn(*shape, generator=g).bfloat16()
+    qn, qp = bf(q_len, n, 128), bf(q_len, n, 64)
+    kc_n, kc_p, vc = bf(ctx, n, 128), bf(ctx, 64), bf(ctx, n, 128)
+    ks_n, ks_p, vs = bf(q_len, n, 128), bf(q_len, 64), bf(q_len, n, 128)
+    ref, _ = O.attention_varlen(qn, qp, torch.cat([kc_n, ks_n]), torch.cat([kc_p, ks_p]), torch.cat([vc, vs]), [0, q_len],
+                                [0, ctx + q_len], scale, True)
+    d = lambda x: x.to(dev)
+    ti = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    o_c = torch.empty(q_len, n, 128, dtype=torch.float32, device=dev)
+    l_c = torch.empty(q_len, n, dtype=torch.float32, device=dev)
+    out = torch.empty(q_len, n, 128, dtype=torch.bfloat16, device=dev)
+    K.prefill_varlen(d(qn), d(qp), d(kc_n), d(kc_p), d(vc), ti([0, q_len]), ti([0, ctx]), q_len, scale, False, o_c, l_c)
+    K.prefill_varlen(d(qn), d(qp), d(ks_n), d(ks_p), d(vs), ti([0, q_len]), ti([0, q_len]), q_len, scale, True, out,
+                     prev_out=o_c, prev_lse=l_c)
+    ma, mr = attn_close(out, ref, 2e-2, 2e-3)
+    assert mr <= 1.6e-3, f"mean_rel={mr:.4g}: the headroom that fp16 probabilities buy is gone"
+
+
+def test_values_outside_the_fp16_range_saturate_and_stay_finite(dev):
+    """V goes through P.V as fp16: magnitudes above 65504 saturate there (never an infinity), magnitudes below 2^-14
+    lose at most 2^-25 absolute.  Rows that only see ordinary values are not affected by an outlier elsewhere."""
+    from omni_npu_amd import kernels as K
+    g = torch.Generator().manual_seed(7)
+    n, q_len = 2, 64
+    scale = 192 ** -0.5
+    bf = lambda *shape: torch.randn(*shape, generator=g).bfloat16()
+    qn, qp, kn, kp, v = bf(q_len, n, 128), bf(q_len, n, 64), bf(q_len, n, 128), bf(q_len, 64), bf(q_len, n, 128)
+    v[40, 0, 3] = 3.0e38                                      # far beyond fp16
+    v[41, 1, 5] = 1.0e-7                                      # an fp16 denormal
+    v[42, 1, 6] = 0.0
+    ref, _ = O.attention_varlen(qn, qp, kn, kp, v, [0, q_len], [0, q_len], scale, True)
+    d = lambda x: x.to(dev)
+    ti = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    out = torch.empty(q_len, n, 128, dtype=torch.float32, device=dev)
+    K.prefill_varlen(d(qn), d(qp), d(kn), d(kp), d(v), ti([0, q_len]), ti([0, q_len]), q_len, scale, True, out)
+    got = out.cpu()
+    assert torch.isfinite(got).all()
+    mask = torch.ones_like(ref, dtype=torch.bool)
+    mask[40:, 0, 3] = False                                   # the rows that see the outlier, in its column
+    attn_close(got[mask].view(1, -1), ref[mask].view(1, -1), 2e-2, 4e-4)
+    sat = got[40:, 0, 3]
+    assert (sat > 0).all() and (sat <= 65504.0 * 1.001).all()
