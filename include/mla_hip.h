@@ -145,6 +145,24 @@ int mla_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h
                     void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out /* fp32 [T,N] or NULL */,
                     void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
 
+/* A whole decode step in two launches: the cache write of the step's new tokens (the reshape-and-cache the reference
+ * runs in front of its decode, attention/backends/mla.py:868-881) rides in the split kernel, then the merge.  Token t
+ * (query_start_loc order, or b * max_q_len + j) brings latent row new_c[t] and rope row new_r[t] for cache row
+ * slot_mapping[t]; negative slots are skipped.  The row of key position p of sequence b is stored by the workgroup
+ * whose chunk holds p, before that workgroup reads any key: the result equals mla_cache_write_bf16 followed by
+ * mla_decode_bf16 for every sequence whose seq_lens counts its new tokens.  (Rows of a request with fewer cached keys
+ * than query tokens - an empty padding request - are not written.)  Page size 128.  With out == NULL only the first
+ * launch runs and the partials stay in the workspace for mla_splitkv_reduce. */
+int mla_decode_bf16_step(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                         int64_t qr_stride_t, int64_t qr_stride_h, void* nope_cache, int64_t nope_page_stride,
+                         int64_t nope_row_stride, void* rope_cache, int64_t rope_page_stride, int64_t rope_row_stride,
+                         int64_t num_pages, const void* new_c /* bf16 [T,512] */, int64_t new_c_stride,
+                         const void* new_r /* bf16 [T,64] */, int64_t new_r_stride, const int64_t* slot_mapping,
+                         const int32_t* block_table, int64_t bt_stride, int32_t max_blocks, const int32_t* seq_lens,
+                         const int32_t* query_start_loc, int32_t batch, int32_t max_q_len, int32_t num_heads,
+                         float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
+                         void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
+
 /* The same decode without a workspace argument, for callers that cannot allocate or hand one over: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  (No counterpart in the reference: its vendor op
  * owns its scratch.)  The split-KV partials live in a device array built into the library,

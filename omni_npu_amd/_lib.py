@@ -49,6 +49,8 @@ SIGNATURES = {
     "mla_splitkv_reduce_vup": (c_int32, [P, SZ, P, P, I32, I32, I32, I32, I32, P, I64, I64, P, I64, I64, P]),
     "mla_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                   I32, I32, F32, P, I64, I64, P, P, SZ, I32, P]),
+    "mla_decode_bf16_step": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, P, I64, P, P, I64,
+                                       I32, P, P, I32, I32, I32, F32, P, I64, I64, P, P, SZ, I32, P]),
     "mla_decode_bf16_static": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, P, I64, I32, P, P, I32,
                                          I32, I32, F32, P, I64, I64, P, I32, P]),
     "mla_prefill_varlen": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, P, I64, I64, P, P, I32, I32, I32, I32,

@@ -41,7 +41,9 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
                                      int32_t max_q_len, int32_t num_heads, float scale, void* workspace,
                                      size_t workspace_bytes, int32_t num_splits, const int32_t* sparse_rows,
                                      int64_t sparse_stride, int32_t page_size, bool fp8, hipStream_t stream,
-                                     const int32_t* win_skip = nullptr, int32_t win_sink = 0, int32_t win_size = 0) {
+                                     const int32_t* win_skip = nullptr, int32_t win_sink = 0, int32_t win_size = 0,
+                                     const void* new_c = nullptr, int64_t new_c_stride = 0, const void* new_r = nullptr,
+                                     int64_t new_r_stride = 0, const int64_t* new_slots = nullptr) {
   MLA_REQUIRE(q_nope && q_rope && nope_cache && rope_cache && (block_table || sparse_rows) && seq_lens, MLA_ERR_NULL,
               "mla_decode_bf16: null pointer argument");
   MLA_REQUIRE(batch >= 0 && max_q_len >= 1 && num_heads >= 1 && num_splits >= 1 && (sparse_rows || max_blocks >= 1) &&
@@ -82,6 +84,8 @@ static int decode_split_impl(const void* q_nope, int64_t qn_stride_t, int64_t qn
   v.sparse_rows = sparse_rows; v.sparse_stride = sparse_stride; v.page_size = page_size;
   v.cache8 = fp8 ? (const uint8_t*)nope_cache : nullptr; v.c8_sp = nope_page_stride;
   v.win_skip = win_skip; v.win_sink = win_sink; v.win_size = win_size;
+  v.new_c = (const __bf16*)new_c; v.new_c_st = new_c_stride; v.new_r = (const __bf16*)new_r; v.new_r_st = new_r_stride;
+  v.new_slots = new_slots;
   // one workgroup per (balanced chunk, group of 128 query rows)
   const dim3 grid((unsigned)(batch * num_splits), 1, (unsigned)((r_max + kRowsPerWg - 1) / kRowsPerWg));
   if (fp8) return launch_decode_v3_fp8(v, grid, stream);
@@ -202,6 +206,37 @@ extern "C" int mla_splitkv_reduce(const void* workspace, size_t workspace_bytes,
   cp.out = (__bf16*)out; cp.out_st = out_stride_t; cp.out_sh = out_stride_h;
   cp.lse_out = lse_out; cp.lse_st = num_heads;
   return launch_chunk_reduce(cp, stream);
+}
+
+// A whole decode step in two launches: the cache write of the step's new tokens (the reshape-and-cache in front of the
+// reference's decode, src/omni_npu/attention/backends/mla.py:868-881) rides in the split kernel, then the merge.  Token t
+// of the batch (query_start_loc order, or b * max_q_len + j) brings latent row new_c[t] and rope row new_r[t] for cache row
+// slot_mapping[t]; negative slots are skipped.  The row of key position p of sequence b is stored by the workgroup
+// whose chunk holds p, before that workgroup reads any key, so the result equals mla_cache_write_bf16 followed by
+// mla_decode_bf16 for every sequence whose seq_lens counts its new tokens (the rows of a request with fewer cached keys
+// than query tokens, e.g. an empty padding request, are not written).  With out == NULL only the first launch runs and
+// the partials stay in the workspace for mla_splitkv_reduce.
+extern "C" int mla_decode_bf16_step(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                    int64_t qr_stride_t, int64_t qr_stride_h, void* nope_cache, int64_t nope_page_stride,
+                                    int64_t nope_row_stride, void* rope_cache, int64_t rope_page_stride,
+                                    int64_t rope_row_stride, int64_t num_pages, const void* new_c, int64_t new_c_stride,
+                                    const void* new_r, int64_t new_r_stride, const int64_t* slot_mapping,
+                                    const int32_t* block_table, int64_t bt_stride, int32_t max_blocks,
+                                    const int32_t* seq_lens, const int32_t* query_start_loc, int32_t batch,
+                                    int32_t max_q_len, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                                    int64_t out_stride_h, float* lse_out, void* workspace, size_t workspace_bytes,
+                                    int32_t num_splits, hipStream_t stream) {
+  MLA_REQUIRE(block_table && new_c && new_r && slot_mapping, MLA_ERR_NULL, "mla_decode_bf16_step: null pointer argument");
+  MLA_REQUIRE(new_c_stride % 8 == 0 && new_r_stride % 8 == 0 && (uintptr_t)new_c % 16 == 0 && (uintptr_t)new_r % 16 == 0,
+              MLA_ERR_SHAPE, "mla_decode_bf16_step: the new rows must be 16-byte aligned");
+  int rc = decode_split_impl(q_nope, qn_stride_t, qn_stride_h, q_rope, qr_stride_t, qr_stride_h, nope_cache,
+                             nope_page_stride, nope_row_stride, rope_cache, rope_page_stride, rope_row_stride, num_pages,
+                             block_table, bt_stride, max_blocks, seq_lens, query_start_loc, batch, max_q_len, num_heads,
+                             scale, workspace, workspace_bytes, num_splits, nullptr, 0, kPage, false, stream, nullptr, 0, 0,
+                             new_c, new_c_stride, new_r, new_r_stride, slot_mapping);
+  if (rc != MLA_OK || out == nullptr) return rc;              // (out == NULL: the first launch only, partials in the workspace)
+  return mla_splitkv_reduce(workspace, workspace_bytes, seq_lens, query_start_loc, batch, max_q_len, num_heads, num_splits,
+                            out, out_stride_t, out_stride_h, lse_out, stream);
 }
 
 // Both phases on one stream.

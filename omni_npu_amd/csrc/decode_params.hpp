@@ -27,6 +27,10 @@ struct DecodeParams {
   // blocks between the sink and the window taken out, win_skip[b] is how many were taken out, and a key behind the
   // sink is visible to a row only if it is one of the newest win_size keys the row may see.
   const int32_t* win_skip; int32_t win_sink, win_size;
+  // The step's cache write folded into the dense kernel (null = the cache already holds the new rows): latent row
+  // new_c[t] and rope row new_r[t] of query token t go to cache row new_slots[t] (negative = skip), written by the
+  // workgroup whose chunk holds that key, before it copies any block.
+  const __bf16* new_c; int64_t new_c_st; const __bf16* new_r; int64_t new_r_st; const int64_t* new_slots;
 };
 
 struct ChunkReduceParams {

@@ -100,9 +100,10 @@ typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scala
 // MFMAs, LDS reads and watts on rows that do not exist, so the small forms leave them out: only the wavefronts that own
 // rows run the S phase and the softmax, P.V covers kRG row groups, and the copies move to wavefronts 4..7, which have
 // nothing else to do in the S phase.  The kernel is then bound by the cache stream alone.
-template <bool kSparse, bool kWindow, int kRG = 4>
+template <bool kSparse, bool kWindow, int kRG = 4, bool kWrite = false>
 __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p) {
   static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
+  static_assert(!kWrite || (!kSparse && !kWindow), "the folded cache write belongs to the dense kernel");
   static_assert(kRG == 1 || kRG == 2 || kRG == 4, "row groups");
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
@@ -236,6 +237,31 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     else if (qsl) { q0 = qsl[b]; qlen = qsl[b + 1] - q0; }
     else { q0 = b * mq; qlen = mq; }
     qlen = qlen < mq ? qlen : mq;
+  }
+  if constexpr (kWrite) {
+    // The step's cache write, folded in: the rows of this request's query tokens are the keys L - qlen .. L - 1; those
+    // that lie in this segment's blocks are stored now (token j by wavefront j: 64 lanes x 16 bytes of latent, 8 lanes of
+    // rope), and every store has been acknowledged before any wavefront asks for a block.  Each key belongs to exactly
+    // one chunk, so a row is written by the workgroups that are going to read it and by nobody else (with more than 128
+    // query rows the row groups of the chunk each store the same bytes: none of them may read before its own store).
+    {
+      KernArgPtr kp = cold();
+      for (int j = wave; j < qlen; j += 8) {
+        const int pos = L - qlen + j;
+        if (pos < blk_begin * kBlk || pos >= blk_end * kBlk) continue;
+        const int64_t slot = kp->new_slots[q0 + j];
+        if (slot < 0 || slot >= kp->num_pages * kPage) continue;
+        const int64_t pg = slot / kPage, off = slot - pg * kPage;
+        const u32x4 vn = *(const u32x4*)(kp->new_c + (int64_t)(q0 + j) * kp->new_c_st + lane * 8);
+        *(u32x4*)(const_cast<__bf16*>(kp->nope) + pg * kp->nope_sp + off * kp->nope_sr + lane * 8) = vn;
+        if (lane < 8) {
+          const u32x4 vr = *(const u32x4*)(kp->new_r + (int64_t)(q0 + j) * kp->new_r_st + lane * 8);
+          *(u32x4*)(const_cast<__bf16*>(kp->rope) + pg * kp->rope_sp + off * kp->rope_sr + lane * 8) = vr;
+        }
+      }
+      MLA_WAIT_VMCNT(0);
+    }
+    lds_barrier();
   }
   const int rows = qlen * p.num_heads;
   const bool has_rows = kRG == 4 || wave * 16 < rows;         // (small forms: one group of rows, grp = 0)
@@ -998,25 +1024,26 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
 
 }  // namespace v3
 
-template <bool kSparse, bool kWindow, int kRG>
+template <bool kSparse, bool kWindow, int kRG, bool kWrite = false>
 static int launch_form(const DecodeParams& p, dim3 grid, hipStream_t stream) {
-  const int rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<kSparse, kWindow, kRG>, v3::kLdsB, "mla_decode_v3_kernel");
+  const int rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<kSparse, kWindow, kRG, kWrite>, v3::kLdsB, "mla_decode_v3_kernel");
   if (rc != MLA_OK) return rc;
-  hipLaunchKernelGGL((v3::mla_decode_v3_kernel<kSparse, kWindow, kRG>), grid, dim3(512), v3::kLdsB, stream, p);
+  hipLaunchKernelGGL((v3::mla_decode_v3_kernel<kSparse, kWindow, kRG, kWrite>), grid, dim3(512), v3::kLdsB, stream, p);
   return check_launch("mla_decode_v3_kernel");
 }
-template <bool kSparse, bool kWindow>
+template <bool kSparse, bool kWindow, bool kWrite = false>
 static int launch_rows(const DecodeParams& p, dim3 grid, hipStream_t stream) {
   // requests with at most 32 / 64 query rows (tokens x heads) take the forms that leave the missing rows out
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
-  if (r_max <= 32) return launch_form<kSparse, kWindow, 1>(p, grid, stream);
-  if (r_max <= 64) return launch_form<kSparse, kWindow, 2>(p, grid, stream);
-  return launch_form<kSparse, kWindow, 4>(p, grid, stream);
+  if (r_max <= 32) return launch_form<kSparse, kWindow, 1, kWrite>(p, grid, stream);
+  if (r_max <= 64) return launch_form<kSparse, kWindow, 2, kWrite>(p, grid, stream);
+  return launch_form<kSparse, kWindow, 4, kWrite>(p, grid, stream);
 }
 
 int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream) {
   if (sparse) return launch_rows<true, false>(p, grid, stream);
   if (p.win_skip) return launch_rows<false, true>(p, grid, stream);
+  if (p.new_c) return launch_rows<false, false, true>(p, grid, stream);
   return launch_rows<false, false>(p, grid, stream);
 }
 

@@ -470,7 +470,8 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
            q_len: int = 1, query_start_loc: Optional[torch.Tensor] = None, lse_out: Optional[torch.Tensor] = None,
            num_splits: Optional[int] = None, max_seq_len: Optional[int] = None,
            workspace: Optional[torch.Tensor] = None, phase: str = "both",
-           w_uv: Optional[torch.Tensor] = None, sink_len: int = 0, window: Optional[int] = None) -> torch.Tensor:
+           w_uv: Optional[torch.Tensor] = None, sink_len: int = 0, window: Optional[int] = None,
+           new_rows: Optional[tuple] = None) -> torch.Tensor:
     """Absorbed-MLA paged decode (reference: FIA decode call, src/omni_npu/attention/backends/mla.py:781-804).
 
     q_nope [T,N,512], q_rope [T,N,64] (any token/head strides), caches [nblk,128,512] / [nblk,128,64],
@@ -484,7 +485,30 @@ def decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.Tensor,
     With ``window`` the call is the static-sink + sliding-window decode of mla.py:705-779 as one attention: the first
     ``sink_len`` keys of every block-table row are the sink, ``seq_lens`` counts the keys behind them, and a token sees
     the sink plus the newest ``window`` keys it may see.
+    ``new_rows`` = (kv_c [T,512], k_pe [T,64] or [T,1,64], slot_mapping int64 [T]): the step's cache write
+    (mla.py:868-881) rides in the split kernel instead of being a launch of its own; the caches must hold the rows
+    of every earlier token, and ``seq_lens`` counts the new ones.
     """
+    if new_rows is not None:
+        if window is not None or w_uv is not None or phase not in ("both", "split"):
+            raise ValueError("decode: new_rows goes with the plain decode (both phases, or the split phase alone)")
+        kv_c, k_pe, slots = new_rows
+        k_pe = k_pe.reshape(k_pe.shape[0], -1)
+        t = q_nope.shape[0]
+        _need_cuda(kv_c, k_pe, slots)
+        if kv_c.shape != (t, D_NOPE) or k_pe.shape != (t, D_ROPE) or kv_c.dtype != torch.bfloat16 or \
+                k_pe.dtype != torch.bfloat16 or kv_c.stride(-1) != 1 or k_pe.stride(-1) != 1:
+            raise ValueError(f"decode: new rows must be bf16 [T,{D_NOPE}] and [T,{D_ROPE}] with contiguous last dims")
+        if slots.dtype != torch.int64 or slots.numel() < t or not slots.is_contiguous():
+            raise TypeError("decode: slot_mapping must be contiguous int64 with an entry per query token")
+        lib, front, ws_args, lse_p, st, qsl, seq_lens, b, n, num_splits = _decode_args(
+            q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out, D_NOPE, q_len, query_start_loc,
+            lse_out, num_splits, max_seq_len, workspace)
+        rc = lib.mla_decode_bf16_step(*front[:13], kv_c.data_ptr(), kv_c.stride(0), k_pe.data_ptr(), k_pe.stride(0),
+                                      slots.data_ptr(), *front[13:], out.data_ptr() if phase == "both" else None,
+                                      out.stride(0), out.stride(1), lse_p, *ws_args, num_splits, st)
+        _lib.check(rc, "mla_decode_bf16_step")
+        return out
     if window is not None:
         return _decode_window(q_nope, q_rope, nope_cache, rope_cache, block_table, seq_lens, scale, out, q_len,
                               query_start_loc, lse_out, num_splits, max_seq_len, workspace, phase, w_uv, sink_len, window)

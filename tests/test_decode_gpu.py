@@ -362,3 +362,43 @@ def test_decode_step_with_many_partials_replayed_from_a_hip_graph(dev):
         O.cache_write(ref_rope, sl, c["new_r"])
         ref = O.absorbed_decode(q1, c["q_rope"], ref_nope, ref_rope, c["block_table"], new_lens, c["scale"])
         attn_close(got, ref, MAX_ABS, MEAN_REL)
+
+
+@pytest.mark.parametrize("batch,heads,q_len,lo,hi,splits", [
+    (5, 128, 1, 100, 900, 3), (4, 128, 2, 31, 700, 2), (3, 128, 4, 30, 40, 1), (6, 16, 1, 60, 500, 2), (3, 40, 2, 64, 66, 5),
+    (2, 128, 3, 1025, 1100, 4), (7, 8, 2, 2, 300, None),
+])
+def test_decode_step_with_the_cache_write_folded_in_equals_the_two_launches(dev, batch, heads, q_len, lo, hi, splits):
+    """mla_decode_bf16_step (the new tokens' rows stored by the split kernel's workgroups before they read) leaves the
+    caches and the output exactly as mla_cache_write_bf16 followed by mla_decode_bf16 does: query tokens whose keys
+    straddle block and chunk borders, padded slots, ragged query lengths."""
+    from omni_npu_amd import kernels as K
+    c = O.make_decode_case(batch, heads, lo, hi, seed=77 + batch, q_len=q_len)
+    t = batch * q_len
+    slots = c["slot_mapping"].clone()
+    if batch > 3:
+        slots[q_len * 2] = -1                                  # a padded slot: that row is not written by either path
+    outs, caches = [], []
+    for fused in (False, True):
+        nope, rope = c["nope"].to(dev), c["rope"].to(dev)
+        out = torch.full((t, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+        lse = torch.full((t, heads), float("nan"), dtype=torch.float32, device=dev)
+        args = [c[k].to(dev) for k in ("q_nope", "q_rope")] + [nope, rope, c["block_table"].to(dev), c["seq_lens"].to(dev)]
+        new = (c["new_c"].to(dev), c["new_r"].to(dev), slots.to(dev))
+        if fused:
+            K.decode(*args, c["scale"], out, q_len=q_len, num_splits=splits, lse_out=lse, new_rows=new)
+        else:
+            K.cache_write(new[0], new[1], new[2], nope, rope)
+            K.decode(*args, c["scale"], out, q_len=q_len, num_splits=splits, lse_out=lse)
+        torch.cuda.synchronize()
+        outs.append((out.cpu(), lse.cpu()))
+        caches.append((nope.cpu(), rope.cpu()))
+    assert torch.equal(caches[0][0].view(torch.int16), caches[1][0].view(torch.int16)), "latent cache differs"
+    assert torch.equal(caches[0][1].view(torch.int16), caches[1][1].view(torch.int16)), "rope cache differs"
+    assert not torch.equal(caches[1][0], c["nope"])           # (and rows were written at all)
+    assert torch.equal(outs[0][0].view(torch.int16), outs[1][0].view(torch.int16)), "outputs differ"
+    assert torch.equal(outs[0][1], outs[1][1]), "log-sum-exps differ"
+    ref_n, ref_r = c["nope"].clone(), c["rope"].clone()
+    O.cache_write(ref_n, slots, c["new_c"])
+    O.cache_write(ref_r, slots, c["new_r"])
+    assert torch.equal(caches[1][0], ref_n) and torch.equal(caches[1][1], ref_r)
