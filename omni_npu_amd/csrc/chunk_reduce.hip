@@ -43,9 +43,11 @@ typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scala
 // sixteen per pass, and the running states are merged through LDS at the end.
 // With one chunk per sequence (large batches) a row has one partial, or two where a chunk border falls inside its
 // sequence: the kFew form then gives a wavefront four rows of two partials, a quarter of the wavefronts and rounds.
-// (eight partials per pass in the one-wavefront form: the eight segments of a sparse-attention token in one pass, 121
-// registers, still four wavefronts per SIMD; six measured 1 us slower there and on four to five partials per row)
-constexpr int kRedPartsNarrow = 8, kRedPartsWide = 16, kRedPartsFew = 2, kRedRowsFew = 4;
+// (four partials per pass in the one-wavefront form: 69 registers, seven wavefronts per SIMD, so the 8192 rows of the
+// headline batch are resident in one round; a row with five or eight partials takes a second pass.  Eight per pass - 121
+// registers, four wavefronts per SIMD, two rounds - measured 1 to 3 us slower per step on both shapes, five and six in
+// between)
+constexpr int kRedPartsNarrow = 4, kRedPartsWide = 16, kRedPartsFew = 2, kRedRowsFew = 4;
 template <bool kWide, bool kFew, int kWideWaves = 4>
 __global__ __launch_bounds__(kWide ? 64 * kWideWaves : 256) void mla_chunk_reduce_kernel(const ChunkReduceParams p) {
   constexpr int kRedParts = kWide ? kRedPartsWide : (kFew ? kRedPartsFew : kRedPartsNarrow);

@@ -252,47 +252,43 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
       lds_barrier();
       if (tile + 1 < tiles) issue(tile + 1, lds0 + ((tile + 1) & 1) * kPfBufB);
       const int key_base = tile * kPfTile;
+      // V of this tile goes from bf16 to fp16 where it lies (thread t takes the 16-byte pieces t, t + 256, ...), then a
+      // barrier: the four wavefronts read each other's pieces.  (Tried: the conversion's arithmetic and writes behind the
+      // first block's score MFMAs, and the next tile converted between the two blocks of this one - both slower.)
       char* vt = buf + kPfKnB + kPfKrB + (int)threadIdx.x * 16;
+      {
+        u32x4 w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = *(const u32x4*)(vt + i * 4096);
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float f_lo = __builtin_bit_cast(float, w[i][e] << 16);
+            const float f_hi = __builtin_bit_cast(float, w[i][e] & 0xffff0000u);
+            w[i][e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(f_lo, f_hi));
+          }
+#pragma unroll
+        for (int i = 0; i < 4; i++) *(u32x4*)(vt + i * 4096) = w[i];
+      }
+      lds_barrier();
 #pragma unroll 1
       for (int tb = 0; tb < 2; tb++) {
-        // (every wavefront runs both rounds, so the barrier below is reached by all; what a wavefront skips is wave-uniform)
-        const bool active = key_base + tb * 32 < wave_max_limit    // else behind everything a row of this wavefront sees
-                            && key_base + tb * 32 + 32 > wg_lo;     // else in front of every row's window
-        // the V conversion of this tile rides on the first block's score MFMAs: reads before, arithmetic and writes behind
-        u32x4 w[4];
-        if (tb == 0) {
-#pragma unroll
-          for (int i = 0; i < 4; i++) w[i] = *(const u32x4*)(vt + i * 4096);
-        }
+        const bool active = key_base + tb * 32 < wave_max_limit && key_base + tb * 32 + 32 > wg_lo;
+        if (!active) continue;
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
-          if (!active) break;
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 256 + koff[kk]);
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
         }
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
-          if (!active) break;
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 128 + roff[kk]);
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[8 + kk], s, 0, 0, 0);
         }
-        if (tb == 0) {
-#pragma unroll
-          for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const float f_lo = __builtin_bit_cast(float, w[i][e] << 16);
-              const float f_hi = __builtin_bit_cast(float, w[i][e] & 0xffff0000u);
-              w[i][e] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(f_lo, f_hi));
-            }
-#pragma unroll
-          for (int i = 0; i < 4; i++) *(u32x4*)(vt + i * 4096) = w[i];
-          lds_barrier();
-        }
-        if (!active) continue;
         // Only blocks that some row of this wave cannot see in full pay for the mask (causal diagonal, end of the keys,
         // rows past the end of the sequence); everywhere else the scores go straight to the maximum.  The scale is
         // folded into the exponent's multiply-add (scale > 0, so the maximum of the raw scores is the raw maximum).
