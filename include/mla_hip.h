@@ -385,6 +385,17 @@ int dsa_sparse_decode_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_s
                            float scale, void* out, int64_t out_stride_t, int64_t out_stride_h, float* lse_out,
                            void* workspace, size_t workspace_bytes, int32_t num_splits, mlahip_stream_t stream);
 
+/* The same sparse attention with the work split over HEADS instead of keys: a workgroup owns (token, 16 heads), walks all
+ * of the token's rows and writes the bf16 result itself - one launch, no workspace, nothing to merge (the form for many
+ * heads and a few thousand selected keys per token: attention/backends/dsa.py:259-291 at decode).  num_heads a multiple
+ * of 16; the caches are addressed as flat rows (num_rows of them, row strides in elements), i.e. pages must be contiguous. */
+int dsa_sparse_decode_heads_bf16(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_rope,
+                                 int64_t qr_stride_t, int64_t qr_stride_h, const void* nope_cache, int64_t nope_row_stride,
+                                 const void* rope_cache, int64_t rope_row_stride, int64_t num_rows,
+                                 const int32_t* sparse_rows, int64_t sparse_stride, const int32_t* counts,
+                                 int32_t num_tokens, int32_t num_heads, float scale, void* out, int64_t out_stride_t,
+                                 int64_t out_stride_h, float* lse_out /* fp32 [T,N] or NULL */, mlahip_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -67,6 +67,8 @@ SIGNATURES = {
     "dsa_build_rows": (c_int32, [P, I64, P, I64, I32, P, P, I32, I32, I32, I32, I64, P, I64, P, P]),
     "dsa_sparse_decode_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, I64, P, I64, I64, I64, I32, P, I64, P, I32, I32,
                                          F32, P, I64, I64, P, P, SZ, I32, P]),
+    "dsa_sparse_decode_heads_bf16": (c_int32, [P, I64, I64, P, I64, I64, P, I64, P, I64, I64, P, I64, P, I32, I32, F32, P, I64,
+                                               I64, P, P]),
 }
 
 

@@ -694,10 +694,16 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
                   rows: torch.Tensor, counts: torch.Tensor, scale: float, out: torch.Tensor,
                   lse_out: Optional[torch.Tensor] = None, num_splits: Optional[int] = None,
                   workspace: Optional[torch.Tensor] = None, w_uv: Optional[torch.Tensor] = None,
-                  counts_bounded: bool = False) -> torch.Tensor:
+                  counts_bounded: bool = False, method: str = "auto") -> torch.Tensor:
     """Absorbed MLA of token t over cache rows rows[t, :counts[t]] (reference: npu_sparse_flash_attention call,
     src/omni_npu/attention/backends/dsa.py:259-291).  out bf16 viewed as [T,N,512]; with ``w_uv`` (bf16 [N,512,128])
     the value up-projection of dsa.py:233-240 is fused into the merge and out is [T, N*128] / [T,N,128].
+
+    ``method``: "keys" cuts every token's keys into ``num_splits`` chunks (split-KV partials + merge: the form for few
+    heads or few tokens); "heads" gives every (token, 16 heads) a workgroup that walks all of the token's keys and
+    writes the result itself (one launch, no scratch, every probability carried as two bf16 numbers; heads a multiple
+    of 16, no ``w_uv``).  Measured at 32 tokens x 128 heads x 2048 keys: 56 us against 50 us for "keys" (split + merge),
+    so "auto" is "keys"; the form is there for callers without scratch memory.
 
     counts[t] must not exceed rows.shape[1]; unless the caller vouches for that (``counts_bounded``: the counts come from
     build_sparse_rows / topk_rows) they are clamped here.  Many tokens (a prefill chunk) run as several launches so that
@@ -722,6 +728,24 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
         raise TypeError("sparse_decode: lse_out must be contiguous fp32 [T,N]")
     if not counts_bounded:
         counts = counts[:t].clamp(max=rows.shape[1])
+    if method not in ("auto", "keys", "heads"):
+        raise ValueError(f"sparse_decode: unknown method {method!r}")
+    heads_ok = w_uv is None and n % 16 == 0 and nope.stride(0) == nope.shape[1] * nope.stride(1) and \
+        rope.stride(0) == rope.shape[1] * rope.stride(1)
+    if method == "heads" and not heads_ok:
+        raise ValueError("sparse_decode: the heads form wants a multiple of 16 heads, contiguous cache pages and no w_uv")
+    if method == "heads":
+        st = _stream(q_nope)
+        for t0 in range(0, t, 1 << 20):
+            t1 = min(t, t0 + (1 << 20))
+            qn, qr, rw, ct, oc = q_nope[t0:t1], q_rope[t0:t1], rows[t0:t1], counts[t0:t1], out[t0:t1]
+            rc = lib.dsa_sparse_decode_heads_bf16(
+                qn.data_ptr(), qn.stride(0), qn.stride(1), qr.data_ptr(), qr.stride(0), qr.stride(1), nope.data_ptr(),
+                nope.stride(1), rope.data_ptr(), rope.stride(1), nope.shape[0] * nope.shape[1], rw.data_ptr(), rw.stride(0),
+                ct.data_ptr(), t1 - t0, n, float(scale), oc.data_ptr(), oc.stride(0), oc.stride(1),
+                lse_out.view(t, n)[t0:t1].data_ptr() if lse_out is not None else None, st)
+            _lib.check(rc, "dsa_sparse_decode_heads_bf16")
+        return out
     if num_splits is None:
         num_splits = default_num_splits(t, 1, n, rows.shape[1])
     per_token = lib.mla_decode_workspace_bytes(1, 1, n, num_splits)

@@ -269,3 +269,92 @@ def test_quant_qk_in_one_launch_equals_the_two_launches(dev):
     sm = slots.cpu()
     ok = sm >= 0
     assert torch.equal(a[2].cpu().view(-1, 128)[sm[ok]], ref8.view(torch.uint8)[ok]) and torch.equal(a[3].cpu().view(-1)[sm[ok]], refs[ok])
+
+
+def _sparse_case(batch, heads, lens, counts, seed):
+    """Row lists over a paged cache: token b attends to counts[b] distinct keys of its sequence (ascending positions)."""
+    c = O.make_decode_case(batch, heads, min(lens), max(lens), seed=seed, q_len=1)
+    k = max(max(counts), 1)
+    g = torch.Generator().manual_seed(seed)
+    idx = torch.full((batch, k), -1, dtype=torch.int32)
+    rows = torch.zeros(batch, k, dtype=torch.int32)
+    cnt = torch.zeros(batch, dtype=torch.int32)
+    for b in range(batch):
+        L = int(c["seq_lens"][b])
+        n = min(counts[b], L)
+        pos = torch.randperm(L, generator=g)[:n].sort().values
+        idx[b, :n] = pos.to(torch.int32)
+        rows[b, :n] = O.slots_for(c["block_table"], b, 0, L)[pos].to(torch.int32)
+        cnt[b] = n
+    return c, idx, rows, cnt
+
+
+@pytest.mark.parametrize("batch,heads,counts", [
+    (3, 128, [2048, 2048, 2048]), (8, 128, [1, 63, 64, 65, 128, 129, 700, 0]), (5, 16, [40, 7, 200, 64, 1]),
+    (2, 32, [300, 17]), (16, 64, [100 + 13 * i for i in range(16)]),
+])
+def test_sparse_decode_split_over_heads_matches_the_oracle_and_the_split_over_keys(dev, batch, heads, counts):
+    """dsa_sparse_decode_heads_bf16 (a workgroup per (token, 16 heads) over all of the token's rows, no partials, no merge)
+    against the oracle and against the split-KV form: attention within the bf16 bar, and - every probability going through
+    P.V as two bf16 numbers - within 1.6e-3 of mean relative error; log-sum-exps within 1e-4 of the other form's; an empty
+    row list gives zeros and -inf."""
+    from omni_npu_amd import kernels as K
+    c, idx, rows, cnt = _sparse_case(batch, heads, [2100] * batch if max(counts) > 1000 else [800] * batch, counts, seed=61 + batch)
+    ref, ref_lse = O.sparse_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], idx,
+                                   c["scale"], return_lse=True)
+    args = [c[x].to(dev) for x in ("q_nope", "q_rope", "nope", "rope")]
+    got = {}
+    for method in ("keys", "heads"):
+        out = torch.full((batch, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+        lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device=dev)
+        K.sparse_decode(*args, rows.to(dev), cnt.to(dev), c["scale"], out, lse_out=lse, method=method)
+        torch.cuda.synchronize()
+        got[method] = (out.cpu(), lse.cpu())
+    ma, mr = attn_close(got["heads"][0], ref, 2e-2, 2e-3)
+    assert mr <= 1.6e-3, mr
+    attn_close(got["keys"][0], ref, 2e-2, 2e-3)
+    fin = torch.isfinite(ref_lse)
+    assert torch.equal(torch.isfinite(got["heads"][1]), fin)
+    assert torch.allclose(got["heads"][1][fin], ref_lse[fin], atol=2e-3, rtol=0)
+    assert torch.allclose(got["heads"][1][fin], got["keys"][1][fin], atol=1e-4, rtol=0)
+    empty = cnt == 0
+    assert (got["heads"][0][empty] == 0).all() and torch.isinf(got["heads"][1][empty]).all()
+
+
+def test_sparse_decode_over_heads_starts_over_when_a_score_outgrows_its_reference(dev):
+    """The references are fixed on the first 64 keys; a key further on whose score lies more than 2^100 above them makes
+    the workgroup run the token again with the maxima it has seen.  Planted: one key, scaled so that its score against
+    every head exceeds the first tile's by several hundred (log2)."""
+    from omni_npu_amd import kernels as K
+    c, idx, rows, cnt = _sparse_case(2, 32, [900, 900], [600, 500], seed=91)
+    q = c["q_nope"].float()
+    big = int(idx[0, 400])                                    # a key position far behind the first tile of token 0
+    slot = int(O.slots_for(c["block_table"], 0, big, big + 1)[0])
+    # make the key point along every head's query at once: the sum of the heads' (sign-aligned) queries, large
+    direction = q[0].sum(0)
+    c["nope"].view(-1, 512)[slot] = (direction / direction.norm() * 60.0).bfloat16()
+    c["q_nope"][0] = (q[0] + direction / direction.norm() * 40.0).bfloat16()     # every head sees it: score ~ 60 * 40 * scale
+    ref = O.sparse_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], idx, c["scale"])
+    args = [c[x].to(dev) for x in ("q_nope", "q_rope", "nope", "rope")]
+    out = torch.full((2, 32, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.sparse_decode(*args, rows.to(dev), cnt.to(dev), c["scale"], out, method="heads")
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    # token 0 is (nearly) the planted key's latent vector; bf16 of values up to 60 -> looser absolute bar there
+    err = (out.float().cpu() - ref).abs()
+    assert err[1].max() <= 2e-2 and err[0].max() <= 60.0 * 2 ** -8 + 2e-2
+    assert (err.sum() / ref.abs().sum()).item() <= 2e-3
+
+
+def test_sparse_decode_method_choice_and_refusals(dev):
+    from omni_npu_amd import kernels as K
+    c, idx, rows, cnt = _sparse_case(2, 24, [300, 300], [100, 50], seed=5)     # 24 heads: no multiple of 16
+    args = [c[x].to(dev) for x in ("q_nope", "q_rope", "nope", "rope")]
+    out = torch.zeros(2, 24, 512, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError, match="multiple of 16"):
+        K.sparse_decode(*args, rows.to(dev), cnt.to(dev), c["scale"], out, method="heads")
+    with pytest.raises(ValueError, match="unknown method"):
+        K.sparse_decode(*args, rows.to(dev), cnt.to(dev), c["scale"], out, method="rows")
+    K.sparse_decode(*args, rows.to(dev), cnt.to(dev), c["scale"], out)          # auto -> the split form
+    ref = O.sparse_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], idx, c["scale"])
+    attn_close(out, ref, 2e-2, 2e-3)
