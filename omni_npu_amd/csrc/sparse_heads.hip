@@ -19,6 +19,13 @@
 //     above it makes the workgroup start over with the maxima seen so far), and publish P^T as TWO bf16 numbers per
 //     probability (value and rounding remainder: 16 significant bits go through P.V);
 //   * all eight wavefronts compute O^T += V^T P^T for their 64 output columns (transposed LDS reads of the same tile).
+//
+// Measured, 32 tokens x 128 heads x 2048 keys: 56 us, against 50 us for the split over keys + merge.  Without the copies
+// the same loop takes 42 us, without the P.V MFMAs 66 (of 72 in that build), without the score MFMAs 65: the time is the
+// chain barrier -> LDS reads -> dependent MFMAs -> barrier of a tile, which one wavefront per SIMD and phase does not
+// hide, not matrix or memory throughput.  Two other schedules were slower: the copies shared by all eight wavefronts (0..3
+// issuing theirs between their P.V MFMAs), 71 us; the tile in four column panels with wavefronts 4..7 doing P.V of
+// tile t-1 and the copy of tile t+1 beside the scores of tile t, one barrier per tile, 83 us.
 #include "mla_common.hpp"
 #include "decode_params.hpp"
 
