@@ -287,9 +287,13 @@ class NPUDSAImpl(MLACommonBaseImpl[NPUDSAMetadata]):
                              self.qk_nope_head_dim + self.v_head_dim), device=k_c_normed.device, dtype=k_c_normed.dtype)
             # the profile run sizes the KV cache: the split-KV scratch a real prefill will need (bounded by
             # SPARSE_WORKSPACE_CAP whatever the chunk size) is allocated now, so that it is counted
+            # (for the split count the real steps will pick; scratch is kept per stream, so a runner that captures its graphs
+            # on another stream pays this once more there: at most SPARSE_WORKSPACE_CAP per stream that runs steps)
             if k_c_normed.is_cuda:
                 toks = max(int(k_c_normed.shape[0]), 1)
-                need = K._lib.load().mla_decode_workspace_bytes(min(toks, 32768), 1, self.num_heads, 1)
+                k_sel = int(self.indexer.topk_indices_buffer.shape[-1]) if self.indexer is not None else 2048
+                splits = K.default_num_splits(toks, 1, self.num_heads, k_sel)
+                need = K._lib.load().mla_decode_workspace_bytes(min(toks, 32768), 1, self.num_heads, splits)
                 K._workspace(k_c_normed.device, min(need, K.SPARSE_WORKSPACE_CAP))
             return output.fill_(0)
 
