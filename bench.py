@@ -1048,10 +1048,9 @@ def main():
     ap.add_argument("--no-power-probe", action="store_true",
                     help="decode, fp8 and prefill workloads: skip the two seconds of queued launches under the socket power reading")
     ap.add_argument("--graph", action="store_true",
-                    help="decode workload: replay the steps from captured HIP graphs instead of launching their kernels one by "
-                         "one.  Measured slower on this part: a graph leaves no idle time between kernels, the engine clock "
-                         "drops within a millisecond, and every kernel of the graph runs 25-30 % longer than in the eager "
-                         "queue, whose few microseconds between launches keep the clock up")
+                    help="decode workload: time the steps as replays of captured HIP graphs (--graph-layers steps per graph) "
+                         "instead of eager launches; the default line carries the one-step-per-graph figure either way "
+                         "(step_us.hip_graph_replay)")
     ap.add_argument("--graph-layers", type=int, default=10,
                     help="with --graph: steps captured into one HIP graph, as a model captures all its layers in one; the "
                          "largest divisor of --steps up to this number is used")
