@@ -95,8 +95,9 @@ __device__ __forceinline__ int wave_incl_scan_dpp(int v) {
 typedef __attribute__((address_space(4))) const int32_t* ConstI32Ptr;   // scalar (constant-cache) loads
 
 
-// kRG = groups of 32 query rows that can hold rows at all (4: any launch; 1 or 2: launches with at most 32 / 64 query rows
-// per request, e.g. the 16 heads a tensor-parallel rank of eight owns).  With few rows the 128-row schedule spends the same
+// kRG = groups of 32 query rows a workgroup handles (4: the general form; 1 or 2: launches with at most 32 / 64 query rows
+// per request, e.g. the 16 heads a tensor-parallel rank of eight owns, and row-list launches whose chunks alone would
+// leave most of the CUs idle, which then give every 32 or 64 rows a workgroup of their own: blockIdx.z).  With few rows the 128-row schedule spends the same
 // MFMAs, LDS reads and watts on rows that do not exist, so the small forms leave them out: only the wavefronts that own
 // rows run the S phase and the softmax, P.V covers kRG row groups, and the copies move to wavefronts 4..7, which have
 // nothing else to do in the S phase.  The kernel is then bound by the cache stream alone.
@@ -105,6 +106,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   static_assert(!(kSparse && kWindow), "the window variant reads the paged cache");
   static_assert(!kWrite || (!kSparse && !kWindow), "the folded cache write belongs to the dense kernel");
   static_assert(kRG == 1 || kRG == 2 || kRG == 4, "row groups");
+  constexpr int kGrpRows = 32 * kRG;                          // query rows of one workgroup (blockIdx.z counts such groups)
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // 0..7
@@ -124,7 +126,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     chunk = (lin & 7) * (gridDim.x >> 3) + j / gridDim.z;
   }
   const int r_max = p.max_q_len * p.num_heads;
-  if (grp * 128 >= r_max) return;
+  if (grp * kGrpRows >= r_max) return;
   const uint32_t lds0 = lds_addr_of(lds);
   // Arguments that only the start and the end of a segment need are read from the argument block where they are used
   // (through a pointer the compiler cannot see through), not held in scalar registers across the block loop: the loop
@@ -264,12 +266,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     lds_barrier();
   }
   const int rows = qlen * p.num_heads;
-  const bool has_rows = kRG == 4 || wave * 16 < rows;         // (small forms: one group of rows, grp = 0)
+  const bool has_rows = kRG == 4 || (wave * 16 < kGrpRows && grp * kGrpRows + wave * 16 < rows);
 
   // this lane's query row for QK / softmax; the four lanes l16 + 16*g share it
-  const int rloc = wave * 16 + l16;                           // row inside the group of 128
-  const int row = grp * 128 + rloc;
-  const bool row_ok = row < rows && L > 0;
+  const int rloc = wave * 16 + l16;                           // row inside the group (the small forms use the first kGrpRows)
+  const int row = grp * kGrpRows + rloc;
+  const bool row_ok = row < rows && rloc < kGrpRows && L > 0;
   const int t_local = row / p.num_heads;
   const int head = row - t_local * p.num_heads;
   {
@@ -290,10 +292,10 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   }
   const int win_skip = kWindow ? p.win_skip[b] : 0;
   const int win_blk0 = kWindow ? p.win_sink / kBlk : 0;
-  const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
+  const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * kGrpRows;   // + row index in the group
 
-  if (grp * 128 >= rows) {
-    if (row < r_max && g == 0) { KernArgPtr kp = cold(); kp->lse_part[part_base + rloc] = -INFINITY; kp->corr_scale[part_base + rloc] = 0.f; }
+  if (grp * kGrpRows >= rows) {
+    if (row < r_max && rloc < kGrpRows && g == 0) { KernArgPtr kp = cold(); kp->lse_part[part_base + rloc] = -INFINITY; kp->corr_scale[part_base + rloc] = 0.f; }
     continue;
   }
 
@@ -506,7 +508,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     KernArgPtr kp = cold();
     const int ln = lane_now();
     const int nh = kp->num_heads;
-    const int r0 = grp * 128 + wave * 16;                    // the wave's first row
+    const int r0 = grp * kGrpRows + wave * 16;               // the wave's first row
     {
       // latent part: row k of the wave is one copy instruction; lane i brings granule i ^ swz(k) (the tile swizzle)
       int t = r0 / nh, h = r0 - t * nh;
@@ -939,8 +941,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   const int e_l16 = e_ln & 15, e_g = e_ln >> 4, e_h32 = e_ln & 31, e_half = e_ln >> 5;
   const int e_rloc = wave * 16 + e_l16;
   {
-    const int e_row = grp * 128 + e_rloc;
-    const bool e_row_ok = e_row < rows && L > 0;
+    const int e_row = grp * kGrpRows + e_rloc;
+    const bool e_row_ok = e_row < rows && e_rloc < kGrpRows && L > 0;
     // the row's four lanes combine their sums and their candidates for the dominant key
     float l_tot = l_run + __shfl_xor(l_run, 16, 64);
     l_tot += __shfl_xor(l_tot, 32, 64);
@@ -980,7 +982,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     }
     if (e_g == 0) {
       *(float*)(lds + kPOff + (e_rloc & 31) * 16 + (e_rloc >> 5) * 4) = inv;
-      if (e_row < r_max) {
+      if (e_row < r_max && e_rloc < kGrpRows) {
         const int64_t pr = part_base + e_rloc;
         kp->lse_part[pr] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
         kp->corr_scale[pr] = corr;
@@ -1015,7 +1017,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
   for (int it = 0; it < 8 * kRG; it++) {
     const int srow = it * 4 + e_g;
     const u32x2 v = *(const u32x2*)(stage + srow * 128 + ((e_l16 ^ ((srow >> 1) & 15)) << 3));
-    if (grp * 128 + srow < r_max)
+    if (grp * kGrpRows + srow < r_max)
       *(u32x2*)(o_part_c + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1031,12 +1033,23 @@ static int launch_form(const DecodeParams& p, dim3 grid, hipStream_t stream) {
   hipLaunchKernelGGL((v3::mla_decode_v3_kernel<kSparse, kWindow, kRG, kWrite>), grid, dim3(512), v3::kLdsB, stream, p);
   return check_launch("mla_decode_v3_kernel");
 }
+constexpr int kNumCUs = 256;                               // MI355X
 template <bool kSparse, bool kWindow, bool kWrite = false>
 static int launch_rows(const DecodeParams& p, dim3 grid, hipStream_t stream) {
   // requests with at most 32 / 64 query rows (tokens x heads) take the forms that leave the missing rows out
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
   if (r_max <= 32) return launch_form<kSparse, kWindow, 1, kWrite>(p, grid, stream);
   if (r_max <= 64) return launch_form<kSparse, kWindow, 2, kWrite>(p, grid, stream);
+  // With few requests and short contexts (and with row lists, which are short by nature) the caller's chunks do not fill
+  // the 256 CUs, and cutting the keys finer makes every workgroup pay a segment's start and end for a handful of blocks.
+  // The rows are cut instead: groups of 64 or 32 rows, each with its own workgroup over the whole chunk (the groups of a
+  // chunk sit next to each other on one XCD and share the cache rows in its L2).  Measured on row lists of 2048 keys,
+  // 128 heads, eight chunks per token: 4 tokens 36.1 -> 26.9 us, 8 tokens 37.7 -> 28.8, 16 tokens 40.4 -> 33.3.
+  {
+    const int64_t wgs = (int64_t)grid.x * grid.z;
+    if (wgs * 4 <= kNumCUs) { grid.z = (unsigned)((r_max + 31) / 32); return launch_form<kSparse, kWindow, 1, kWrite>(p, grid, stream); }
+    if (wgs * 2 <= kNumCUs) { grid.z = (unsigned)((r_max + 63) / 64); return launch_form<kSparse, kWindow, 2, kWrite>(p, grid, stream); }
+  }
   return launch_form<kSparse, kWindow, 4, kWrite>(p, grid, stream);
 }
 

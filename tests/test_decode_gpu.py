@@ -77,8 +77,8 @@ def test_decode_dominant_key_records_name_the_right_cache_row(dev, heads, num_sp
     row's weight must be recorded."""
     from omni_npu_amd import kernels as K
     from omni_npu_amd import _lib
-    case = O.make_decode_case(4, heads, 128, 1024, seed=0)
-    b, n = 4, heads
+    b, n = 256 // (2 * num_splits) + 2, heads            # enough chunks that the launch takes the 128-row form, which is
+    case = O.make_decode_case(b, heads, 128, 1024, seed=0)  # the one that leaves records (fewer: the rows are cut instead)
     nope = case["nope"].to(dev)
     ws = torch.zeros(_lib.load().mla_decode_workspace_bytes(b, 1, n, num_splits), dtype=torch.uint8, device=dev)
     out = torch.empty(b, n, 512, dtype=torch.bfloat16, device=dev)

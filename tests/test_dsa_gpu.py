@@ -321,6 +321,34 @@ def test_sparse_decode_split_over_heads_matches_the_oracle_and_the_split_over_ke
     assert (got["heads"][0][empty] == 0).all() and torch.isinf(got["heads"][1][empty]).all()
 
 
+@pytest.mark.parametrize("batch,heads,counts,splits", [
+    (3, 128, [2048, 2048, 2048], 1), (3, 128, [2048, 1500, 2048], 2), (8, 128, [1, 63, 64, 65, 128, 129, 700, 0], 2),
+    (16, 128, [2048] * 16, 4), (32, 128, [2048] * 31 + [5], 2), (2, 96, [300, 17], 1), (4, 80, [900, 33, 0, 512], 3),
+    (1, 256, [1024], 4),
+])
+def test_sparse_decode_with_few_chunks_cuts_the_rows_instead(dev, batch, heads, counts, splits):
+    """When tokens x chunks would leave most CUs idle the row-list kernel gives every 32 or 64 query rows a workgroup of
+    their own (the small-row forms over several row groups).  Against the oracle, at the margin those forms keep
+    (two-term probabilities), log-sum-exps included; an empty row list gives zeros and -inf; heads that do not fill the
+    last group of rows leave their neighbours' partials alone."""
+    from omni_npu_amd import kernels as K
+    c, idx, rows, cnt = _sparse_case(batch, heads, [2100] * batch if max(counts) > 1000 else [1000] * batch, counts, seed=17 + batch)
+    ref, ref_lse = O.sparse_decode(c["q_nope"], c["q_rope"], c["nope"], c["rope"], c["block_table"], c["seq_lens"], idx,
+                                   c["scale"], return_lse=True)
+    args = [c[x].to(dev) for x in ("q_nope", "q_rope", "nope", "rope")]
+    out = torch.full((batch, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.full((batch, heads), float("nan"), dtype=torch.float32, device=dev)
+    K.sparse_decode(*args, rows.to(dev), cnt.to(dev), c["scale"], out, lse_out=lse, num_splits=splits, method="keys")
+    torch.cuda.synchronize()
+    ma, mr = attn_close(out.cpu(), ref, 2e-2, 2e-3)
+    assert mr <= 1.8e-3, mr
+    fin = torch.isfinite(ref_lse)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert torch.allclose(lse.cpu()[fin], ref_lse[fin], atol=2e-3, rtol=0)
+    empty = cnt == 0
+    assert (out.cpu()[empty] == 0).all()
+
+
 def test_sparse_decode_over_heads_starts_over_when_a_score_outgrows_its_reference(dev):
     """The references are fixed on the first 64 keys; a key further on whose score lies more than 2^100 above them makes
     the workgroup run the token again with the maxima it has seen.  Planted: one key, scaled so that its score against
