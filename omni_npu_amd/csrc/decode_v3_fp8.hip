@@ -109,7 +109,8 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     chunk = (lin & 7) * (gridDim.x >> 3) + j / gridDim.z;
   }
   const int r_max = p.max_q_len * p.num_heads;
-  if (grp * 128 >= r_max) return;
+  constexpr int kGrpRows = 32 * kRG;                          // query rows of one workgroup (blockIdx.z counts such groups)
+  if (grp * kGrpRows >= r_max) return;
   const uint32_t lds0 = lds_addr_of(lds);
   // Arguments that only the start and the end of a segment need are read from the argument block where they are used
   // (through a pointer the compiler cannot see through), not held in scalar registers across the block loop: the loop
@@ -224,12 +225,12 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     qlen = qlen < mq ? qlen : mq;
   }
   const int rows = qlen * p.num_heads;
-  const bool has_rows = kRG == 4 || wave * 16 < rows;         // (small forms: one group of rows, grp = 0)
+  const bool has_rows = kRG == 4 || (wave * 16 < kGrpRows && grp * kGrpRows + wave * 16 < rows);
 
   // this lane's query row for QK / softmax; the four lanes l16 + 16*g share it
   const int rloc = wave * 16 + l16;                           // row inside the group of 128
-  const int row = grp * 128 + rloc;
-  const bool row_ok = row < rows && L > 0;
+  const int row = grp * kGrpRows + rloc;
+  const bool row_ok = row < rows && rloc < kGrpRows && L > 0;
   const int t_local = row / p.num_heads;
   const int head = row - t_local * p.num_heads;
   {
@@ -250,10 +251,10 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   }
   const int win_skip = kWindow ? p.win_skip[b] : 0;
   const int win_blk0 = kWindow ? p.win_sink / kBlk : 0;
-  const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * 128;   // + row index in the group
+  const int64_t part_base = (int64_t)(chunk + b) * r_max + grp * kGrpRows;   // + row index in the group
 
-  if (grp * 128 >= rows) {
-    if (row < r_max && g == 0) { KernArgPtr kp = cold(); kp->lse_part[part_base + rloc] = -INFINITY; kp->corr_scale[part_base + rloc] = 0.f; }
+  if (grp * kGrpRows >= rows) {
+    if (row < r_max && rloc < kGrpRows && g == 0) { KernArgPtr kp = cold(); kp->lse_part[part_base + rloc] = -INFINITY; kp->corr_scale[part_base + rloc] = 0.f; }
     continue;
   }
 
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     KernArgPtr kp = cold();
     const int ln = lane_now();
     const int nh = kp->num_heads;
-    const int r0 = grp * 128 + wave * 16;                    // the wave's first row
+    const int r0 = grp * kGrpRows + wave * 16;               // the wave's first row
     {
       // latent part: row k of the wave is one copy instruction; lane i brings granule i ^ swz(k) (the tile swizzle)
       int t = r0 / nh, h = r0 - t * nh;
@@ -740,7 +741,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   const int e_l16 = e_ln & 15, e_g = e_ln >> 4, e_h32 = e_ln & 31, e_half = e_ln >> 5;
   const int e_rloc = wave * 16 + e_l16;
   {
-    const int e_row = grp * 128 + e_rloc;
+    const int e_row = grp * kGrpRows + e_rloc;
     // the row's four lanes combine their sums
     float l_tot = l_run + __shfl_xor(l_run, 16, 64);
     l_tot += __shfl_xor(l_tot, 32, 64);
@@ -750,7 +751,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
     KernArgPtr kp = cold();
     if (e_g == 0) {
       *(float*)(lds + kPOff + (e_rloc & 31) * 16 + (e_rloc >> 5) * 4) = inv;
-      if (e_row < r_max) {
+      if (e_row < r_max && e_rloc < kGrpRows) {
         const int64_t pr = part_base + e_rloc;
         kp->lse_part[pr] = l_tot > 0.f ? (m_ref + fast_log2(l_tot)) * kLn2 : -INFINITY;
         kp->corr_scale[pr] = corr;
@@ -785,7 +786,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_fp8_kernel(const DecodePara
   for (int it = 0; it < 8 * kRG; it++) {
     const int srow = it * 4 + e_g;
     const u32x2 v = *(const u32x2*)(stage + srow * 128 + ((e_l16 ^ ((srow >> 1) & 15)) << 3));
-    if (grp * 128 + srow < r_max)
+    if (grp * kGrpRows + srow < r_max)
       *(u32x2*)(o_part_c + (part_base + srow) * kDNope + wave * 64 + e_l16 * 4) = v;
   }
   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -807,6 +808,12 @@ static int launch_rows_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream)
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
   if (r_max <= 32) return launch_form_fp8<kWindow, 1>(p, grid, stream);
   if (r_max <= 64) return launch_form_fp8<kWindow, 2>(p, grid, stream);
+  // (few chunks: the rows are cut into groups of 32 or 64 with a workgroup each, as in the kernel over the bf16 cache)
+  {
+    const int64_t wgs = (int64_t)grid.x * grid.z;
+    if (wgs * 4 <= 256) { grid.z = (unsigned)((r_max + 31) / 32); return launch_form_fp8<kWindow, 1>(p, grid, stream); }
+    if (wgs * 2 <= 256) { grid.z = (unsigned)((r_max + 63) / 64); return launch_form_fp8<kWindow, 2>(p, grid, stream); }
+  }
   return launch_form_fp8<kWindow, 4>(p, grid, stream);
 }
 

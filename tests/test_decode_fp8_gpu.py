@@ -32,7 +32,8 @@ def _fill_cache(c, dev):
 
 @pytest.mark.parametrize("batch,heads,lo,hi,q_len,splits", [(4, 16, 128, 1024, 1, 2), (3, 128, 1, 200, 2, 3),
                                                            (5, 128, 60, 700, 1, None), (3, 128, 6000, 9000, 2, None),
-                                                           (4, 128, 100, 800, 2, 2)])
+                                                           (4, 128, 100, 800, 2, 2), (4, 80, 100, 800, 1, 2),
+                                                           (2, 96, 300, 900, 2, 1)])
 def test_decode_fp8_matches_oracle(dev, batch, heads, lo, hi, q_len, splits):
     from omni_npu_amd import kernels as K
     c = _fp8_case(batch, heads, lo, hi, seed=batch, q_len=q_len)
