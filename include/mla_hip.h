@@ -169,10 +169,10 @@ int mla_decode_bf16_step(const void* q_nope, int64_t qn_stride_t, int64_t qn_str
  * MLA_DECODE_STATIC_SCRATCH_BYTES per GPU, held until the process ends; a shape that needs more
  * (mla_decode_workspace_bytes) is refused with -4.  The call allocates and frees nothing.  Calls that overlap in time
  * on one GPU share the array and race: keep them on one stream or order them with events.
- * The FIRST call on each device must run outside stream capture, once per kernel form the caller will use (forms
- * differ by max_q_len x num_heads: up to 32, up to 64, more): it looks the array's address up (which makes the runtime
- * load the code object that holds the array) and raises the kernels' dynamic LDS limit, neither of which may be
- * recorded into a graph.  Every later call only launches kernels and can be captured.  The array is part of the
+ * The FIRST call on each device must run outside stream capture: it looks the array's address up (which makes the
+ * runtime load the code object that holds the array) and raises the dynamic LDS limit of the split kernel in all its
+ * forms, neither of which may be recorded into a graph.  Every later call, of any shape, only launches kernels and can
+ * be captured.  The array is part of the
  * library's image: every process that loads the library pays the 48 MiB on each GPU it touches, whether or not it
  * ever calls this entry point. */
 #define MLA_DECODE_STATIC_SCRATCH_BYTES ((size_t)48 << 20)

@@ -283,6 +283,9 @@ static int static_scratch(void** out) {
     const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr)
       return fail(MLA_ERR_LAUNCH, "mla_decode_bf16_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+    // (every form the entry point may pick later gets its LDS limit now: a later call under capture then only launches)
+    const int rc = prepare_decode_v3_dense_forms();
+    if (rc != MLA_OK) return rc;
     g_scratch_ptr[dev] = ptr;
   }
   *out = g_scratch_ptr[dev];

@@ -56,6 +56,8 @@ int launch_reduce_vup(const ChunkReduceParams& r, const void* w_uv, int64_t w_st
 // The eight-wavefront kernel over the bf16 cache (decode_v3.hip): dense, row-list (sparse) and, with p.win_skip set, sink +
 // window.  Returns 0 or a negative error code.
 int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream);
+// The dynamic-LDS limit of all dense bf16 forms raised on the current device, ahead of a launch under stream capture.
+int prepare_decode_v3_dense_forms();
 // The same over the fp8 block-scaled cache p.cache8 (decode_v3_fp8.hip): dense and, with p.win_skip set, sink + window.
 int launch_decode_v3_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream);
 

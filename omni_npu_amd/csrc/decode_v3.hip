@@ -1053,6 +1053,15 @@ static int launch_rows(const DecodeParams& p, dim3 grid, hipStream_t stream) {
   return launch_form<kSparse, kWindow, 4, kWrite>(p, grid, stream);
 }
 
+// Raises the dynamic-LDS limit of every dense form on the current device (what a launch does for its own form the first
+// time it runs): a caller that will launch under stream capture, where that cannot be recorded, does it beforehand.
+int prepare_decode_v3_dense_forms() {
+  int rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<false, false, 1, false>, v3::kLdsB, "mla_decode_v3_kernel");
+  if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<false, false, 2, false>, v3::kLdsB, "mla_decode_v3_kernel");
+  if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<false, false, 4, false>, v3::kLdsB, "mla_decode_v3_kernel");
+  return rc;
+}
+
 int launch_decode_v3(const DecodeParams& p, bool sparse, dim3 grid, hipStream_t stream) {
   if (sparse) return launch_rows<true, false>(p, grid, stream);
   if (p.win_skip) return launch_rows<false, true>(p, grid, stream);

@@ -78,7 +78,7 @@ def test_static_scratch_decode_allocates_nothing_and_replays_from_a_graph(dev):
     out = torch.zeros(batch, heads, 512, dtype=torch.bfloat16, device=dev)
     lse = torch.zeros(batch, heads, dtype=torch.float32, device=dev)
 
-    def call():
+    def call(splits=splits):
         stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
         rc = lib.mla_decode_bf16_static(_ptr(qn), qn.stride(0), qn.stride(1), _ptr(qr), qr.stride(0), qr.stride(1),
                                         _ptr(nope), nope.stride(0), nope.stride(1), _ptr(rope), rope.stride(0), rope.stride(1),
@@ -114,3 +114,18 @@ def test_static_scratch_decode_allocates_nothing_and_replays_from_a_graph(dev):
         torch.cuda.synchronize()
         assert torch.equal(out.view(torch.int16), eager[0].view(torch.int16)), f"replay {rep}: output differs from eager"
         assert torch.equal(lse, eager[1]), f"replay {rep}: log-sum-exp differs from eager"
+
+    # A launch with many more chunks takes another form of the split kernel (groups of 128 rows instead of 32), one that
+    # this process may never have launched: the first static call has prepared every form, so this one is captured cold.
+    many = 24
+    assert lib.mla_decode_workspace_bytes(batch, 1, heads, many) <= (48 << 20)
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2):
+        call(many)
+    out.zero_()
+    lse.zero_()
+    graph2.replay()
+    torch.cuda.synchronize()
+    assert (out.float().cpu() - ref).abs().max().item() <= 2e-2
+    assert torch.allclose(lse, eager[1], atol=1e-4, rtol=0)
+
