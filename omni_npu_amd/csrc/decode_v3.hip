@@ -1038,6 +1038,14 @@ template <bool kSparse, bool kWindow, bool kWrite = false>
 static int launch_rows(const DecodeParams& p, dim3 grid, hipStream_t stream) {
   // requests with at most 32 / 64 query rows (tokens x heads) take the forms that leave the missing rows out
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
+  // (the form depends on the shape; all three get their LDS limit with the family's first launch, so that a later launch
+  // under stream capture, where the limit cannot be raised, finds every form ready)
+  {
+    int rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<kSparse, kWindow, 1, kWrite>, v3::kLdsB, "mla_decode_v3_kernel");
+    if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<kSparse, kWindow, 2, kWrite>, v3::kLdsB, "mla_decode_v3_kernel");
+    if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)v3::mla_decode_v3_kernel<kSparse, kWindow, 4, kWrite>, v3::kLdsB, "mla_decode_v3_kernel");
+    if (rc != MLA_OK) return rc;
+  }
   if (r_max <= 32) return launch_form<kSparse, kWindow, 1, kWrite>(p, grid, stream);
   if (r_max <= 64) return launch_form<kSparse, kWindow, 2, kWrite>(p, grid, stream);
   // With few requests and short contexts (and with row lists, which are short by nature) the caller's chunks do not fill

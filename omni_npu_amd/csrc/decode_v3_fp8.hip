@@ -806,6 +806,13 @@ template <bool kWindow>
 static int launch_rows_fp8(const DecodeParams& p, dim3 grid, hipStream_t stream) {
   // requests with at most 32 / 64 query rows (tokens x heads) take the forms that leave the missing rows out
   const int64_t r_max = (int64_t)p.max_q_len * p.num_heads;
+  // (all three forms get their LDS limit with the family's first launch: a later launch under stream capture finds them ready)
+  {
+    int rc = ensure_dynamic_lds((const void*)f8v3::mla_decode_v3_fp8_kernel<kWindow, 1>, f8v3::kLdsB, "mla_decode_v3_fp8_kernel");
+    if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)f8v3::mla_decode_v3_fp8_kernel<kWindow, 2>, f8v3::kLdsB, "mla_decode_v3_fp8_kernel");
+    if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)f8v3::mla_decode_v3_fp8_kernel<kWindow, 4>, f8v3::kLdsB, "mla_decode_v3_fp8_kernel");
+    if (rc != MLA_OK) return rc;
+  }
   if (r_max <= 32) return launch_form_fp8<kWindow, 1>(p, grid, stream);
   if (r_max <= 64) return launch_form_fp8<kWindow, 2>(p, grid, stream);
   // (few chunks: the rows are cut into groups of 32 or 64 with a workgroup each, as in the kernel over the bf16 cache)
