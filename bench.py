@@ -58,6 +58,26 @@ def parity_fields(err: torch.Tensor, ref: torch.Tensor, kind: str, **extra) -> d
             "parity_ok": bool(max_abs <= bar[0] and mean_rel <= bar[1]), **extra}
 
 
+def gemm_probe(dev) -> dict:
+    """torch.matmul of square bf16 matrices, 50 queued calls between one pair of events, after a ramp of the clock."""
+    out = {}
+    for n in (4096, 8192):
+        for name, make in (("normal", lambda: torch.randn(n, n, device=dev).bfloat16()), ("zeros", lambda: torch.zeros(n, n, device=dev, dtype=torch.bfloat16))):
+            a, b_ = make(), make()
+            f = lambda: torch.matmul(a, b_)
+            clock_ramp(f, 0.2, 5)
+            s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            s_.record()
+            for _ in range(50):
+                f()
+            e_.record()
+            torch.cuda.synchronize()
+            out[f"{n}^3 {name}"] = round(2 * n ** 3 * 50 / (s_.elapsed_time(e_) * 1e-3) / 1e12, 1)
+            del a, b_
+    return out
+
+
 def median3(fn):
     ts, res = [], None
     for _ in range(3):
@@ -1059,6 +1079,12 @@ def main():
                          "WRITE_SIZE counters of a rocprofv3 --pmc run of this script")
     ap.add_argument("--workload", default="decode", choices=["decode", "dsa", "prefill", "fp8", "prologue", "epilogue", "window", "layer", "dsa-layer"],
                     help="decode = configs[1] (the headline metric); dsa = configs[3], per-stage times of the sparse path; prefill = configs[2], the chunked-prefill attention kernels; fp8 = configs[4], the quantised-cache decode; prologue = the fused norm + rotary + cache write in front of the path; epilogue = merge of the partials + value up-projection behind the split kernel; layer = the attention part of a decode layer through the backend classes (NPUMLAMetadataBuilder + NPUMLAImpl.forward with the fused steps around it); dsa-layer = the same for configs[3] (LightningIndexer + NPUDSAImpl.forward)")
+    ap.add_argument("--l2-resident", action="store_true",
+                    help="decode workload, a probe and not the workload: every block-table entry folded onto 8 pages, so the "
+                         "cache rows come from L2 instead of HBM (same kernel, same instructions, same result check)")
+    ap.add_argument("--gemm-probe", action="store_true",
+                    help="decode workload: also time the vendor library's bf16 GEMM (torch.matmul, 4096^3 and 8192^3, N(0,1) and "
+                         "all-zero operands) on this part: what its matrix pipes sustain under the same power cap")
     ap.add_argument("--cpu-seqs", type=int, default=64, help="sequences in the CPU-baseline sample")
     ap.add_argument("--no-secondary", action="store_true",
                     help="decode workload: leave out the short runs of configs[2], [3] and [4] that the default line carries "
@@ -1086,6 +1112,8 @@ def main():
         finish(others[args.workload](K, dev, args))
         return
     case = build_workload(args.seed, args.batch, args.heads, args.len_lo, args.len_hi, args.q_len)
+    if args.l2_resident:
+        case["block_table"] = case["block_table"] % 8        # (the oracle reads through the same table)
     heads, b, q_len = args.heads, args.batch, args.q_len
     t = b * q_len
     g = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in case.items()}
@@ -1191,7 +1219,7 @@ def main():
     achieved = kern_bytes / (k_avg * 1e-6) / 1e9
     # HBM bytes per launch of the split kernel from the FETCH_SIZE / WRITE_SIZE counter runs (scaled on a plain copy) of
     # exactly this workload; a counter run cannot be made from inside this script, so other shapes report null
-    default_shape = (args.seed, b, args.len_lo, args.len_hi, q_len, splits) == (0, 64, 4096, 8192, 1, 4)
+    default_shape = (args.seed, b, args.len_lo, args.len_hi, q_len, splits) == (0, 64, 4096, 8192, 1, 4) and not args.l2_resident
     profile_of = {128: "mla_decode_v3_b64_ctx8k.md", 16: "mla_decode_v3_b64_ctx8k_16heads.md"}
     traffic, traffic_src = profile_traffic(profile_of.get(heads, ""), default_shape and heads in profile_of)
     row_groups = 1 if heads * q_len <= 32 else (2 if heads * q_len <= 64 else 4)   # the kernel form the library picks
@@ -1252,7 +1280,11 @@ def main():
                                "sample_seconds": round(sorted(ts)[1], 3), "gpu_vs_oracle_max_abs": round(err.max().item(), 5)}
         res["gpu_vs_oracle"] = parity_fields(err, ref, "bf16", sequences=ns)
         res["parity_ok"] = res["gpu_vs_oracle"]["parity_ok"]
-    default_run = (args.seed, b, heads, args.len_lo, args.len_hi, q_len) == (0, 64, 128, 4096, 8192, 1)
+    if args.l2_resident:
+        res["config"]["probe"] = "block table folded onto 8 pages: cache rows from L2, not the workload's HBM traffic"
+    if args.gemm_probe:
+        res["gemm_probe_tflops"] = gemm_probe(dev)
+    default_run = (args.seed, b, heads, args.len_lo, args.len_hi, q_len) == (0, 64, 128, 4096, 8192, 1) and not args.l2_resident
     if default_run and not args.no_secondary:
         # the other single-GPU configurations, short: after the headline measurement and outside its timed region
         del g, out, out_v, ws
