@@ -426,8 +426,15 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     return (uint32_t)(((ln & 7) ^ swz_rw ^ ((t & 1) << 2) ^ (t & 2) ^ (t >> 2)) << 4);      // swz_rope(t) = (t0 << 2) | (t1 << 1) | t2
   };
   // kFull: every row of the block exists and the source is the paged cache
-  auto issue_piece = [&](IssueCtx& c, int k, auto full) {
+  // When a chunk's cache rows are read by this workgroup alone (one group of query rows per chunk) they are read once in
+  // the whole launch, and the copies are marked non-temporal: 1-2 us of 120 on the headline shape.  With several row
+  // groups per chunk the groups find each other's rows in the XCD's L2, and the mark costs that (16 short sequences in
+  // groups of 32 rows: 30.1 -> 33.7 us), so it is left off there.
+  const bool stream_once = !kSparse && gridDim.z == 1;
+  // kNt: the copy is marked non-temporal
+  auto issue_piece = [&](IssueCtx& c, int k, auto full, auto nt) {
     constexpr bool kFull = decltype(full)::value && !kSparse;
+    constexpr bool kNt = decltype(nt)::value && !kSparse;
     auto clampi = [&](int64_t s_) -> int64_t { return s_ < 0 ? 0 : (s_ > max_row ? max_row : s_); };
 
     if (k < 8) {
@@ -435,11 +442,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       if constexpr (kFull) {
         uint32_t d = dma_off;
         asm volatile("" : "+v"(d));                           // (opaque: the eight offsets are not precomputed and spilled)
-        dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + cw * 8192, k * 1024);
+        if constexpr (kNt) dma16_sv_m0add_nt(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + cw * 8192, k * 1024);
+        else dma16_sv_m0add(c.np, (d ^ (uint32_t)(swz_nope(k) << 4)) + s_rowoff[k], c.nbuf + cw * 8192, k * 1024);
       } else {
         const uint32_t off = (uint32_t)((lane_now() ^ swz_nw ^ swz_nope(k)) << 4);
         const int re = r < c.last ? r : c.last;
         if constexpr (kSparse) dma16_sv(c.np + clampi(ids_row[k]) * n_sr2, off, c.nbuf + r * 1024);
+        else if constexpr (kNt) dma16_sv_nt(c.np + (uint64_t)re * n_sr2, off, c.nbuf + r * 1024);
         else dma16_sv(c.np + (uint64_t)re * n_sr2, off, c.nbuf + r * 1024);
       }
     } else {
@@ -447,11 +456,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
       if constexpr (kSparse) {
         dma16_v(c.rp + clampi(ids_rope) * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
       } else if constexpr (kFull) {
-        dma16_sv(c.rp, (uint32_t)(cw * 8 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
+        if constexpr (kNt) dma16_sv_nt(c.rp, (uint32_t)(cw * 8 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
+        else dma16_sv(c.rp, (uint32_t)(cw * 8 + rope_lane_row()) * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
       } else {
         const int r = cw * 8 + rope_lane_row();
         const int re = r < c.last ? r : c.last;
-        dma16_sv(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
+        if constexpr (kNt) dma16_sv_nt(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
+        else dma16_sv(c.rp, (uint32_t)re * r_sr2 + rope_lane_off(), c.rbuf + cw * 1024);
       }
     }
   };
@@ -459,7 +470,7 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     IssueCtx c = issue_begin(blk);
     if (copier) {
 #pragma unroll
-      for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{});
+      for (int k = 0; k < kCopies; k++) issue_piece(c, k, std::false_type{}, std::false_type{});
     }
   };
   // Row list: the rows of the first kLead blocks are fetched together (one round trip) before any copy goes out
@@ -605,8 +616,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
     // clocks behind the other wave of its SIMD (which copies nothing), and the two want the LDS and the matrix pipe at
     // different moments (measured against the copies spread between the MFMAs: 121.8 / 123.4 -> 119.5 / 121.5 us).
     if constexpr (kIssue) {
+      if (stream_once) {
 #pragma unroll
-      for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::integral_constant<bool, kIssueMode == 2>{});
+        for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::integral_constant<bool, kIssueMode == 2>{}, std::true_type{});
+      } else {
+#pragma unroll
+        for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::integral_constant<bool, kIssueMode == 2>{}, std::false_type{});
+      }
     }
     bf16x8 ka[kAhead];
     // fragment j: contraction step kk = j >> 1, key group kg = j & 1; each statement is wait + MFMA + the read that
@@ -904,10 +920,13 @@ __global__ __launch_bounds__(512) void mla_decode_v3_kernel(const DecodeParams p
             IssueCtx ic = issue_begin(blk + kLead);
             if (kSparse || !full_ok || L - 1 - (blk + kLead) * kBlk < kBlk - 1) {
 #pragma unroll
-              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::false_type{});
+              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::false_type{}, std::false_type{});
+            } else if (stream_once) {
+#pragma unroll
+              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::true_type{}, std::true_type{});
             } else {
 #pragma unroll
-              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::true_type{});
+              for (int k = 0; k < kCopies; k++) issue_piece(ic, k, std::true_type{}, std::false_type{});
             }
           }
         } else if (has_rows) {

@@ -77,6 +77,21 @@ __device__ __forceinline__ void dma16_sv_m0add(const void* gbase_uniform, uint32
                : "s"(lds_base_uniform), "v"(voff), "s"(gbase_uniform), "n"(lds_imm)
                : "memory", "m0", "scc");
 }
+// The same two copies marked non-temporal, for bytes that are read once (the cache rows a decode launch streams): measured on
+// the headline decode shape 1-2 us of 120 against the default policy; system scope (sc1, sc0 sc1) measured no different from
+// the default.  Not for data that other workgroups on the XCD read at about the same time (queries, prefill tiles).
+__device__ __forceinline__ void dma16_sv_nt(const void* gbase_uniform, uint32_t voff, uint32_t lds_addr_uniform) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+               :
+               : "s"(lds_addr_uniform), "v"(voff), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void dma16_sv_m0add_nt(const void* gbase_uniform, uint32_t voff, uint32_t lds_base_uniform, int lds_imm) {
+  asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+               :
+               : "s"(lds_base_uniform), "v"(voff), "s"(gbase_uniform), "n"(lds_imm)
+               : "memory", "m0", "scc");
+}
 // source = per-lane 64-bit address
 __device__ __forceinline__ void dma16_v(const void* gaddr, uint32_t lds_addr_uniform) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
