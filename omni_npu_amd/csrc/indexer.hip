@@ -163,7 +163,7 @@ __global__ __launch_bounds__(256, 2) void dsa_indexer_fp8_kernel(const IndexerPa
     const float* sc = p.k_scale + blk * p.ks_sp + nxt_off;
     const uint32_t dst = ring + (uint32_t)slot * kIdxSlotB;
 #pragma unroll
-    for (int i = 0; i < 4; i++) dma16_sv(rows, src_off[i], dst + i * 1024);
+    for (int i = 0; i < 4; i++) dma16_sv_nt(rows, src_off[i], dst + i * 1024);
     dma4_sv_lo32(sc, (uint32_t)lane * 4, dst + 32 * kIdxDim);
     nxt_off += 32;
     if (nxt_off >= p.page_size) { nxt_off = 0; nxt_pg++; }
