@@ -29,7 +29,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 
 
 def test_parity_fields_and_the_exit_status_they_drive(capsys):
-    """Every workload's comparison with the oracle carries the bar of its cache type and a verdict; a missed bar, also in a
+    """Every workload's comparison with the oracle carries the bar of its cache type and whether it was met; a missed bar, also in a
     secondary workload, turns into exit status 1 after the JSON line is out."""
     import json
 
