@@ -60,7 +60,13 @@ __global__ __launch_bounds__(kWide ? 64 * kWideWaves : 256) void mla_chunk_reduc
   const int groups = (r_max + kRedRows - 1) / kRedRows;     // row groups per sequence
   // (the wave number is made a scalar: everything derived from it, the addresses of the per-row records included, then
   // lives in scalar registers and is fetched with scalar loads)
-  const int64_t gw_first = kWide ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + wave;
+  // Workgroups go to the eight XCDs round-robin in launch order; every XCD takes a contiguous eighth of the rows, as the split
+  // kernels give every XCD a contiguous eighth of the chunks: a row's partials were written, and its neighbours' partials
+  // are being read, through the same part of the memory system (headline merge 17.1 -> 16.0 us, row lists 53.8 -> 52.3 us
+  // for split + merge).
+  int64_t wg_id = blockIdx.x;
+  if (!kWide && (gridDim.x & 7) == 0) wg_id = (int64_t)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const int64_t gw_first = kWide ? (int64_t)blockIdx.x : wg_id * 4 + wave;
   const int64_t gw_step = kWide ? (int64_t)gridDim.x : (int64_t)gridDim.x * 4;
   for (int64_t gw = gw_first; gw < (int64_t)p.batch * groups; gw += gw_step) {
   const int b = (int)(gw / groups);
