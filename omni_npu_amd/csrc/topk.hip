@@ -425,6 +425,23 @@ __device__ __forceinline__ TopkRow topk_row(const TopkParams& p, int slot) {
   return r;
 }
 
+// (slice, token slot) of a workgroup of the multi-workgroup kernels.  Workgroups go to the eight XCDs round-robin in launch
+// order (x fastest); renumbered, every XCD takes a contiguous eighth of the tokens with all their slices, so what one kernel
+// of the chain leaves for the next (slice histograms, candidates, counts, the logits themselves) is read through the XCD
+// that wrote it.
+struct SliceOf { int s, slot; };
+__device__ __forceinline__ SliceOf slice_of_workgroup() {
+  SliceOf r{(int)blockIdx.x, (int)blockIdx.y};
+  const uint32_t total = gridDim.x * gridDim.y;
+  if ((total & 7) == 0 && ((total >> 3) % gridDim.x) == 0) {
+    const uint32_t lin = blockIdx.x + gridDim.x * blockIdx.y;
+    const uint32_t nl = (lin & 7) * (total >> 3) + (lin >> 3);
+    r.s = (int)(nl % gridDim.x);
+    r.slot = (int)(nl / gridDim.x);
+  }
+  return r;
+}
+
 // This thread's eight keys of slice s: positions pos(j, e) = s*kSliceKeys + w*512 + j*256 + lane*4 + e (j < 2, e < 4), so
 // that a wavefront holds 512 consecutive keys in (j, lane, e) order.  Keys at or past n read as 0 and are never used.
 struct SliceKeys { float v[2][4]; int base; };
@@ -451,8 +468,9 @@ __global__ __launch_bounds__(kTopkThreads) void dsa_topk_hist_kernel(const TopkM
   __shared__ int hist[kBins];
   __shared__ float fscratch[2 * kMwWaves];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int s = blockIdx.x;
-  const TopkRow r = topk_row(p.t, blockIdx.y);
+  const SliceOf so = slice_of_workgroup();
+  const int s = so.s;
+  const TopkRow r = topk_row(p.t, so.slot);
   if (!r.live || r.n <= p.t.k || s * kSliceKeys >= r.n) return;
   const int n = r.n;
   // all loads first: four runs of 1024 consecutive keys spread over the whole row (the sample that fixes the bins, the
@@ -495,8 +513,9 @@ __global__ __launch_bounds__(kTopkThreads) void dsa_topk_gather_kernel(const Top
   __shared__ int hist[kBins];
   __shared__ int scratch[64];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int s = blockIdx.x;
-  const TopkRow r = topk_row(p.t, blockIdx.y);
+  const SliceOf so = slice_of_workgroup();
+  const int s = so.s;
+  const TopkRow r = topk_row(p.t, so.slot);
   if (!r.live || r.n <= p.t.k || s * kSliceKeys >= r.n) return;
   const int n = r.n;
   const int live_slices = (n + kSliceKeys - 1) / kSliceKeys;
@@ -541,8 +560,9 @@ __global__ __launch_bounds__(kTopkThreads) void dsa_topk_write_kernel(const Topk
   __shared__ uint32_t cand_u[kMwCandLds];
   __shared__ uint32_t cand_i[kMwCandLds];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int s = blockIdx.x;
-  const TopkRow r = topk_row(p.t, blockIdx.y);
+  const SliceOf so = slice_of_workgroup();
+  const int s = so.s;
+  const TopkRow r = topk_row(p.t, so.slot);
   if (!r.live) return;
   const int n = r.n, k = p.t.k;
   const TopkSink out = topk_sink(p.t, r.b, r.t);
