@@ -263,7 +263,11 @@ int mla_merge_n_states(const void* outs, int64_t outs_stride_n, int64_t outs_str
  * cu_q / cu_k int32 [B+1] on the device; out [T,N,128] bf16 (0) or fp32 (1); lse_out fp32 [T,N] or NULL.
  * window = w > 0 keeps only the newest w visible keys of each row: the band of mla.py:525-541 (sparse_mode 4,
  * pre_tokens = sliding_window - 1, next_tokens 0); 0 = no window.
- * Rows with no visible key give zeros and lse = -inf. */
+ * Rows with no visible key give zeros and lse = -inf.
+ * out_dtype + MLA_PREFILL_KV_F16: k_nope, k_pe and v hold fp16 instead of bf16 (a caller that makes them with an fp16
+ * GEMM; the queries stay bf16).  Both products then run on fp16 and the kernel skips the bf16 -> fp16 conversion of the value
+ * tiles that it otherwise does for the P.V product. */
+#define MLA_PREFILL_KV_F16 16
 int mla_prefill_varlen(const void* q_nope, int64_t qn_stride_t, int64_t qn_stride_h, const void* q_pe,
                        int64_t qp_stride_t, int64_t qp_stride_h, const void* k_nope, int64_t kn_stride_t,
                        int64_t kn_stride_h, const void* k_pe, int64_t kp_stride_t, const void* v, int64_t v_stride_t,

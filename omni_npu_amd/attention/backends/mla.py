@@ -236,10 +236,26 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         out2 = torch.bmm(x, self.W_UV)
         return out2.transpose(0, 1).contiguous().view(-1, self.num_heads * self.v_head_dim)
 
-    def _kv_up(self, kv_c: torch.Tensor):
-        kv = self.kv_b_proj(kv_c)
-        kv = kv[0] if isinstance(kv, tuple) else kv
-        kv = kv.view(-1, self.num_heads, self.qk_nope_head_dim + self.v_head_dim)
+    # The prefill kernel multiplies the probabilities with fp16 values (the bf16 bar of the output leaves no room for bf16
+    # probabilities), so it converts every value tile it is given in bf16.  Where the up-projection is a plain weight the
+    # keys and values are made in fp16 in the first place - the same GEMM on fp16 copies of its operands, no extra pass -
+    # and the kernel converts nothing (configs of 4 x 2048 over 16k: 13.2 -> 12.2 ms).  fp16 holds every bf16 number of
+    # magnitude 2^-14 .. 65504 exactly; set prefill_kv_fp16 = False for a model whose keys or values can exceed that range.
+    prefill_kv_fp16 = True
+
+    def _kv_up(self, kv_c: torch.Tensor, allow_fp16: bool = False):
+        """(k_nope [T,N,128], v [T,N,128]) of latent rows kv_c [T,512] (reference: ``self.kv_b_proj(kv_c_normed)[0]``,
+        mla.py:405-413, 566-571).  With ``allow_fp16`` both may come back as fp16."""
+        n, d = self.num_heads, self.qk_nope_head_dim + self.v_head_dim
+        w = getattr(self.kv_b_proj, "weight", None)
+        if (allow_fp16 and self.prefill_kv_fp16 and isinstance(w, torch.Tensor) and w.dtype in (torch.bfloat16, torch.float16)
+                and tuple(w.shape) == (n * d, kv_c.shape[-1]) and getattr(self.kv_b_proj, "bias", None) is None
+                and kv_c.dtype in (torch.bfloat16, torch.float16)):
+            kv = torch.matmul(kv_c.to(torch.float16), w.to(torch.float16).t())
+        else:
+            kv = self.kv_b_proj(kv_c)
+            kv = kv[0] if isinstance(kv, tuple) else kv
+        kv = kv.view(-1, n, d)
         return kv[..., :self.qk_nope_head_dim], kv[..., self.qk_nope_head_dim:]
 
     # ---- prefill ----
@@ -264,7 +280,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
                                                scale=k_scale, seq_starts=cc.starts[i], total_rows=toks)
             kv_c_normed = cc.workspace[:toks][..., :self.kv_lora_rank]
             k_pe = cc.workspace[:toks][..., self.kv_lora_rank:]
-            k_nope, v = self._kv_up(kv_c_normed)
+            k_nope, v = self._kv_up(kv_c_normed, allow_fp16=True)
+            k_pe = k_pe.to(k_nope.dtype)
             # running results stay fp32: each bf16 rounding in between would add 2^-10 of mean relative error to the
             # layer's output
             first = output is None
@@ -287,7 +304,7 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
         t, n = q.shape[0], self.num_heads
         has_context = prefill.chunked_context is not None
         q_nope, q_pe = q[..., :self.qk_nope_head_dim], q[..., self.qk_nope_head_dim:]
-        k_nope, v = self._kv_up(kv_c_normed)
+        k_nope, v = self._kv_up(kv_c_normed, allow_fp16=True)
         cu_q = prefill.query_start_loc.to(torch.int32).contiguous()
         ctx_out = ctx_lse = None
         if has_context:
@@ -295,8 +312,8 @@ class NPUMLAImpl(MLACommonBaseImpl[NPUMLAMetadata]):
             ctx_out, ctx_lse = self._compute_prefill_context(q_nope, q_pe, kv_cache[0],
                                                              None if self.fp8_cache else kv_cache[1], attn_metadata, k_scale)
         output = torch.empty(t, n, self.v_head_dim, dtype=torch.bfloat16, device=q.device)
-        K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1), v, cu_q, cu_q, prefill.max_query_len, self.scale, True,
-                         output, prev_out=ctx_out, prev_lse=ctx_lse)
+        K.prefill_varlen(q_nope, q_pe, k_nope, k_pe.reshape(t, -1).to(k_nope.dtype), v, cu_q, cu_q, prefill.max_query_len,
+                         self.scale, True, output, prev_out=ctx_out, prev_lse=ctx_lse)
         return output.flatten(start_dim=-2)
 
     def _forward_prefill_sink(self, q, kv_c_normed, k_pe, prefill) -> torch.Tensor:

@@ -115,6 +115,9 @@ __device__ __forceinline__ void pf_issue_full_tile(const PrefillParams& p, const
   for (int i = 0; i < 2; i++) dma16_sv(kp, o.kp[i], buf + kPfKnB + (wave * 2 + i) * 1024);
 }
 
+// kHalf: k_nope, k_pe and v hold fp16 instead of bf16 (a caller that makes them with an fp16 GEMM): both products run on
+// fp16 (the query is converted once, in registers) and no tile is converted.
+template <bool kHalf>
 __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const PrefillParams p) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
@@ -224,6 +227,15 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
       for (int kk = 0; kk < 8; kk++) { bf16x8 v = *(const bf16x8*)(qn + kk * 16); qf[kk] = row_ok ? v : zero; }
 #pragma unroll
       for (int kk = 0; kk < 4; kk++) { bf16x8 v = *(const bf16x8*)(qp + kk * 16); qf[8 + kk] = row_ok ? v : zero; }
+      if constexpr (kHalf) {
+#pragma unroll
+        for (int kk = 0; kk < 12; kk++) {
+          f16x8 h;
+#pragma unroll
+          for (int e = 0; e < 8; e++) h[e] = (_Float16)(float)qf[kk][e];
+          qf[kk] = __builtin_bit_cast(bf16x8, h);
+        }
+      }
     }
     // per-lane LDS offsets
     const int fk = pf_swz16(h32 & 15), fr = pf_swz8(h32 & 15);
@@ -256,7 +268,7 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
       // barrier: the four wavefronts read each other's pieces.  (Tried: the conversion's arithmetic and writes behind the
       // first block's score MFMAs, and the next tile converted between the two blocks of this one - both slower.)
       char* vt = buf + kPfKnB + kPfKrB + (int)threadIdx.x * 16;
-      {
+      if constexpr (!kHalf) {
         u32x4 w[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) w[i] = *(const u32x4*)(vt + i * 4096);
@@ -270,8 +282,8 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
           }
 #pragma unroll
         for (int i = 0; i < 4; i++) *(u32x4*)(vt + i * 4096) = w[i];
+        lds_barrier();
       }
-      lds_barrier();
 #pragma unroll 1
       for (int tb = 0; tb < 2; tb++) {
         const bool active = key_base + tb * 32 < wave_max_limit && key_base + tb * 32 + 32 > wg_lo;
@@ -282,12 +294,14 @@ __global__ __launch_bounds__(256, 2) void mla_prefill_varlen_kernel(const Prefil
 #pragma unroll
         for (int kk = 0; kk < 8; kk++) {
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 256 + koff[kk]);
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
+          if constexpr (kHalf) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, qf[kk]), s, 0, 0, 0);
+          else s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[kk], s, 0, 0, 0);
         }
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
           bf16x8 a = *(const bf16x8*)(buf + tb * 32 * 128 + roff[kk]);
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[8 + kk], s, 0, 0, 0);
+          if constexpr (kHalf) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, qf[8 + kk]), s, 0, 0, 0);
+          else s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[8 + kk], s, 0, 0, 0);
         }
         // Only blocks that some row of this wave cannot see in full pay for the mask (causal diagonal, end of the keys,
         // rows past the end of the sequence); everywhere else the scores go straight to the maximum.  The scale is
@@ -379,6 +393,8 @@ static int prefill_varlen_impl(const char* what, const void* q_nope, int64_t qn_
   MLA_REQUIRE(q_nope && q_pe && k_nope && k_pe && v && cu_q && cu_k && out, MLA_ERR_NULL, "%s: null pointer argument", what);
   MLA_REQUIRE(batch >= 0 && num_heads >= 1 && max_q_len >= 0 && batch <= 65535 && num_heads <= 65535 && window >= 0,
               MLA_ERR_SHAPE, "%s: batch=%d num_heads=%d max_q_len=%d window=%d", what, batch, num_heads, max_q_len, window);
+  const bool kv_half = (out_dtype & 16) != 0;              // k_nope, k_pe and v hold fp16 (MLA_PREFILL_KV_F16)
+  out_dtype &= ~16;
   MLA_REQUIRE(out_dtype == 0 || out_dtype == 1, MLA_ERR_UNSUPPORTED, "%s: out dtype code %d", what, out_dtype);
   MLA_REQUIRE(scale > 0.f, MLA_ERR_UNSUPPORTED, "%s: the softmax scale must be positive (got %g)", what, (double)scale);
   MLA_REQUIRE(qn_stride_t % 8 == 0 && qn_stride_h % 8 == 0 && qp_stride_t % 8 == 0 && qp_stride_h % 8 == 0 &&
@@ -402,10 +418,12 @@ static int prefill_varlen_impl(const char* what, const void* q_nope, int64_t qn_
   p.out = out; p.o_st = out_stride_t; p.o_sh = out_stride_h; p.out_fp32 = out_dtype;
   p.lse = lse_out;
   p.prev_out = prev_out; p.po_st = prev_stride_t; p.po_sh = prev_stride_h; p.prev_lse = prev_lse;
-  const int rc = ensure_dynamic_lds((const void*)mla_prefill_varlen_kernel, kPfLdsB, what);
+  int rc = ensure_dynamic_lds((const void*)mla_prefill_varlen_kernel<false>, kPfLdsB, what);
+  if (rc == MLA_OK) rc = ensure_dynamic_lds((const void*)mla_prefill_varlen_kernel<true>, kPfLdsB, what);
   if (rc != MLA_OK) return rc;
   dim3 grid((max_q_len + kPfRows - 1) / kPfRows, num_heads, batch);
-  hipLaunchKernelGGL(mla_prefill_varlen_kernel, grid, dim3(256), kPfLdsB, stream, p);
+  if (kv_half) hipLaunchKernelGGL(mla_prefill_varlen_kernel<true>, grid, dim3(256), kPfLdsB, stream, p);
+  else hipLaunchKernelGGL(mla_prefill_varlen_kernel<false>, grid, dim3(256), kPfLdsB, stream, p);
   return check_launch("mla_prefill_varlen_kernel");
 }
 

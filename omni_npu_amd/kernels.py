@@ -774,6 +774,9 @@ def sparse_decode(q_nope: torch.Tensor, q_rope: torch.Tensor, nope_cache: torch.
 
 
 # ------------------------------------------------------------------------------------------------
+_PREFILL_KV_F16 = 16                                       # added to the output dtype code: k_nope, k_pe, v hold fp16
+
+
 def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tensor, k_pe: torch.Tensor, v: torch.Tensor,
                    cu_q: torch.Tensor, cu_k: torch.Tensor, max_q_len: int, scale: float, causal: bool,
                    out: torch.Tensor, lse_out: Optional[torch.Tensor] = None, window: Optional[int] = None,
@@ -784,7 +787,9 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
     newest ``window`` visible keys of each row (the sliding-window band of mla.py:525-541).
     ``prev_out`` (fp32 [T,N,128]) / ``prev_lse`` (fp32 [T,N]): the result of an earlier call over OTHER keys of the same
     rows; the call then returns the attention over the union, i.e. what this attention followed by merge_attn_states
-    (src/omni_npu/attention/ops.py:5-42) gives, in one launch.  ``out`` may be ``prev_out``."""
+    (src/omni_npu/attention/ops.py:5-42) gives, in one launch.  ``out`` may be ``prev_out``.
+    k_nope, k_pe and v may all three be fp16 (a caller that makes them with an fp16 GEMM): both products then run on fp16
+    and the kernel skips the conversion of the value tiles it otherwise does (the queries stay bf16)."""
     if window is not None and window < 1:
         raise ValueError(f"prefill_varlen: window must be positive (got {window})")
     _need_cuda(q_nope, q_pe, k_nope, k_pe, v, cu_q, cu_k, out, lse_out)
@@ -794,9 +799,11 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
     if p != 128 or q_pe.shape != (t, n, 64) or k_nope.shape[1:] != (n, 128) or v.shape != k_nope.shape or \
             k_pe.shape != (k_nope.shape[0], 64) or out.shape != (t, n, 128):
         raise ValueError("prefill_varlen: shapes must be q_nope [T,N,128], q_pe [T,N,64], k_nope/v [Tk,N,128], k_pe [Tk,64]")
-    for x in (q_nope, q_pe, k_nope, k_pe, v):
-        if x.dtype != torch.bfloat16 or x.stride(-1) != 1:
-            raise TypeError("prefill_varlen: bf16 inputs with a contiguous last dim")
+    kv_half = k_nope.dtype == torch.float16
+    for x, want in ((q_nope, torch.bfloat16), (q_pe, torch.bfloat16), (k_nope, None), (k_pe, k_nope.dtype), (v, k_nope.dtype)):
+        if x.dtype != (want or x.dtype) or x.dtype not in (torch.bfloat16, torch.float16) or x.stride(-1) != 1:
+            raise TypeError("prefill_varlen: bf16 queries, keys and values all bf16 or all fp16, with a contiguous last dim")
+    kv_code = _PREFILL_KV_F16 if kv_half else 0
     if out.dtype not in _DT or out.stride(-1) != 1:
         raise TypeError("prefill_varlen: out must be bf16 or fp32")
     if cu_q.dtype != torch.int32 or cu_k.dtype != torch.int32 or cu_q.numel() != cu_k.numel() or \
@@ -829,7 +836,7 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
             q_nope.data_ptr(), q_nope.stride(0), q_nope.stride(1), q_pe.data_ptr(), q_pe.stride(0), q_pe.stride(1),
             k_nope.data_ptr(), k_nope.stride(0), k_nope.stride(1), k_pe.data_ptr(), k_pe.stride(0), v.data_ptr(), v.stride(0),
             v.stride(1), cu_q.data_ptr(), cu_k.data_ptr(), cu_q.numel() - 1, n, int(max_q_len), 1 if causal else 0,
-            int(window or 0), float(scale), out.data_ptr(), out.stride(0), out.stride(1), _DT[out.dtype],
+            int(window or 0), float(scale), out.data_ptr(), out.stride(0), out.stride(1), _DT[out.dtype] | kv_code,
             lse_out.data_ptr() if lse_out is not None else None, prev_out.data_ptr(), prev_out.stride(0), prev_out.stride(1),
             prev_lse.data_ptr(), _stream(q_nope))
         _lib.check(rc, "mla_prefill_varlen_continue")
@@ -839,7 +846,7 @@ def prefill_varlen(q_nope: torch.Tensor, q_pe: torch.Tensor, k_nope: torch.Tenso
                                 k_pe.stride(0), v.data_ptr(), v.stride(0), v.stride(1), cu_q.data_ptr(), cu_k.data_ptr(),
                                 cu_q.numel() - 1, n, int(max_q_len), 1 if causal else 0, int(window or 0), float(scale),
                                 out.data_ptr(),
-                                out.stride(0), out.stride(1), _DT[out.dtype],
+                                out.stride(0), out.stride(1), _DT[out.dtype] | kv_code,
                                 lse_out.data_ptr() if lse_out is not None else None, _stream(q_nope))
     _lib.check(rc, "mla_prefill_varlen")
     return out

@@ -101,8 +101,8 @@ class NPUDeepseekMLAAttention(torch.nn.Module):
         q_pe = q[..., self.qk_nope_head_dim:]
         K.kv_rmsnorm_rope_cache(kv, self.kv_a_layernorm.weight, cos, sin, meta.slot_mapping, nope_c, rope_c,
                                 eps=self._eps(), kv_a_out=kv_a, k_pe_out=k_pe, q_rope=q_pe)
-        k_nope, v = impl._kv_up(kv_a)
+        k_nope, v = impl._kv_up(kv_a, allow_fp16=True)
         cu = meta.prefill.query_start_loc.to(torch.int32).contiguous()
-        K.prefill_varlen(q[..., :self.qk_nope_head_dim], q_pe, k_nope, k_pe, v, cu, cu, meta.prefill.max_query_len,
-                         impl.scale, True, attn_output)
+        K.prefill_varlen(q[..., :self.qk_nope_head_dim], q_pe, k_nope, k_pe.to(k_nope.dtype), v, cu, cu,
+                         meta.prefill.max_query_len, impl.scale, True, attn_output)
         return self.o_proj(attn_output.view(t, -1))[0]

@@ -87,6 +87,51 @@ def test_mla_impl_forward_matches_reference_semantics(dev, q_lens, seq_lens, n):
     attn_close(out[:t], ref, 3e-2, 8e-3)                                                # the reference's 3e-2 bar
 
 
+class _PlainLinear:
+    """An up-projection as the model owns it when nothing is quantised: a weight [out, in] and a call that returns a tuple."""
+
+    def __init__(self, w_in_out, dev):
+        self.weight = w_in_out.t().contiguous().to(dev)
+        self.bias = None
+        self.calls = 0
+
+    def __call__(self, x):
+        self.calls += 1
+        return (x @ self.weight.t(),)
+
+
+@pytest.mark.parametrize("fp16_path", [True, False])
+def test_mla_prefill_with_a_plain_up_projection_makes_keys_and_values_in_fp16(dev, fp16_path):
+    """Where kv_b_proj is a plain weight the prefill makes k_nope and v with an fp16 GEMM (the kernel then converts no value
+    tile) instead of calling the module; prefill_kv_fp16 = False keeps the module's bf16 call.  Both against the oracle,
+    mixed batch with a chunked context, and against each other."""
+    q_lens, seq_lens, n = [1, 1, 16, 16], [300, 77, 64, 64], 4
+    g = torch.Generator().manual_seed(11)
+    common = _common(q_lens, seq_lens)
+    t = common.num_actual_tokens
+    nblk = int(common.block_table_tensor.max()) + 1
+    nope = torch.randn(nblk, 128, 512, generator=g).bfloat16()
+    rope = torch.randn(nblk, 128, 64, generator=g).bfloat16()
+    q = torch.randn(t, n, 192, generator=g).bfloat16()
+    kvc, kpe = torch.randn(t, 512, generator=g).bfloat16(), torch.randn(t, 1, 64, generator=g).bfloat16()
+    common.slot_mapping = torch.cat([O.slots_for(common.block_table_tensor, b, s - ql, s)
+                                     for b, (ql, s) in enumerate(zip(q_lens, seq_lens))])
+    impl, w = _mk_impl(mla.NPUMLAImpl, n, dev)
+    impl.kv_b_proj = _PlainLinear(w, dev)
+    impl.prefill_kv_fp16 = fp16_path
+    builder = mla.NPUMLAMetadataBuilder(V.AttentionSpec(128, 1, 576, torch.bfloat16), ["l"], _cfg(cap=2), dev)
+    builder.chunked_prefill_workspace_size = 64
+    ref = _oracle_mla(q.float(), kvc, kpe, w, nope.clone(), rope.clone(), common, n, impl.scale)
+    meta = builder.build(0, _to(common, dev))
+    raw = torch.cat([nope.reshape(-1), rope.reshape(-1)]).to(dev).view(torch.uint8)
+    kv_cache = mla.NPUMLABackend.reshape_kv_cache(raw, nblk, 128, 1, 576, dtype=torch.bfloat16)
+    out = torch.zeros(t, n * 128, dtype=torch.bfloat16, device=dev)
+    impl.forward(SimpleNamespace(_k_scale=None), q.to(dev), kvc.to(dev), kpe.to(dev), kv_cache, meta, output=out)
+    attn_close(out, ref, 3e-2, 8e-3)
+    # the module is called only where the fp16 path is off (prefill: the suffix and one context chunk)
+    assert (impl.kv_b_proj.calls == 0) == fp16_path
+
+
 def test_mla_impl_forward_fp8_cache_with_chunked_context(dev):
     """NPUMLAImpl.forward over the fp8 block-scaled cache, mixed batch: decodes read the quantised cache (the new token
     included), prefills attend over their own un-quantised suffix plus a chunked context gathered and dequantised from

@@ -57,6 +57,20 @@ def test_prefill_varlen_matches_oracle(dev, causal, q_lens, k_lens, n):
     # bf16 output: its rounding alone is 1.4e-3 of mean relative error; the probabilities go through P.V as fp16 (11
     # significant bits), which leaves the rest of the 2e-3 bar unused whatever the number of keys
     attn_close(out_bf, ref, 2e-2, 2e-3)
+    # keys and values handed over as fp16 (what a caller with an fp16 up-projection GEMM has): both products on fp16, no
+    # tile converted; the same numbers, so the same oracle, at the same bars
+    out_h = torch.full((q.shape[0], n, 128), float("nan"), dtype=torch.float32, device=dev)
+    lse_h = torch.full((q.shape[0], n), float("nan"), dtype=torch.float32, device=dev)
+    hkv, hpe = dkv.to(torch.float16), dpe.to(torch.float16)
+    K.prefill_varlen(dq[..., :128], dq[..., 128:], hkv[..., :128], hpe, hkv[..., 128:],
+                     torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
+                     max(q_lens), scale, causal, out_h, lse_h)
+    attn_close(out_h, ref, 2e-2, 4e-4)
+    assert torch.equal(torch.isfinite(lse_h.cpu()), fin) and torch.allclose(lse_h.cpu()[fin], ref_lse[fin], atol=2e-2)
+    with pytest.raises(TypeError):                            # all three, or none
+        K.prefill_varlen(dq[..., :128], dq[..., 128:], hkv[..., :128], dpe, dkv[..., 128:],
+                         torch.tensor(cu_q, dtype=torch.int32, device=dev), torch.tensor(cu_k, dtype=torch.int32, device=dev),
+                         max(q_lens), scale, causal, out_h)
 
 
 def test_chunked_context_flow_gather_attend_merge(dev):
