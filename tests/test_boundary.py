@@ -270,6 +270,31 @@ def test_process_weights_after_loading_layout():
     assert torch.equal(impl.W_UK_T, w[..., :128].permute(1, 2, 0)) and torch.equal(impl.W_UV, w[..., 128:].transpose(0, 1))
 
 
+def test_kv_up_projection_goes_fp16_only_for_a_plain_weight():
+    """_kv_up (reference: ``self.kv_b_proj(kv_c_normed)[0]``, mla.py:405-413) hands the prefill kernel fp16 keys and values
+    when it is allowed to, the projection is a plain bf16 weight without bias and the switch is on; otherwise it calls the
+    module.  Either way the numbers are the module's, up to the rounding of the result."""
+    n = 2
+    lin = torch.nn.Linear(512, n * 256, bias=False).to(torch.bfloat16)
+    impl = _impl(mla.NPUMLAImpl, num_heads=n, kv_b_proj=lin)
+    x = torch.randn(5, 512, generator=torch.Generator().manual_seed(1)).bfloat16()
+    k16, v16 = impl._kv_up(x, allow_fp16=True)
+    k, v = impl._kv_up(x)
+    assert k16.dtype == v16.dtype == torch.float16 and k.dtype == v.dtype == torch.bfloat16
+    assert k16.shape == k.shape == (5, n, 128) and v16.shape == v.shape == (5, n, 128)
+    ref = (x.float() @ lin.weight.float().t()).view(5, n, 256)
+    assert torch.allclose(k16.float(), ref[..., :128], atol=2e-3, rtol=2e-3) and torch.allclose(v16.float(), ref[..., 128:], atol=2e-3, rtol=2e-3)
+    assert torch.allclose(k.float(), ref[..., :128], atol=2e-2, rtol=2e-2)
+    impl.prefill_kv_fp16 = False
+    assert impl._kv_up(x, allow_fp16=True)[0].dtype == torch.bfloat16
+    impl.prefill_kv_fp16 = True
+    impl.kv_b_proj = lambda t: (lin(t),)                       # no weight to be seen: the module is called
+    assert impl._kv_up(x, allow_fp16=True)[0].dtype == torch.bfloat16
+    biased = torch.nn.Linear(512, n * 256, bias=True).to(torch.bfloat16)
+    impl.kv_b_proj = biased
+    assert impl._kv_up(x, allow_fp16=True)[0].dtype == torch.bfloat16
+
+
 # ---- graph wrapper (no GPU: pass-through paths only) ---------------------------------------------------------------
 def test_graph_wrapper_pass_through_and_pad_list():
     calls = []
