@@ -106,3 +106,24 @@ def test_few_query_rows_keep_a_tenth_of_the_bar_in_hand(dev, batch, heads, q_len
         assert mr <= 1.6e-3, f"mean_rel={mr:.4g}: the headroom of the two-term probabilities is gone"
     else:
         assert mr <= 1.8e-3, f"mean_rel={mr:.4g}"
+
+
+# Launches whose chunks fill the compute units keep whole groups of 128 rows and single-term bf16 probabilities with the
+# dominant key's rounding repaired afterwards.  Many short sequences are where that repair helps least (a few hundred
+# keys of similar weight): 1.74e-3 to 1.85e-3 of mean relative error, against 1.66e-3 to 1.68e-3 on long contexts.
+@pytest.mark.parametrize("batch,q_len,lo,hi,splits,seed", [
+    (200, 1, 64, 512, 1, 1), (140, 1, 16, 200, 1, 2), (160, 1, 300, 1500, 2, 3), (70, 2, 100, 900, 1, 4),
+    (130, 1, 33, 64, 1, 5), (256, 1, 1000, 2000, 1, 6),
+])
+def test_many_short_sequences_through_whole_row_groups_stay_under_the_bar(dev, batch, q_len, lo, hi, splits, seed):
+    from omni_npu_amd import kernels as K
+    heads, checked = 128, 24
+    c = O.make_decode_case(batch, heads, lo, hi, seed=seed, q_len=q_len)
+    args = [c[k].to(dev) for k in ("q_nope", "q_rope", "nope", "rope", "block_table", "seq_lens")]
+    out = torch.full((batch * q_len, heads, 512), float("nan"), dtype=torch.bfloat16, device=dev)
+    K.decode(*args, c["scale"], out, q_len=q_len, num_splits=splits)
+    assert torch.isfinite(out.float()).all()
+    ref = O.absorbed_decode(c["q_nope"][:checked * q_len], c["q_rope"][:checked * q_len], c["nope"], c["rope"],
+                            c["block_table"][:checked], c["seq_lens"][:checked], c["scale"])
+    ma, mr = attn_close(out[:checked * q_len], ref, 2e-2, 2e-3)
+    assert mr <= 1.92e-3, f"mean_rel={mr:.4g}: whole row groups have read 1.74e-3 to 1.85e-3 on these shapes"
